@@ -1,0 +1,266 @@
+#!/usr/bin/env python3
+"""Benchmark of the JL projection hot path (and, beside it, the scoring GEMMs) on one MI355X.
+
+`python bench.py [--gpus 1] [--steps K] [--warmup W]` prints ONE JSON line.
+
+step      = one `trakhip_project` call on one resident batch [32, 11_689_512] fp16
+            (ResNet-18-sized Rademacher projection to k = 4096, seed 7, 16 distinct batches
+            cycled back to back; inputs are in HBM before the timed region starts).
+value     = 2*B*P*k flop per step / time per step, in TFLOP/s.
+roofline  = the projection kernel alone (phase 1 of the call), timed with HIP events recorded
+            on the launch stream around every launch, against the dense fp16 MFMA peak.
+cpu_baseline = the CPU restatement of trak's BasicProjector (oracle/basic_projector.py) on the
+            CPU-runnable configuration ([16, 1_048_576] fp32 -> 512), timed on this host.
+`scoring` = BasicScoreComputer at N=50_000, M=10_000, k=4096 fp32: GEMM TFLOP/s against the fp32
+            MFMA peak, the SPD inverse separately, and a CPU sample beside it.
+"""
+import argparse
+import ctypes
+import json
+import math
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_FP16_TFLOPS = 2500.0   # MI355X dense fp16/bf16 MFMA
+PEAK_FP32_TFLOPS = 157.3    # MI355X fp32 MFMA
+METRIC = "JL proj TFLOP/s & % MFMA peak at P=11.7M,k=4096,B=32; scoring TFLOP/s"
+
+
+class Hip:
+    """Minimal HIP event API through ctypes (events on an explicit stream)."""
+
+    def __init__(self):
+        self.lib = ctypes.CDLL("libamdhip64.so")
+        self.lib.hipEventCreate.argtypes = [ctypes.POINTER(ctypes.c_void_p)]
+        self.lib.hipEventRecord.argtypes = [ctypes.c_void_p, ctypes.c_void_p]
+        self.lib.hipEventSynchronize.argtypes = [ctypes.c_void_p]
+        self.lib.hipEventElapsedTime.argtypes = [ctypes.POINTER(ctypes.c_float), ctypes.c_void_p, ctypes.c_void_p]
+        self.lib.hipEventDestroy.argtypes = [ctypes.c_void_p]
+
+    def event(self):
+        e = ctypes.c_void_p()
+        assert self.lib.hipEventCreate(ctypes.byref(e)) == 0
+        return e
+
+    def record(self, e, stream):
+        assert self.lib.hipEventRecord(e, ctypes.c_void_p(stream)) == 0
+
+    def elapsed_ms(self, a, b):
+        assert self.lib.hipEventSynchronize(b) == 0
+        ms = ctypes.c_float()
+        assert self.lib.hipEventElapsedTime(ctypes.byref(ms), a, b) == 0
+        return ms.value
+
+
+def make_batches(torch, dev, n_batches, B, P, seed):
+    """ResNet-18-sized synthetic gradients: 62 parameter blocks with log-uniform scales in
+    [1e-5, 1e-2] times N(0,1), fp16, generated on the device."""
+    gen = torch.Generator(device=dev).manual_seed(seed)
+    blocks = 62
+    edges = torch.linspace(0, P, blocks + 1).long().tolist()
+    out = []
+    for _ in range(n_batches):
+        scale = 10 ** (torch.rand(blocks, generator=gen, device=dev) * 3 - 5)
+        g = torch.empty(B, P, dtype=torch.float16, device=dev)
+        for i in range(blocks):
+            lo, hi = edges[i], edges[i + 1]
+            g[:, lo:hi] = (torch.randn(B, hi - lo, generator=gen, device=dev) * scale[i]).half()
+        out.append(g)
+    return out
+
+
+def bench_projection(torch, dev, steps, warmup, n_batches):
+    from trak_amd import _lib, fast_jl
+
+    lib = _lib.load()
+    hip = Hip()
+    B, P, k, seed = 32, 11_689_512, 4096, 7
+    tiles = torch.cuda.get_device_properties(dev).multi_processor_count
+    batches = make_batches(torch, dev, n_batches, B, P, 20_003)
+    out = torch.empty(B, k, dtype=torch.float32, device=dev)
+    ws = torch.empty(lib.trakhip_project_workspace(B, P, k, tiles), dtype=torch.uint8, device=dev)
+    stream = torch.cuda.current_stream(dev).cuda_stream
+    vp = ctypes.c_void_p
+
+    def full(g):
+        _lib.check(lib.trakhip_project(vp(g.data_ptr()), _lib.F16, B, P, P, vp(out.data_ptr()), vp(ws.data_ptr()),
+                                       ws.numel(), k, seed, tiles, _lib.RADEMACHER, vp(stream)))
+
+    for i in range(warmup):
+        full(batches[i % n_batches])
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(steps):
+        full(batches[i % n_batches])
+    torch.cuda.synchronize()
+    ms_per_step = (time.perf_counter() - t0) * 1e3 / steps
+
+    # the projection kernel alone: events around each phase-1 launch on the launch stream
+    evs = [(hip.event(), hip.event()) for _ in range(steps)]
+    for i in range(steps):
+        g = batches[i % n_batches]
+        hip.record(evs[i][0], stream)
+        _lib.check(lib.trakhip_project_partials(vp(g.data_ptr()), _lib.F16, B, P, P, vp(ws.data_ptr()), ws.numel(), k,
+                                                seed, tiles, _lib.RADEMACHER, vp(stream)))
+        hip.record(evs[i][1], stream)
+        _lib.check(lib.trakhip_project_reduce(vp(ws.data_ptr()), B, P, k, tiles, 1.0, vp(out.data_ptr()), vp(stream)))
+    torch.cuda.synchronize()
+    kernel_ms = sorted(hip.elapsed_ms(a, b) for a, b in evs)
+    kernel_avg = sum(kernel_ms) / len(kernel_ms)
+    flop = 2.0 * B * P * k
+    return {
+        "flop": flop,
+        "ms_per_step": ms_per_step,
+        "tflops": flop / (ms_per_step * 1e-3) / 1e12,
+        "kernel_ms_avg": kernel_avg,
+        "kernel_ms_min": kernel_ms[0],
+        "kernel_tflops": flop / (kernel_avg * 1e-3) / 1e12,
+        "tiles": tiles,
+        "shape": {"B": B, "P": P, "k": k},
+    }
+
+
+def bench_scoring(torch, dev, reps=3):
+    from trak_amd import BasicScoreComputer
+
+    N, M, k, lam = 50_000, 10_000, 4096, 1e-3
+    gen = torch.Generator(device=dev).manual_seed(20_005)
+    X = torch.randn(N, k, generator=gen, device=dev) / 64
+    Xt = torch.randn(M, k, generator=gen, device=dev) / 64
+    otl = torch.rand(N, generator=gen, device=dev)
+    sc = BasicScoreComputer(dtype=torch.float32, device=dev, lambda_reg=lam)
+
+    def timed(fn):
+        best = None
+        for _ in range(reps):
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record()
+            r = fn()
+            b.record()
+            torch.cuda.synchronize()
+            ms = a.elapsed_time(b)
+            best = ms if best is None else min(best, ms)
+        return r, best
+
+    from trak_amd.utils import gemm_nt, gemm_tn, spd_inverse
+
+    xtx, t_xtx = timed(lambda: gemm_tn(X, X))
+    (inv, _), t_inv = timed(lambda: spd_inverse(xtx, lambda_reg=lam, normalize=True))
+    feats, t_feat = timed(lambda: gemm_nt(X, inv))
+    scores, t_sc = timed(lambda: gemm_nt(feats, Xt, row_scale=otl))
+    gemm_flop = 2.0 * N * k * k * 2 + 2.0 * N * M * k
+    gemm_ms = t_xtx + t_feat + t_sc
+    return {
+        "shape": {"N": N, "M": M, "k": k, "lambda": lam},
+        "xtx_ms": t_xtx, "inverse_ms": t_inv, "x_xtx_inv_ms": t_feat, "scores_ms": t_sc,
+        "gemm_tflops": gemm_flop / (gemm_ms * 1e-3) / 1e12,
+        "gemm_frac_fp32_mfma_peak": gemm_flop / (gemm_ms * 1e-3) / 1e12 / PEAK_FP32_TFLOPS,
+        "inverse_flop": float(k) ** 3,
+        "scores_orientation": "[N_train, M_targets]",
+    }
+
+
+def cpu_baseline(torch):
+    """trak's BasicProjector CPU path (restated in oracle/basic_projector.py) on its CPU-runnable
+    configuration, all host cores; plus a bounded BasicScoreComputer sample."""
+    from oracle.basic_projector import BasicProjectorCPU
+    from oracle.score_oracle import BasicScoreComputerCPU
+
+    cores = int(os.environ.get("OMP_NUM_THREADS", 0)) or os.cpu_count()
+    torch.set_num_threads(cores)
+    B, P, k = 16, 1_048_576, 512
+    gen = torch.Generator().manual_seed(20_001)
+    g = torch.randn(B, P, generator=gen) * 1e-3
+    proj = BasicProjectorCPU(grad_dim=P, proj_dim=k, seed=42, proj_type="rademacher")
+    t0 = time.perf_counter()
+    proj.project(g, model_id=0)
+    dt = time.perf_counter() - t0
+    flop = 2.0 * B * P * k
+    res = {
+        "value": flop / dt / 1e12, "unit": "TFLOP/s", "cores": cores, "kind": "port",
+        "sample": f"BasicProjector restatement, full config [16,1048576] fp32 -> 512 rademacher, {dt:.2f} s",
+    }
+    N, M, kk = 4000, 1000, 1024
+    X = torch.randn(N, kk, generator=gen) / 32
+    Xt = torch.randn(M, kk, generator=gen) / 32
+    sc = BasicScoreComputerCPU(lambda_reg=1e-3)
+    t0 = time.perf_counter()
+    xtx = sc.get_xtx(X)
+    f = sc.get_x_xtx_inv(X, xtx)
+    acc = torch.zeros(N, M)
+    sc.get_scores(f, Xt, acc)
+    dts = time.perf_counter() - t0
+    res["scoring_tflops"] = (4.0 * N * kk * kk + 2.0 * N * M * kk) / dts / 1e12
+    res["scoring_sample"] = f"BasicScoreComputer restatement N={N}, M={M}, k={kk} fp32, {dts:.2f} s (inverse included)"
+    return res
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--batches", type=int, default=16, help="distinct resident batches cycled through")
+    ap.add_argument("--no-scoring", action="store_true")
+    ap.add_argument("--no-cpu", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (see DESIGN.md, sharding note); "
+              "run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        sys.exit(1)
+    dev = torch.device("cuda:0")
+    proj = bench_projection(torch, dev, args.steps, args.warmup, args.batches)
+    torch.cuda.empty_cache()
+    scoring = None if args.no_scoring else bench_scoring(torch, dev)
+    torch.cuda.empty_cache()
+    cpu = None if args.no_cpu else cpu_baseline(torch)
+
+    line = {
+        "metric": METRIC,
+        "value": round(proj["tflops"], 3),
+        "unit": "TFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(proj["ms_per_step"], 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f16",
+        "data": "synthetic",
+        "config": {
+            "workload": "ResNet-18-sized Rademacher JL projection: gradients [32, 11689512] fp16 "
+                        "(62 blocks, log-uniform scales 1e-5..1e-2), k=4096, seed 7, "
+                        f"{args.batches} resident batches cycled, num_feature_tiles={proj['tiles']}",
+            "flop_per_step": proj["flop"],
+            "frac_fp16_mfma_peak": round(proj["tflops"] / PEAK_FP16_TFLOPS, 4),
+        },
+        "roofline": {
+            "bound": "mfma",
+            "achieved": round(proj["kernel_tflops"], 3),
+            "peak": PEAK_FP16_TFLOPS,
+            "unit": "TFLOP/s",
+            "frac": round(proj["kernel_tflops"] / PEAK_FP16_TFLOPS, 4),
+            "traffic": None,
+            "kernel": "jl_project_kernel<f16, rademacher>",
+            "kernel_ms_avg": round(proj["kernel_ms_avg"], 4),
+            "kernel_ms_min": round(proj["kernel_ms_min"], 4),
+        },
+        "cpu_baseline": cpu,
+        "scoring": scoring,
+    }
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,122 @@
+/* C ABI of libtrakhip.so: JL gradient projection and attribution-scoring kernels for
+ * AMD MI355X (gfx950).
+ *
+ * Conventions
+ *   - every pointer named *_dev is device memory on the current HIP device; the caller owns
+ *     all buffers, the library never allocates device memory and never synchronizes;
+ *   - work is enqueued on `stream` (a hipStream_t passed as void*; NULL = default stream);
+ *   - return value 0 = success, negative = error (trakhip_strerror gives the text); nothing
+ *     is thrown across this boundary;
+ *   - matrices are row-major, leading dimensions are counted in elements.
+ *
+ * Each entry point names the reference code (MadryLab/trak) it stands in for.
+ */
+#ifndef TRAKHIP_H
+#define TRAKHIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* input element types of the projection */
+#define TRAKHIP_F16 0
+#define TRAKHIP_BF16 1
+#define TRAKHIP_F32 2
+
+/* projection types: enum ProjectionType of fast_jl/types.cuh:4-7 */
+#define TRAKHIP_RADEMACHER 0
+#define TRAKHIP_NORMAL 1
+
+#define TRAKHIP_OK 0
+#define TRAKHIP_ERR_PROJ_DIM -1  /* proj dim not a multiple of 512 (fast_jl/fast_jl_kernel.cuh:113-115) */
+#define TRAKHIP_ERR_SHAPE -2     /* empty / oversized / inconsistent shape */
+#define TRAKHIP_ERR_DTYPE -3     /* unknown element type (fast_jl/fast_jl.cu:26) */
+#define TRAKHIP_ERR_PROJ_TYPE -4
+#define TRAKHIP_ERR_NULL -5      /* null pointer */
+#define TRAKHIP_ERR_WORKSPACE -6 /* workspace too small */
+#define TRAKHIP_ERR_ALIGN -7     /* pointer not aligned as documented */
+#define TRAKHIP_ERR_LAUNCH -8    /* HIP refused the launch (hipGetLastError != hipSuccess) */
+#define TRAKHIP_ERR_NOT_SPD -9   /* matrix handed to the SPD inverse is not positive definite */
+#define TRAKHIP_ERR_NO_DEVICE -10
+
+const char* trakhip_strerror(int code);
+
+/* Version of this ABI (bumped on incompatible change). */
+int trakhip_abi_version(void);
+
+/* ---- JL projection -------------------------------------------------------------------- */
+
+/* Bytes of scratch trakhip_project needs for these sizes.  Stands in for the
+ * torch::zeros({B_pad, T, N}) intermediate of fast_jl/fast_jl.cu:48-49. */
+size_t trakhip_project_workspace(uint64_t B, uint64_t P, uint32_t proj_dim, uint32_t num_feature_tiles);
+
+/* out[B, proj_dim] (fp32) = in[B, P] x S, S generated on the fly from (seed, proj_dim,
+ * num_feature_tiles, P).  Stands in for the six functions project_{rademacher,normal}_{8,16,32}
+ * of fast_jl/fast_jl.cu:81-110 (host loop over batches of rows at fast_jl/fast_jl.cu:44-76, kernel
+ * fast_jl/fast_jl_kernel.cuh:24-105, cross-tile sum fast_jl/fast_jl.cu:78).
+ *   in_dev      row-major [B, P] with row pitch ld_in >= P elements, aligned to its element size
+ *   in_dtype    TRAKHIP_F16 | TRAKHIP_BF16 | TRAKHIP_F32
+ *   out_dev     [B, proj_dim] fp32, contiguous, 16-byte aligned; fully overwritten
+ *   workspace   >= trakhip_project_workspace(...) bytes, 16-byte aligned
+ *   proj_dim    multiple of 512;  P < 2^32;  any B >= 1
+ */
+int trakhip_project(const void* in_dev, int in_dtype, uint64_t B, uint64_t P, uint64_t ld_in,
+                    float* out_dev, void* workspace_dev, size_t workspace_bytes, uint32_t proj_dim,
+                    uint32_t seed, uint32_t num_feature_tiles, int proj_type, void* stream);
+
+/* The two phases of trakhip_project as separate calls, for B <= 32 rows: phase 1 writes the
+ * per-feature-tile partial sums [T, B, proj_dim] (T = min(P, num_feature_tiles)) to the workspace
+ * (the kernel of fast_jl/fast_jl_kernel.cuh:24-105 writing `output[row][tile][col]`), phase 2 adds
+ * them up in tile order into out_dev (the `.sum(1)` of fast_jl/fast_jl.cu:78), multiplied by
+ * `scale` (1.0f for the plain sum; 1/sqrt(P) gives the `grads /= normalize_factor` of
+ * trak/traker.py:426 for free).  A caller can time the phases or put its own epilogue between. */
+int trakhip_project_partials(const void* in_dev, int in_dtype, uint64_t B, uint64_t P, uint64_t ld_in,
+                             void* workspace_dev, size_t workspace_bytes, uint32_t proj_dim, uint32_t seed,
+                             uint32_t num_feature_tiles, int proj_type, void* stream);
+int trakhip_project_reduce(const void* workspace_dev, uint64_t B, uint64_t P, uint32_t proj_dim,
+                           uint32_t num_feature_tiles, float scale, float* out_dev, void* stream);
+
+/* Writes the block S[f0 : f0+nf, c0 : c0+nc] of the projection matrix that trakhip_project uses
+ * for (seed, num_feature_tiles, P) as fp32, row-major [nf, nc].  The reference never stores S
+ * (it exists only inside fast_jl/random.cuh:27-60); this is the hook that lets a caller check
+ * the stream.  on_device != 0: out is device memory and a kernel on `stream` writes it;
+ * on_device == 0: out is host memory, filled by host code before returning. */
+int trakhip_materialize(uint32_t seed, uint32_t num_feature_tiles, uint64_t P, uint64_t f0, uint64_t nf,
+                        uint32_t c0, uint32_t nc, int proj_type, float* out, int on_device, void* stream);
+
+/* ---- scoring (BasicScoreComputer) ---------------------------------------------------------- */
+
+/* C[M, N] = alpha * A[M, K] * B[N, K]^T + beta * C, then row i scaled by row_scale[i] when
+ * row_scale_dev != NULL; all fp32.  Stands in for `block @ xtx_inv` (trak/score_computers.py:176,
+ * xtx_inv symmetric) and `features @ target_grads.t()` (trak/utils.py:131); the optional row scale
+ * is the out_to_loss factor of trak/traker.py:670-678. */
+int trakhip_gemm_nt(const float* A_dev, uint64_t lda, const float* B_dev, uint64_t ldb, float* C_dev,
+                    uint64_t ldc, uint64_t M, uint64_t N, uint64_t K, float alpha, float beta,
+                    const float* row_scale_dev, void* stream);
+
+/* C[M, N] = alpha * A[K, M]^T * B[K, N] + beta * C; fp32.  With A == B this is the
+ * `block.T @ block` accumulation of trak/score_computers.py:145-155. */
+int trakhip_gemm_tn(const float* A_dev, uint64_t lda, const float* B_dev, uint64_t ldb, float* C_dev,
+                    uint64_t ldc, uint64_t M, uint64_t N, uint64_t K, float alpha, float beta,
+                    void* stream);
+
+/* Bytes of scratch trakhip_spd_inverse needs for an n x n matrix. */
+size_t trakhip_spd_inverse_workspace(uint64_t n);
+
+/* inv[n, n] = (A + lambda * I)^-1 for symmetric positive definite A + lambda*I (fp32), then
+ * divided by mean(|inv|) when normalize != 0; *mean_abs_dev (device, 1 float, may be NULL)
+ * receives that mean.  Stands in for torch.linalg.inv + `xtx_inv /= xtx_inv.abs().mean()` of
+ * trak/score_computers.py:160-166.  A_dev is not modified; inv_dev may not alias it.
+ * status_dev (device, 1 int32, may be NULL) is set to 0, or to 1 + the index of the first
+ * non-positive pivot. */
+int trakhip_spd_inverse(const float* A_dev, uint64_t lda, float lambda, float* inv_dev, uint64_t ldi,
+                        uint64_t n, int normalize, float* mean_abs_dev, int32_t* status_dev,
+                        void* workspace_dev, size_t workspace_bytes, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TRAKHIP_H */

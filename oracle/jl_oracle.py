@@ -1,0 +1,299 @@
+"""TEST INFRASTRUCTURE ONLY -- numpy oracle for the JL projection matrix, plus the loader of
+the C oracle (oracle/jl_oracle.c).
+
+This is a second, independent statement of the random stream (vectorized numpy, written
+from the specification, not from the C oracle or the library's header).  Only tests/,
+__graft_entry__.smoke() and the cpu_baseline leg of bench.py may import it.
+
+Restated reference behaviour (MadryLab/trak):
+  * stream_seed   -- fast_jl/random.cuh:15-17
+  * tiling        -- fast_jl/fast_jl.cu:42, fast_jl/fast_jl_kernel.cuh:124
+  * Rademacher: one random bit per entry, bit set -> +1 -- fast_jl/random.cuh:33-37
+  * Normal: Box-Muller normal rounded to fp16 -- fast_jl/random.cuh:50-60
+The generator is Philox4x32-10 (Random123), pinned by Random123's known-answer vectors in
+tests/test_oracle_philox.py; the position -> (block, bit) map is this build's definition and
+is pinned by agreement of this file with oracle/jl_oracle.c and by the property tests.
+"""
+import ctypes
+import os
+import subprocess
+
+import numpy as np
+
+RADEMACHER = 0
+NORMAL = 1
+
+_M0 = np.uint64(0xD2511F53)
+_M1 = np.uint64(0xCD9E8D57)
+_W0 = 0x9E3779B9
+_W1 = 0xBB67AE85
+_MASK = np.uint64(0xFFFFFFFF)
+
+
+def philox4x32_10(ctr, key):
+    """ctr: (..., 4) uint32, key: (..., 2) uint32 -> (..., 4) uint32."""
+    ctr = np.asarray(ctr, dtype=np.uint32)
+    key = np.asarray(key, dtype=np.uint32)
+    c = [ctr[..., i].astype(np.uint64) for i in range(4)]
+    k0 = key[..., 0].astype(np.uint64)
+    k1 = key[..., 1].astype(np.uint64)
+    for r in range(10):
+        kk0 = (k0 + np.uint64((_W0 * r) & 0xFFFFFFFF)) & _MASK
+        kk1 = (k1 + np.uint64((_W1 * r) & 0xFFFFFFFF)) & _MASK
+        p0 = _M0 * c[0]
+        p1 = _M1 * c[2]
+        c = [
+            (p1 >> np.uint64(32)) ^ c[1] ^ kk0,
+            p1 & _MASK,
+            (p0 >> np.uint64(32)) ^ c[3] ^ kk1,
+            p0 & _MASK,
+        ]
+    return np.stack(c, axis=-1).astype(np.uint32)
+
+
+def stream_seed(seed, column, tile):
+    v = (
+        np.uint64(seed)
+        + np.uint64(658105236) * np.asarray(column, dtype=np.uint64)
+        + np.uint64(359124577) * np.asarray(tile, dtype=np.uint64)
+    )
+    return (v & _MASK).astype(np.uint32)
+
+
+def tiling(P, num_feature_tiles):
+    tiles = min(int(P), int(num_feature_tiles))
+    tile_size = -(-int(P) // tiles)
+    return tiles, tile_size
+
+
+# ---- exact binary32 fma on numpy arrays -----------------------------------------------------
+
+
+def _fma32(a, b, c):
+    """Correctly rounded float32 fma(a, b, c) for float32 arrays.
+
+    a*b is exact in float64 (24+24 bits).  p + c is computed in float64 with its rounding
+    error (TwoSum); if the float64 sum lands exactly half way between two float32 values the
+    error term decides the direction, which removes the double-rounding hazard."""
+    shape = np.broadcast(np.asarray(a), np.asarray(b), np.asarray(c)).shape
+    a = np.atleast_1d(np.asarray(a, dtype=np.float32)).astype(np.float64)
+    b = np.atleast_1d(np.asarray(b, dtype=np.float32)).astype(np.float64)
+    c = np.atleast_1d(np.asarray(c, dtype=np.float32)).astype(np.float64)
+    a, b, c = np.broadcast_arrays(a, b, c)
+    p = a * b
+    s = p + c
+    bb = s - p
+    err = (p - (s - bb)) + (c - bb)
+    r = s.astype(np.float32)
+    low = np.ascontiguousarray(s).view(np.uint64) & np.uint64((1 << 29) - 1)
+    tie = (low == np.uint64(1 << 28)) & (err != 0.0) & np.isfinite(s) & (s != 0.0)
+    if tie.any():
+        # the true value is s + err: it lies strictly on one side of the midpoint
+        lo = np.nextafter(s[tie], -np.inf)
+        hi = np.nextafter(s[tie], np.inf)
+        r[tie] = np.where(err[tie] > 0, hi, lo).astype(np.float32)
+    return r.reshape(shape)
+
+
+def _f32(x):
+    return np.asarray(x, dtype=np.float32)
+
+
+def box_muller_unrounded(wa, wb):
+    """Two float32 normals (cos branch, sin branch) from two uint32 words, following the
+    specified binary32 operation sequence."""
+    wa = np.asarray(wa, dtype=np.uint32)
+    wb = np.asarray(wb, dtype=np.uint32)
+    one = np.float32(1.0)
+    odd = ((wa >> np.uint32(9)) << np.uint32(1)) | np.uint32(1)
+    xf = odd.astype(np.float32)  # exact, < 2^24
+    xb = xf.view(np.uint32)
+    expo = (xb >> np.uint32(23)).astype(np.int32) - 127
+    mant = ((xb & np.uint32(0x7FFFFF)) | np.uint32(0x3F800000)).view(np.float32)
+    big = mant > np.float32(1.41421354)
+    mant = np.where(big, mant * np.float32(0.5), mant).astype(np.float32)
+    expo = np.where(big, expo + 1, expo)
+    t = (mant - one).astype(np.float32)
+    z = (t * t).astype(np.float32)
+    coef = [
+        7.0376836292e-2,
+        -1.1514610310e-1,
+        1.1676998740e-1,
+        -1.2420140846e-1,
+        1.4249322787e-1,
+        -1.6668057665e-1,
+        2.0000714765e-1,
+        -2.4999993993e-1,
+        3.3333331174e-1,
+    ]
+    poly = np.full(t.shape, np.float32(coef[0]), dtype=np.float32)
+    for cf in coef[1:]:
+        poly = _fma32(poly, t, np.float32(cf))
+    y = (t * (z * poly).astype(np.float32)).astype(np.float32)
+    y = _fma32(np.float32(-0.5), z, y)
+    ln_m = (t + y).astype(np.float32)
+    ln_u = _fma32((expo - 24).astype(np.float32), np.float32(0.693147182), ln_m)
+    s = (np.float32(-2.0) * ln_u).astype(np.float32)
+    guess = (np.uint32(0x5F3759DF) - (s.view(np.uint32) >> np.uint32(1))).view(np.float32)
+    half_s = (np.float32(0.5) * s).astype(np.float32)
+    for _ in range(3):
+        gg = (guess * guess).astype(np.float32)
+        corr = _fma32(-half_s, gg, np.float32(1.5))
+        guess = (guess * corr).astype(np.float32)
+    radius = (s * guess).astype(np.float32)
+
+    quadrant = wb >> np.uint32(30)
+    frac = ((wb >> np.uint32(6)) & np.uint32(0xFFFFFF)).astype(np.float32)
+    yv = ((frac - np.float32(8388608.0)).astype(np.float32) * np.float32(9.36266447e-8)).astype(np.float32)
+    y2 = (yv * yv).astype(np.float32)
+    ps = _fma32(np.float32(-1.9515295891e-4), y2, np.float32(8.3321608736e-3))
+    ps = _fma32(ps, y2, np.float32(-1.6666654611e-1))
+    sn = _fma32((ps * y2).astype(np.float32), yv, yv)
+    pc = _fma32(np.float32(2.443315711809948e-5), y2, np.float32(-1.388731625493765e-3))
+    pc = _fma32(pc, y2, np.float32(4.166664568298827e-2))
+    cs = _fma32((pc * y2).astype(np.float32), y2, _fma32(np.float32(-0.5), y2, one))
+    cosv = np.select([quadrant == 0, quadrant == 1, quadrant == 2], [cs, -sn, -cs], default=sn)
+    sinv = np.select([quadrant == 0, quadrant == 1, quadrant == 2], [sn, cs, -sn], default=-cs)
+    z0 = (radius * cosv.astype(np.float32)).astype(np.float32)
+    z1 = (radius * sinv.astype(np.float32)).astype(np.float32)
+    return z0, z1
+
+
+def materialize(seed, num_feature_tiles, P, f0, nf, c0, nc, proj_type):
+    """S[f0:f0+nf, c0:c0+nc] as float32 (every value is exactly an fp16 value)."""
+    tiles, tile_size = tiling(P, num_feature_tiles)
+    f = np.arange(f0, f0 + nf, dtype=np.uint64)[:, None]
+    c = np.arange(c0, c0 + nc, dtype=np.uint64)[None, :]
+    tile = f // np.uint64(tile_size)
+    off = (f - tile * np.uint64(tile_size)).astype(np.uint32)
+    off = np.broadcast_to(off, (nf, nc))
+    key = np.zeros((nf, nc, 2), dtype=np.uint32)
+    key[..., 0] = stream_seed(seed, np.broadcast_to(c, (nf, nc)), np.broadcast_to(tile, (nf, nc)))
+    ctr = np.zeros((nf, nc, 4), dtype=np.uint32)
+    if proj_type == RADEMACHER:
+        ctr[..., 0] = off // np.uint32(128)
+        w = philox4x32_10(ctr, key)
+        j = off % np.uint32(128)
+        shift_index = j // np.uint32(8)
+        slot = j % np.uint32(8)
+        word = np.take_along_axis(w, (slot // np.uint32(2))[..., None].astype(np.int64), axis=-1)[..., 0]
+        bitpos = np.where(slot % np.uint32(2) == 1, 31, 15).astype(np.uint32) - shift_index
+        bit = (word >> bitpos) & np.uint32(1)
+        return np.where(bit == 1, np.float32(1.0), np.float32(-1.0)).astype(np.float32)
+    ctr[..., 0] = off // np.uint32(4)
+    w = philox4x32_10(ctr, key)
+    e = off % np.uint32(4)
+    wa = np.where(e < 2, w[..., 0], w[..., 2])
+    wb = np.where(e < 2, w[..., 1], w[..., 3])
+    z0, z1 = box_muller_unrounded(wa, wb)
+    z = np.where(e % np.uint32(2) == 1, z1, z0).astype(np.float32)
+    return z.astype(np.float16).astype(np.float32)  # numpy's float16 cast is round-to-nearest-even
+
+
+def project_fp64(G, seed, num_feature_tiles, proj_dim_cols, proj_type, chunk=4096):
+    """float64 contraction G[B, P] x S[:, cols] with S from this file (small shapes only)."""
+    G = np.asarray(G)
+    B, P = G.shape
+    cols = np.asarray(proj_dim_cols)
+    out = np.zeros((B, len(cols)), dtype=np.float64)
+    c0, nc = int(cols[0]), len(cols)
+    assert np.array_equal(cols, np.arange(c0, c0 + nc))
+    for f0 in range(0, P, chunk):
+        nf = min(chunk, P - f0)
+        S = materialize(seed, num_feature_tiles, P, f0, nf, c0, nc, proj_type).astype(np.float64)
+        out += G[:, f0 : f0 + nf].astype(np.float64) @ S
+    return out
+
+
+# ---- C oracle loader ---------------------------------------------------------------------------
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_SO = os.path.join(_HERE, "libjl_oracle.so")
+
+
+def build_c_oracle(force=False):
+    src = os.path.join(_HERE, "jl_oracle.c")
+    if force or not os.path.exists(_SO) or os.path.getmtime(_SO) < os.path.getmtime(src):
+        subprocess.check_call(["make", "-C", _HERE, "-s", "libjl_oracle.so"])
+    return _SO
+
+
+class COracle:
+    """ctypes view of oracle/libjl_oracle.so."""
+
+    def __init__(self):
+        if not os.path.exists(_SO):
+            build_c_oracle()
+        lib = ctypes.CDLL(_SO)
+        u32, u64, i32 = ctypes.c_uint32, ctypes.c_uint64, ctypes.c_int
+        fp = ctypes.POINTER(ctypes.c_float)
+        dp = ctypes.POINTER(ctypes.c_double)
+        up = ctypes.POINTER(u32)
+        lib.jlo_philox4x32_10.argtypes = [up, up, up]
+        lib.jlo_philox4x32_10.restype = None
+        lib.jlo_stream_seed.argtypes = [u32, u32, u32]
+        lib.jlo_stream_seed.restype = u32
+        lib.jlo_tiling.argtypes = [u64, u32, up, ctypes.POINTER(u64)]
+        lib.jlo_tiling.restype = None
+        lib.jlo_entry.argtypes = [u32, u32, u64, u64, u32, i32]
+        lib.jlo_entry.restype = ctypes.c_float
+        lib.jlo_normal_unrounded.argtypes = [u32, u32, i32]
+        lib.jlo_normal_unrounded.restype = ctypes.c_float
+        lib.jlo_half_bits.argtypes = [ctypes.c_float]
+        lib.jlo_half_bits.restype = ctypes.c_uint16
+        lib.jlo_materialize.argtypes = [u32, u32, u64, u64, u64, u32, u32, i32, fp]
+        lib.jlo_materialize.restype = None
+        lib.jlo_project.argtypes = [fp, u64, u64, u64, u32, u32, u32, u32, i32, dp]
+        lib.jlo_project.restype = None
+        self.lib = lib
+
+    def philox(self, ctr, key):
+        c = (ctypes.c_uint32 * 4)(*[int(x) for x in ctr])
+        k = (ctypes.c_uint32 * 2)(*[int(x) for x in key])
+        o = (ctypes.c_uint32 * 4)()
+        self.lib.jlo_philox4x32_10(c, k, o)
+        return [int(x) for x in o]
+
+    def stream_seed(self, seed, column, tile):
+        return int(self.lib.jlo_stream_seed(seed, column, tile))
+
+    def tiling(self, P, num_feature_tiles):
+        t = ctypes.c_uint32()
+        s = ctypes.c_uint64()
+        self.lib.jlo_tiling(P, num_feature_tiles, ctypes.byref(t), ctypes.byref(s))
+        return int(t.value), int(s.value)
+
+    def entry(self, seed, tiles, P, f, c, proj_type):
+        return float(self.lib.jlo_entry(seed, tiles, P, f, c, proj_type))
+
+    def normal_unrounded(self, wa, wb, second):
+        return float(self.lib.jlo_normal_unrounded(wa, wb, int(second)))
+
+    def half_bits(self, v):
+        return int(self.lib.jlo_half_bits(ctypes.c_float(v)))
+
+    def materialize(self, seed, tiles, P, f0, nf, c0, nc, proj_type):
+        out = np.empty((nf, nc), dtype=np.float32)
+        self.lib.jlo_materialize(
+            seed, tiles, P, f0, nf, c0, nc, proj_type, out.ctypes.data_as(ctypes.POINTER(ctypes.c_float))
+        )
+        return out
+
+    def project(self, G32, seed, tiles, c0, nc, proj_type):
+        """G32: float32 [B, P] C-contiguous (exact image of the fp16/bf16/fp32 input)."""
+        G32 = np.ascontiguousarray(G32, dtype=np.float32)
+        B, P = G32.shape
+        out = np.empty((B, nc), dtype=np.float64)
+        self.lib.jlo_project(
+            G32.ctypes.data_as(ctypes.POINTER(ctypes.c_float)),
+            B,
+            P,
+            P,
+            seed,
+            tiles,
+            c0,
+            nc,
+            proj_type,
+            out.ctypes.data_as(ctypes.POINTER(ctypes.c_double)),
+        )
+        return out

@@ -1,0 +1,102 @@
+"""No-GPU checks of libtrakhip.so: it loads, exports every symbol the public header declares,
+validates arguments before touching the device, and its host-side matrix materializer agrees
+with the oracle bit for bit."""
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+
+from oracle import jl_oracle as npo
+from trak_amd import _lib, fast_jl
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared_symbols():
+    text = open(os.path.join(ROOT, "include", "trakhip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(trakhip_[a-z_0-9]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    lib = _lib.load()
+    names = _declared_symbols()
+    assert len(names) >= 9
+    for name in names:
+        assert getattr(lib, name) is not None, name
+
+
+def test_abi_version_and_strerror():
+    lib = _lib.load()
+    assert lib.trakhip_abi_version() == 1
+    assert _lib.strerror(0) == "success"
+    # the text the reference throws at fast_jl/fast_jl_kernel.cuh:113-115
+    assert _lib.strerror(-1) == "Invalid Number of JL dimensions it has to be a multiple of 512"
+    for code in range(-10, 0):
+        assert "unknown trakhip error" not in _lib.strerror(code)
+    assert "unknown trakhip error" in _lib.strerror(-999)
+
+
+def test_project_argument_validation_needs_no_device():
+    lib = _lib.load()
+    p = ctypes.c_void_p(4096)  # never dereferenced: every call below fails validation first
+    call = lambda **kw: lib.trakhip_project(
+        kw.get("inp", p), kw.get("dtype", 0), kw.get("B", 8), kw.get("P", 1000), kw.get("ld", 1000),
+        kw.get("out", p), kw.get("ws", p), kw.get("wsb", 1 << 40), kw.get("k", 512), 0, kw.get("tiles", 256),
+        kw.get("pt", 0), None)
+    assert call(k=100) == -1 and call(k=0) == -1 and call(k=768) == -1
+    assert call(B=0) == -2 and call(P=0) == -2 and call(P=2**32) == -2 and call(ld=999) == -2 and call(tiles=0) == -2
+    assert call(dtype=3) == -3 and call(dtype=-1) == -3
+    assert call(pt=2) == -4
+    assert call(inp=None) == -5 and call(out=None) == -5 and call(ws=None) == -5
+    assert call(wsb=16) == -6
+    assert call(inp=ctypes.c_void_p(4097)) == -7 and call(out=ctypes.c_void_p(4100)) == -7
+    with pytest.raises(ValueError, match="multiple of 512"):
+        _lib.check(-1)
+    with pytest.raises(RuntimeError):
+        _lib.check(-2)
+
+
+def test_workspace_size():
+    lib = _lib.load()
+    # T * min(B, 32) * k floats with T = min(P, tiles)
+    assert lib.trakhip_project_workspace(32, 11_689_512, 4096, 256) == 256 * 32 * 4096 * 4
+    assert lib.trakhip_project_workspace(48, 1000, 512, 256) == 256 * 32 * 512 * 4
+    assert lib.trakhip_project_workspace(8, 25, 1024, 256) == 25 * 8 * 1024 * 4
+    assert lib.trakhip_project_workspace(0, 25, 1024, 256) == 0
+    assert lib.trakhip_spd_inverse_workspace(4096) >= 3 * 4096 * 4096 * 4
+    assert lib.trakhip_spd_inverse_workspace(100) >= 3 * 128 * 128 * 4
+
+
+@pytest.mark.parametrize("proj_type,name", [(npo.RADEMACHER, "rademacher"), (npo.NORMAL, "normal")])
+@pytest.mark.parametrize(
+    "seed,tiles,P,f0,nf,c0,nc",
+    [(0, 256, 1000, 0, 1000, 0, 8), (42, 256, 1_048_576, 4090, 300, 500, 12), (7, 108, 10_241, 9_900, 341, 2040, 8),
+     (2**32 - 1, 256, 25, 0, 25, 0, 16), (7 + 10_000 * 3, 256, 11_689_512, 11_689_000, 512, 4064, 32)],
+)
+def test_host_materialize_equals_oracle(c_oracle, proj_type, name, seed, tiles, P, f0, nf, c0, nc):
+    got = fast_jl.materialize(seed, tiles, P, f0, nf, c0, nc, name).numpy()
+    want = c_oracle.materialize(seed, tiles, P, f0, nf, c0, nc, proj_type)
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+
+
+def test_materialize_argument_validation():
+    lib = _lib.load()
+    buf = (ctypes.c_float * 16)()
+    assert lib.trakhip_materialize(0, 256, 100, 90, 20, 0, 1, 0, buf, 0, None) == -2   # f0 + nf > P
+    assert lib.trakhip_materialize(0, 256, 100, 0, 4, 0, 4, 5, buf, 0, None) == -4
+    assert lib.trakhip_materialize(0, 256, 100, 0, 4, 0, 4, 0, None, 0, None) == -5
+    assert lib.trakhip_materialize(0, 256, 100, 0, 0, 0, 4, 0, None, 0, None) == 0      # empty block
+
+
+def test_gemm_argument_validation_needs_no_device():
+    lib = _lib.load()
+    p = ctypes.c_void_p(4096)
+    assert lib.trakhip_gemm_nt(p, 8, p, 8, p, 4, 4, 4, 16, 1.0, 0.0, None, None) == -2   # lda < K
+    assert lib.trakhip_gemm_nt(None, 16, p, 16, p, 4, 4, 4, 16, 1.0, 0.0, None, None) == -5
+    assert lib.trakhip_gemm_nt(p, 16, p, 16, p, 4, 0, 4, 16, 1.0, 0.0, None, None) == 0  # empty
+    assert lib.trakhip_gemm_tn(p, 2, p, 8, p, 8, 4, 4, 16, 1.0, 0.0, None) == -2          # lda < M
+    assert lib.trakhip_spd_inverse(p, 2, 0.0, p, 4, 4, 0, None, None, p, 1 << 30, None) == -2
+    assert lib.trakhip_spd_inverse(p, 4, 0.0, p, 4, 4, 0, None, None, p, 16, None) == -6

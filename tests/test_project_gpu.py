@@ -1,0 +1,303 @@
+"""GPU parity tests of the JL projection: every call goes through the C ABI of libtrakhip.so
+(via trak_amd.fast_jl / trak_amd.projectors) and is compared with the CPU oracle.
+
+Tolerances (from the acceptance criteria of this build): matrix entries bit-exact; projected rows
+within 1e-3 relative L2 for fp16/bf16 inputs and 1e-5 for fp32 inputs against a float64
+contraction with the same matrix.
+"""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import jl_oracle as npo
+from trak_amd import ChunkedCudaProjector, CudaProjector, ProjectionType, fast_jl
+
+pytestmark = pytest.mark.gpu
+
+R, G = npo.RADEMACHER, npo.NORMAL
+NAMES = {R: "rademacher", G: "normal"}
+TOL = {torch.float16: 1e-3, torch.bfloat16: 1e-3, torch.float32: 1e-5}
+
+
+def fn(proj_type, n=32):
+    return getattr(fast_jl, f"project_{NAMES[proj_type]}_{n}")
+
+
+def rel_l2_rows(got, want):
+    got = np.asarray(got, dtype=np.float64)
+    want = np.asarray(want, dtype=np.float64)
+    return np.linalg.norm(got - want, axis=1) / np.maximum(np.linalg.norm(want, axis=1), 1e-300)
+
+
+def to_f32_numpy(t):
+    return t.detach().float().cpu().numpy()
+
+
+# ---- the matrix itself ------------------------------------------------------------------------
+
+
+@pytest.mark.parametrize("proj_type", [R, G])
+@pytest.mark.parametrize(
+    "seed,tiles,P,f0,nf,c0,nc",
+    [(0, 256, 1000, 0, 1000, 0, 8), (42, 256, 1_048_576, 4090, 300, 500, 12), (7, 108, 10_241, 9_900, 341, 2040, 8),
+     (2**32 - 1, 256, 25, 0, 25, 0, 16), (7, 256, 11_689_512, 11_689_000, 512, 4064, 32)],
+)
+def test_device_matrix_is_bit_exact(gpu, c_oracle, proj_type, seed, tiles, P, f0, nf, c0, nc):
+    got = fast_jl.materialize(seed, tiles, P, f0, nf, c0, nc, NAMES[proj_type], device=gpu).cpu().numpy()
+    want = c_oracle.materialize(seed, tiles, P, f0, nf, c0, nc, proj_type)
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+
+
+@pytest.mark.parametrize("proj_type", [R, G])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
+def test_one_hot_rows_read_the_matrix_back_exactly(gpu, c_oracle, proj_type, dtype):
+    # project(e_f) = S[f, :] exactly: the MFMA path uses the same entries as the materializer
+    P, k, tiles, seed = 5_000, 1024, 256, 17
+    feats = [0, 1, 7, 8, 127, 128, 255, 256, 19, 20, 2559, 4096, 4998, 4999, 1234, 3333,
+             39, 40, 41, 599, 600, 777, 2048, 2049, 3071, 3072, 4095, 4097, 4500, 4990, 4991, 4992]
+    g = torch.zeros(32, P, dtype=dtype, device=gpu)
+    for r, f in enumerate(feats):
+        g[r, f] = 1.0
+    out = fn(proj_type)(g, k, seed, tiles).cpu().numpy()
+    for r, f in enumerate(feats):
+        want = c_oracle.materialize(seed, tiles, P, f, 1, 0, k, proj_type)[0]
+        assert np.array_equal(out[r], want), (r, f)
+
+
+# ---- contraction parity against the float64 oracle --------------------------------------------
+
+
+@pytest.mark.parametrize("proj_type", [R, G])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
+@pytest.mark.parametrize(
+    "B,P,k,tiles",
+    [(32, 20_000, 512, 256), (16, 10_002, 1024, 256), (9, 10_001, 512, 108), (1, 25, 512, 256), (45, 1049, 512, 256),
+     (8, 70_001, 512, 7)],
+)
+def test_projection_matches_float64_contraction(gpu, c_oracle, proj_type, dtype, B, P, k, tiles):
+    gen = torch.Generator(device="cpu").manual_seed(1000 + B + P)
+    g = (torch.randn(B, P, generator=gen) * 1e-2).to(dtype).to(gpu)
+    seed = 123 + B
+    out = fn(proj_type)(g, k, seed, tiles)
+    assert out.shape == (B, k) and out.dtype == torch.float32 and out.device == g.device  # fast_jl.cu:48-49,78
+    cols = [0, 31, 32, 511] if k == 512 else [0, 500, 1023]
+    g32 = to_f32_numpy(g)
+    for c in cols:
+        want = c_oracle.project(g32, seed, tiles, c, 1, proj_type)
+        got = out[:, c : c + 1].cpu().numpy().astype(np.float64)
+        err = np.abs(got - want).max() / max(np.abs(want).max(), 1e-30)
+        assert err < TOL[dtype], (c, err)
+    # and whole rows on a window of 64 columns
+    want = c_oracle.project(g32, seed, tiles, k - 64, 64, proj_type)
+    err = rel_l2_rows(out[:, k - 64 :].cpu().numpy(), want)
+    assert err.max() < TOL[dtype], err.max()
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
+def test_tiny_values_and_exact_zeros(gpu, c_oracle, dtype):
+    # gradient scales down to 1e-5 (fp16 subnormals) and 1 % exact zeros, as in the benchmark inputs
+    B, P, k, tiles, seed = 32, 30_000, 512, 256, 7
+    gen = torch.Generator(device="cpu").manual_seed(5)
+    scale = 10 ** (torch.rand(P // 100, generator=gen) * 3 - 5)
+    g = torch.randn(B, P, generator=gen) * scale.repeat_interleave(100)[None, :]
+    g[torch.rand(B, P, generator=gen) < 0.01] = 0.0
+    g = g.to(dtype).to(gpu)
+    out = fn(R)(g, k, seed, tiles)
+    want = c_oracle.project(to_f32_numpy(g), seed, tiles, 0, 64, R)
+    assert rel_l2_rows(out[:, :64].cpu().numpy(), want).max() < TOL[dtype]
+
+
+def test_row_pitch_and_unaligned_rows(gpu, c_oracle):
+    # a column slice of a wider buffer (pitch > P) whose rows start at odd element offsets
+    B, P, k, tiles, seed = 16, 3001, 512, 256, 3
+    gen = torch.Generator(device="cpu").manual_seed(6)
+    wide = torch.randn(B, 4099, generator=gen).half().to(gpu)
+    view = wide[:, 77 : 77 + P]
+    assert not view.is_contiguous()
+    out = fn(R)(view, k, seed, tiles)
+    out_c = fn(R)(view.contiguous(), k, seed, tiles)
+    assert torch.equal(out, out_c)
+    want = c_oracle.project(to_f32_numpy(view), seed, tiles, 100, 32, R)
+    assert rel_l2_rows(out[:, 100:132].cpu().numpy(), want).max() < 1e-3
+
+
+# ---- properties the reference's own tests assert ----------------------------------------------
+
+
+@pytest.mark.parametrize("bs,input_size,output_size,seed", [(8, 1024, 512, 0), (8, 2048, 1024, 1), (8, 1024, 2048, 1)])
+def test_shape(gpu, bs, input_size, output_size, seed):
+    # tests/test_rademacher.py:21-39
+    x = torch.ones((bs, input_size), dtype=torch.float16, device=gpu)
+    num_sms = torch.cuda.get_device_properties(0).multi_processor_count
+    assert fast_jl.project_rademacher_8(x, output_size, seed, num_sms).shape == (bs, output_size)
+
+
+@pytest.mark.parametrize("P,seed,k,odd", [(10_240, 64, 1024, False), (10_241, 78, 2048, True)])
+def test_even_odd(gpu, P, seed, k, odd):
+    # tests/test_rademacher.py:65-108: all-ones input -> every output has the parity of P
+    x = torch.ones((8, P), dtype=torch.float16, device=gpu)
+    num_sms = torch.cuda.get_device_properties(0).multi_processor_count
+    out = fast_jl.project_rademacher_8(x, k, seed, num_sms)
+    assert torch.all(out % 2 == (1 if odd else 0))
+
+
+def test_invalid_proj_dim_raises_value_error(gpu):
+    # fast_jl/fast_jl_kernel.cuh:113-115 -> std::invalid_argument -> ValueError
+    x = torch.ones((8, 1000), dtype=torch.float16, device=gpu)
+    with pytest.raises(ValueError, match="multiple of 512"):
+        fast_jl.project_rademacher_8(x, 1000, 0, 256)
+    with pytest.raises(RuntimeError):
+        fast_jl.project_rademacher_8(x.double(), 512, 0, 256)
+    with pytest.raises(RuntimeError):
+        fast_jl.project_rademacher_8(x[0], 512, 0, 256)
+
+
+def _projector(P, k, seed, proj_type, dtype, **kw):
+    return CudaProjector(grad_dim=P, proj_dim=k, seed=seed, proj_type=proj_type, device="cuda:0", dtype=dtype,
+                         max_batch_size=32, **kw)
+
+
+PROP = [
+    (s, t, d, shape, k)
+    for s in (0, 10**8)
+    for t in (ProjectionType.normal, ProjectionType.rademacher)
+    for d in (torch.float16, torch.float32)
+    for shape, k in (((8, 10_000), 1024), ((9, 10_002), 1024), ((45, 1049), 1024), ((1, 25), 512))
+]
+
+
+@pytest.mark.parametrize("seed,proj_type,dtype,shape,k", PROP)
+def test_seed_consistency(gpu, seed, proj_type, dtype, shape, k):
+    # tests/test_jl.py:78-154: same seed -> same result, same instance and a new one
+    g = torch.testing.make_tensor(*shape, device=gpu, dtype=dtype)
+    p1 = _projector(shape[1], k, seed, proj_type, dtype)
+    a = p1.project(g, model_id=0)
+    assert torch.equal(a, p1.project(g, model_id=0))
+    assert torch.equal(a, _projector(shape[1], k, seed, proj_type, dtype).project(g, model_id=0))
+    # another model id or seed is another matrix (trak/projectors.py:409)
+    assert not torch.equal(a, p1.project(g, model_id=1))
+    assert not torch.equal(a, _projector(shape[1], k, seed + 1, proj_type, dtype).project(g, model_id=0))
+    # model_id enters as seed + 10^4 * model_id
+    assert torch.equal(p1.project(g, model_id=2), _projector(shape[1], k, seed + 20_000, proj_type, dtype).project(g, model_id=0))
+
+
+@pytest.mark.parametrize("proj_type", [ProjectionType.normal, ProjectionType.rademacher])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
+def test_norm_and_product_preservation(gpu, proj_type, dtype):
+    # tests/test_jl.py:159-285 with the tests' own tolerances
+    shape, k, seed = (16, 10_002), 4096, 1
+    g = torch.testing.make_tensor(*shape, device=gpu, dtype=dtype)
+    p = _projector(shape[1], k, seed, proj_type, dtype).project(g, model_id=0)
+    rng = np.random.default_rng(0)
+    delta = 0.05
+    eps = np.sqrt(np.log(1 / delta) / k)
+    ok = 0
+    for _ in range(100):
+        i, j = rng.choice(shape[0], size=2)
+        n = (g[i].float() - g[j].float()).norm()
+        pn = (p[i] - p[j]).norm() / np.sqrt(k)
+        ok += int((n - pn).abs().item() <= 35 * eps * n.item())
+    assert ok >= 100 * (1 - 3 * delta)
+    # JL proper: squared norms within a few standard deviations (sqrt(2/k) relative)
+    ratio = (p.norm(dim=1) ** 2 / k) / (g.float().norm(dim=1) ** 2)
+    assert torch.all((ratio - 1).abs() < 6 * math.sqrt(2 / k))
+
+
+@pytest.mark.parametrize("proj_type", [ProjectionType.normal, ProjectionType.rademacher])
+def test_every_feature_contributes(gpu, proj_type):
+    # tests/test_jl.py:290-389: single / first / last non-zero coordinate -> no output is zero
+    B, P, k = 9, 10_002, 1024
+    rng = np.random.default_rng(1)
+    proj = _projector(P, k, 123, proj_type, torch.float32)
+    for coords in ([0] * B, [P - 1] * B, rng.integers(0, P, size=B).tolist()):
+        g = torch.zeros(B, P, device=gpu)
+        for r, c in enumerate(coords):
+            g[r, c] = 1.0 + r
+        p = proj.project(g, model_id=0)
+        assert (~torch.isclose(p, torch.zeros_like(p))).all().item()
+
+
+@pytest.mark.parametrize("proj_type", [ProjectionType.normal, ProjectionType.rademacher])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
+def test_same_rows_same_features_through_chunks(gpu, proj_type, dtype):
+    # tests/test_jl.py:394-446 and tests/test_jl_additional.py:63-87, on a forced 3-chunk split
+    B, P, k = 8, 30_003, 512
+    g = torch.testing.make_tensor(B, P, device=gpu, dtype=dtype)
+    g[-1] = g[0]
+    chunks = {i: x for i, x in enumerate(torch.chunk(g, 3, dim=1))}
+    sizes = [v.size(1) for v in chunks.values()]
+    seeds = np.random.default_rng(5).integers(low=0, high=500, size=3)   # trak/traker.py:294-296
+    per_chunk = [_projector(sz, k, int(seeds[i]), proj_type, dtype) for i, sz in enumerate(sizes)]
+    proj = ChunkedCudaProjector(per_chunk, max(sizes), sizes, B, "cuda:0", dtype)
+    p = proj.project(chunks, model_id=0)
+    assert p.shape == (B, k) and p.dtype == dtype               # trak/projectors.py:472-474
+    assert torch.equal(p[0], p[-1])
+    # the chunked result is the sum of the per-chunk projections (trak/projectors.py:490-514)
+    want = sum(per_chunk[i].project(chunks[i].contiguous(), model_id=0) for i in range(3))
+    assert torch.allclose(p.float(), want.to(dtype).float(), rtol=2e-2 if dtype != torch.float32 else 1e-6, atol=1e-2)
+    proj.free_memory()
+
+
+def test_orthogonality(gpu):
+    # tests/test_jl.py:451-490
+    B, P, k = 8, 10_000, 4096
+    proj = _projector(P, k, 0, ProjectionType.rademacher, torch.float32)
+    ok = 0
+    for _ in range(10):
+        g = torch.testing.make_tensor(B, P, device=gpu, dtype=torch.float32)
+        g[-1] -= g[0] @ g[-1] / (g[0].norm() ** 2) * g[0]
+        p = proj.project(g, model_id=0)
+        ok += int(abs((p[0] @ p[-1]).item()) / k < 0.1 * (g[0].norm() * g[-1].norm()).item())
+    assert ok > 3
+
+
+def test_tile_count_changes_the_matrix_and_can_be_pinned(gpu):
+    # the matrix depends on num_feature_tiles (fast_jl/random.cuh:15-17 with tile = blockIdx.y);
+    # pinning num_sms reproduces another device's matrix (tests/test_jl_gpu_compatibility.py:59)
+    g = torch.testing.make_tensor(8, 10_000, device=gpu, dtype=torch.float16)
+    a = _projector(10_000, 512, 0, ProjectionType.rademacher, torch.float16, num_sms=108).project(g, 0)
+    b = _projector(10_000, 512, 0, ProjectionType.rademacher, torch.float16, num_sms=108).project(g, 0)
+    c = _projector(10_000, 512, 0, ProjectionType.rademacher, torch.float16).project(g, 0)
+    assert torch.equal(a, b) and not torch.equal(a, c)
+    assert torch.equal(a, fast_jl.project_rademacher_8(g, 512, 0, 108))
+
+
+def test_dict_input_is_vectorized_in_dict_order(gpu):
+    g = {"w": torch.randn(4, 3, 50, device=gpu), "b": torch.randn(4, device=gpu), "v": torch.randn(4, 70, device=gpu)}
+    flat = torch.cat([g["w"].reshape(4, -1), g["b"].reshape(4, 1), g["v"]], dim=1)
+    proj = _projector(flat.shape[1], 512, 9, ProjectionType.rademacher, torch.float32)
+    assert torch.equal(proj.project(g, model_id=0), proj.project(flat, model_id=0))
+
+
+# ---- full benchmark shape: size-independent properties and a column sample ---------------------
+
+
+def test_full_size_resnet18_shape(gpu, c_oracle):
+    B, P, k, seed = 32, 11_689_512, 4096, 7
+    tiles = 256
+    ones = torch.ones(B, P, dtype=torch.float16, device=gpu)
+    out = fast_jl.project_rademacher_32(ones, k, seed, tiles)
+    assert torch.all(out == out.round()) and torch.all(out % 2 == P % 2)      # parity closed form
+    assert torch.all(out == out[0:1])                                          # equal rows
+    # column sums of S are ~ N(0, P): the spread of the all-ones outputs must look like it
+    z = out[0].double() / math.sqrt(P)
+    assert abs(z.mean().item()) < 5 / math.sqrt(k) and abs(z.std().item() - 1) < 0.1
+    del ones
+    gen = torch.Generator(device="cpu").manual_seed(20_003)
+    blocks = 62
+    scale = 10 ** (torch.rand(blocks, generator=gen) * 3 - 5)
+    edges = torch.linspace(0, P, blocks + 1).long()
+    g = torch.randn(B, P, generator=gen)
+    for i in range(blocks):
+        g[:, edges[i] : edges[i + 1]] *= scale[i]
+    g = g.half().to(gpu)
+    out = fast_jl.project_rademacher_32(g, k, seed, tiles)
+    # exact linearity under a power-of-two scale (fp16 * 2 is exact away from overflow)
+    assert torch.equal(fast_jl.project_rademacher_32(g * 2, k, seed, tiles), out * 2)
+    g32 = to_f32_numpy(g)
+    for c in (0, 2049, 4095):
+        want = c_oracle.project(g32, seed, tiles, c, 1, R)[:, 0]
+        got = out[:, c].cpu().numpy().astype(np.float64)
+        assert np.linalg.norm(got - want) / np.linalg.norm(want) < 1e-3

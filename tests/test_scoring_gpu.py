@@ -1,0 +1,116 @@
+"""GPU parity tests of the scoring path (fp32 MFMA GEMMs + SPD inverse) against the float64
+oracle.  Tolerance: 1e-4 relative (to the largest magnitude of the result) as stated for the
+scores; GEMMs alone are held to 2e-6."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import score_oracle as so
+from trak_amd import BasicScoreComputer, get_matrix_mult
+from trak_amd.utils import gemm_nt, gemm_tn, spd_inverse
+
+pytestmark = pytest.mark.gpu
+
+
+def rel_max(got, want):
+    got = np.asarray(got, dtype=np.float64)
+    want = np.asarray(want, dtype=np.float64)
+    return np.abs(got - want).max() / max(np.abs(want).max(), 1e-300)
+
+
+@pytest.mark.parametrize("M,N,K", [(128, 128, 16), (256, 384, 64), (1, 1, 1), (130, 70, 33), (1000, 513, 257), (64, 2048, 4096)])
+def test_gemm_nt(gpu, M, N, K):
+    gen = torch.Generator(device="cpu").manual_seed(M * 7 + N)
+    a, b = torch.randn(M, K, generator=gen), torch.randn(N, K, generator=gen)
+    want = a.double().numpy() @ b.double().numpy().T
+    got = gemm_nt(a.to(gpu), b.to(gpu))
+    assert got.shape == (M, N) and rel_max(got.cpu().numpy(), want) < 2e-6
+    # alpha, beta and the row scale epilogue
+    c0 = torch.randn(M, N, generator=gen)
+    rs = torch.rand(M, generator=gen)
+    got = gemm_nt(a.to(gpu), b.to(gpu), out=c0.clone().to(gpu), alpha=0.5, beta=-2.0, row_scale=rs.to(gpu))
+    want2 = (0.5 * want - 2.0 * c0.double().numpy()) * rs.double().numpy()[:, None]
+    assert rel_max(got.cpu().numpy(), want2) < 2e-6
+
+
+@pytest.mark.parametrize("M,N,K", [(128, 128, 16), (96, 200, 1000), (33, 17, 5), (512, 512, 2050)])
+def test_gemm_tn(gpu, M, N, K):
+    gen = torch.Generator(device="cpu").manual_seed(M + N + K)
+    a, b = torch.randn(K, M, generator=gen), torch.randn(K, N, generator=gen)
+    want = a.double().numpy().T @ b.double().numpy()
+    got = gemm_tn(a.to(gpu), b.to(gpu))
+    assert rel_max(got.cpu().numpy(), want) < 2e-6
+    acc = gemm_tn(a.to(gpu), b.to(gpu), out=got.clone(), beta=1.0)
+    assert rel_max(acc.cpu().numpy(), 2 * want) < 2e-6
+
+
+def test_gemm_on_strided_views(gpu):
+    gen = torch.Generator(device="cpu").manual_seed(3)
+    big_a, big_b = torch.randn(300, 200, generator=gen).to(gpu), torch.randn(150, 200, generator=gen).to(gpu)
+    a, b = big_a[10:210, 3:131], big_b[5:105, 3:131]           # unaligned start, pitch 200
+    out = torch.zeros(256, 160, device=gpu)
+    gemm_nt(a, b, out=out[20:220, 7:107])
+    want = a.double().cpu().numpy() @ b.double().cpu().numpy().T
+    assert rel_max(out[20:220, 7:107].cpu().numpy(), want) < 2e-6
+    assert out[:20].abs().max() == 0 and out[:, :7].abs().max() == 0 and out[:, 107:].abs().max() == 0
+
+
+@pytest.mark.parametrize("n,lam", [(128, 0.0), (100, 0.5), (384, 1e-3), (513, 0.0), (1000, 1e-3)])
+def test_spd_inverse(gpu, n, lam):
+    gen = torch.Generator(device="cpu").manual_seed(n)
+    x = torch.randn(3 * n, n, generator=gen) / math.sqrt(n)
+    a = (x.T @ x).contiguous()
+    a = (a + a.T) / 2
+    want = np.linalg.inv(a.double().numpy() + lam * np.eye(n))
+    inv, mean_abs = spd_inverse(a.to(gpu), lambda_reg=lam, normalize=False)
+    assert rel_max(inv.cpu().numpy(), want) < 1e-4
+    assert abs(mean_abs.item() - np.abs(want).mean()) / np.abs(want).mean() < 1e-4
+    invn, m2 = spd_inverse(a.to(gpu), lambda_reg=lam, normalize=True)
+    assert rel_max(invn.cpu().numpy(), want / np.abs(want).mean()) < 1e-4
+    assert torch.equal(m2, mean_abs)
+    # (A + lambda I) inv = I
+    prod = (a.double().numpy() + lam * np.eye(n)) @ inv.double().cpu().numpy()
+    assert np.abs(prod - np.eye(n)).max() < 1e-3
+
+
+def test_spd_inverse_closed_forms_and_failure(gpu):
+    d = torch.arange(1, 201, dtype=torch.float32)
+    inv, _ = spd_inverse(torch.diag(d * d).to(gpu), lambda_reg=0.5)
+    assert torch.allclose(inv.diagonal().cpu(), 1.0 / (d * d + 0.5), rtol=1e-6)
+    assert (inv - torch.diag(inv.diagonal())).abs().max() == 0
+    ident, m = spd_inverse(torch.eye(300, device=gpu), lambda_reg=1.0, normalize=True)
+    assert torch.allclose(ident, torch.eye(300, device=gpu) * 300.0)        # (I/2) / mean|I/2|
+    assert abs(m.item() - 0.5 / 300) < 1e-9
+    bad = torch.eye(140)
+    bad[130, 130] = -1.0
+    with pytest.raises(torch.linalg.LinAlgError):
+        spd_inverse(bad.to(gpu))
+
+
+@pytest.mark.parametrize("N,k,M,lam,max_dim", [(700, 512, 90, 1e-3, 20_000), (2500, 1024, 300, 0.0, 1000), (333, 100, 17, 1e-2, 100)])
+def test_score_computer_matches_float64_oracle(gpu, N, k, M, lam, max_dim):
+    gen = torch.Generator(device="cpu").manual_seed(N + k)
+    X = torch.randn(N, k, generator=gen) / math.sqrt(k)
+    Xt = torch.randn(M, k, generator=gen) / math.sqrt(k)
+    otl = torch.rand(N, generator=gen)
+    sc = BasicScoreComputer(dtype=torch.float32, device="cuda:0", CUDA_MAX_DIM_SIZE=max_dim, lambda_reg=lam)
+    xtx_want = so.xtx_f64(X.numpy())
+    feats_want, _, _ = so.x_xtx_inv_f64(X.numpy(), xtx_want, lam)
+    scores_want = so.scores_f64(feats_want, Xt.numpy())
+
+    for src in (X, X.to(gpu)):                               # host-resident (blocked) and device-resident
+        xtx = sc.get_xtx(src)
+        assert xtx.shape == (k, k) and rel_max(xtx.cpu().numpy(), xtx_want) < 1e-5
+        feats = sc.get_x_xtx_inv(src, xtx)
+        assert feats.shape == (N, k) and rel_max(feats.cpu().numpy(), feats_want) < 1e-4
+        acc = torch.zeros(N, M)
+        sc.get_scores(feats, Xt.to(gpu), accumulator=acc)     # [N_train, M_targets] (trak/score_computers.py:90)
+        sc.get_scores(feats, Xt.to(gpu), accumulator=acc)
+        assert rel_max(acc.numpy(), 2 * scores_want) < 1e-4
+    # lambda = 0 identity: features^T X = I / mean|inv|
+    # fused finalize_scores epilogue (trak/traker.py:670-678) for one model
+    fused = sc.get_scaled_scores(feats, Xt.to(gpu), otl.to(gpu))
+    assert rel_max(fused.cpu().numpy(), so.finalize_scores_f64(scores_want, otl.numpy(), 1)) < 1e-4
+    assert rel_max(get_matrix_mult(feats, Xt.to(gpu)).cpu().numpy(), scores_want) < 1e-4

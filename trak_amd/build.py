@@ -1,0 +1,66 @@
+"""Builds trak_amd/libtrakhip.so from trak_amd/csrc/*.hip with hipcc for gfx950.
+
+Run as `python -m trak_amd.build`.  hipcc cross-compiles, so no GPU is needed to build.
+"""
+import os
+import subprocess
+import sys
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(HERE, "csrc")
+LIB = os.path.join(HERE, "libtrakhip.so")
+SOURCES = ["capi.hip", "project.hip", "gemm.hip", "spd.hip"]
+FLAGS = [
+    "--offload-arch=gfx950",
+    "-O3",
+    "-std=c++17",
+    "-fPIC",
+    "-Xclang",
+    "-target-feature",
+    "-Xclang",
+    "-packed-fp32-ops",
+    "-Wno-unused-command-line-argument",
+]
+
+
+def build(verbose=True, jobs=4):
+    """Compile every source to an object (in parallel) and link the shared library."""
+    hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+    objdir = os.path.join(HERE, "build")
+    os.makedirs(objdir, exist_ok=True)
+    procs = []
+    objs = []
+    for src in SOURCES:
+        obj = os.path.join(objdir, src.replace(".hip", ".o"))
+        objs.append(obj)
+        cmd = [hipcc, *FLAGS, "-c", os.path.join(CSRC, src), "-o", obj]
+        if verbose:
+            print(" ".join(cmd), flush=True)
+        procs.append((src, subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT)))
+        if len(procs) >= jobs:
+            _drain(procs)
+    _drain(procs)
+    cmd = [hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB, *objs]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    subprocess.check_call(cmd)
+    return LIB
+
+
+def _drain(procs):
+    while procs:
+        src, p = procs.pop(0)
+        out, _ = p.communicate()
+        text = out.decode(errors="replace")
+        # hipcc's host pass does not know the device-only target feature; that line is noise
+        text = "\n".join(l for l in text.splitlines() if "packed-fp32-ops" not in l)
+        if text.strip():
+            print(text)
+        if p.returncode != 0:
+            raise RuntimeError(f"hipcc failed on {src}")
+
+
+if __name__ == "__main__":
+    build()
+    print(LIB)
+    sys.exit(0)

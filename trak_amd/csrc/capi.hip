@@ -1,0 +1,80 @@
+// extern "C" surface of libtrakhip.so (declared in include/trakhip.h).
+#include "trakhip_internal.h"
+
+extern "C" {
+
+const char* trakhip_strerror(int code) {
+    switch (code) {
+        case TRAKHIP_OK: return "success";
+        case TRAKHIP_ERR_PROJ_DIM:
+            return "Invalid Number of JL dimensions it has to be a multiple of 512";
+        case TRAKHIP_ERR_SHAPE: return "invalid shape (empty, too large, or pitch smaller than row length)";
+        case TRAKHIP_ERR_DTYPE: return "input must be fp16, bf16 or fp32";
+        case TRAKHIP_ERR_PROJ_TYPE: return "unknown projection type";
+        case TRAKHIP_ERR_NULL: return "null pointer argument";
+        case TRAKHIP_ERR_WORKSPACE: return "workspace too small";
+        case TRAKHIP_ERR_ALIGN: return "pointer not sufficiently aligned";
+        case TRAKHIP_ERR_LAUNCH: return "HIP kernel launch failed";
+        case TRAKHIP_ERR_NOT_SPD: return "matrix is not positive definite";
+        case TRAKHIP_ERR_NO_DEVICE: return "no HIP device";
+        default: return "unknown trakhip error";
+    }
+}
+
+int trakhip_abi_version(void) { return 1; }
+
+size_t trakhip_project_workspace(uint64_t B, uint64_t P, uint32_t proj_dim, uint32_t num_feature_tiles) {
+    return trakhip::project_workspace_bytes(B, P, proj_dim, num_feature_tiles);
+}
+
+int trakhip_project(const void* in_dev, int in_dtype, uint64_t B, uint64_t P, uint64_t ld_in, float* out_dev,
+                    void* workspace_dev, size_t workspace_bytes, uint32_t proj_dim, uint32_t seed,
+                    uint32_t num_feature_tiles, int proj_type, void* stream) {
+    return trakhip::project(in_dev, in_dtype, B, P, ld_in, out_dev, workspace_dev, workspace_bytes, proj_dim,
+                            seed, num_feature_tiles, proj_type, static_cast<hipStream_t>(stream));
+}
+
+int trakhip_project_partials(const void* in_dev, int in_dtype, uint64_t B, uint64_t P, uint64_t ld_in,
+                             void* workspace_dev, size_t workspace_bytes, uint32_t proj_dim, uint32_t seed,
+                             uint32_t num_feature_tiles, int proj_type, void* stream) {
+    return trakhip::project_partials(in_dev, in_dtype, B, P, ld_in, workspace_dev, workspace_bytes, proj_dim, seed,
+                                     num_feature_tiles, proj_type, static_cast<hipStream_t>(stream));
+}
+
+int trakhip_project_reduce(const void* workspace_dev, uint64_t B, uint64_t P, uint32_t proj_dim,
+                           uint32_t num_feature_tiles, float scale, float* out_dev, void* stream) {
+    return trakhip::project_reduce(workspace_dev, B, P, proj_dim, num_feature_tiles, scale, out_dev,
+                                   static_cast<hipStream_t>(stream));
+}
+
+int trakhip_materialize(uint32_t seed, uint32_t num_feature_tiles, uint64_t P, uint64_t f0, uint64_t nf,
+                        uint32_t c0, uint32_t nc, int proj_type, float* out, int on_device, void* stream) {
+    if (on_device)
+        return trakhip::materialize_device(seed, num_feature_tiles, P, f0, nf, c0, nc, proj_type, out,
+                                           static_cast<hipStream_t>(stream));
+    return trakhip::materialize_host(seed, num_feature_tiles, P, f0, nf, c0, nc, proj_type, out);
+}
+
+int trakhip_gemm_nt(const float* A_dev, uint64_t lda, const float* B_dev, uint64_t ldb, float* C_dev,
+                    uint64_t ldc, uint64_t M, uint64_t N, uint64_t K, float alpha, float beta,
+                    const float* row_scale_dev, void* stream) {
+    return trakhip::gemm_nt(A_dev, lda, B_dev, ldb, C_dev, ldc, M, N, K, alpha, beta, row_scale_dev,
+                            static_cast<hipStream_t>(stream));
+}
+
+int trakhip_gemm_tn(const float* A_dev, uint64_t lda, const float* B_dev, uint64_t ldb, float* C_dev,
+                    uint64_t ldc, uint64_t M, uint64_t N, uint64_t K, float alpha, float beta, void* stream) {
+    return trakhip::gemm_tn(A_dev, lda, B_dev, ldb, C_dev, ldc, M, N, K, alpha, beta,
+                            static_cast<hipStream_t>(stream));
+}
+
+size_t trakhip_spd_inverse_workspace(uint64_t n) { return trakhip::spd_inverse_workspace_bytes(n); }
+
+int trakhip_spd_inverse(const float* A_dev, uint64_t lda, float lambda, float* inv_dev, uint64_t ldi,
+                        uint64_t n, int normalize, float* mean_abs_dev, int32_t* status_dev,
+                        void* workspace_dev, size_t workspace_bytes, void* stream) {
+    return trakhip::spd_inverse(A_dev, lda, lambda, inv_dev, ldi, n, normalize, mean_abs_dev, status_dev,
+                                workspace_dev, workspace_bytes, static_cast<hipStream_t>(stream));
+}
+
+}  // extern "C"

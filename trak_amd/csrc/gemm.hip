@@ -1,0 +1,228 @@
+// fp32 GEMM on the gfx950 matrix cores (v_mfma_f32_32x32x2_f32) for the scoring path.
+//
+// Stands in for the three torch matmuls of BasicScoreComputer: `block.T @ block`
+// (trak/score_computers.py:153), `block @ xtx_inv` (:176) and `features @ target_grads.t()`
+// (trak/utils.py:131), and is the building block of the blocked SPD inverse (spd.hip).
+//
+//   C[M, N] = alpha * op(A) * op(B) + beta * C      (then row i *= row_scale[i])
+//
+// Each operand is described by how it is stored relative to the contraction index k:
+//   "row-k"  (KMAJOR = false): element (x, k) at ptr[x * ld + k]   (k contiguous)
+//   "k-row"  (KMAJOR = true):  element (x, k) at ptr[k * ld + x]   (x contiguous)
+// NT = (row-k, row-k), TN = (k-row, k-row), NN = (row-k, k-row).
+//
+// Workgroup = 256 threads = 4 waves in a 2x2 grid, 128x128 tile of C, k step 16, two LDS
+// buffers.  A wave owns 64x64 of C = 2x2 MFMA tiles (64 accumulator VGPRs).  The MFMA sums
+// over k in any order, so lane half h (= lane / 32) is given k = 8*s + 4*h + t for the t-th
+// MFMA of sub-step s: a row-k operand then needs ONE 16-byte LDS read per four MFMAs.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "trakhip_internal.h"
+
+namespace {
+
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+
+constexpr int BM = 128, BN = 128, BKT = 16;
+constexpr int kThreads = 256;
+constexpr int kRowKStride = BKT + 4;   // floats; 80 B rows keep 16-byte reads conflict free
+constexpr int kKRowStride = BM;        // floats
+constexpr int kTileFloats = BM * kRowKStride;  // 2560 >= BKT * kKRowStride (2048)
+
+// ---- global -> registers -------------------------------------------------------------------
+
+template <bool KMAJOR, bool ALIGNED>
+__device__ __forceinline__ void load_tile(const float* __restrict__ p, uint64_t ld, uint64_t x0, uint64_t X,
+                                          uint64_t k0, uint64_t K, int tid, float4 (&r)[2]) {
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        const int id = tid + kThreads * i;
+        float4 v = {0.f, 0.f, 0.f, 0.f};
+        if (!KMAJOR) {
+            const uint64_t x = x0 + (id >> 2), k = k0 + 4 * (id & 3);
+            if (x < X && k < K) {
+                const float* q = p + x * ld + k;
+                if (ALIGNED && k + 4 <= K) {
+                    v = *reinterpret_cast<const float4*>(q);
+                } else {
+                    v.x = q[0];
+                    if (k + 1 < K) v.y = q[1];
+                    if (k + 2 < K) v.z = q[2];
+                    if (k + 3 < K) v.w = q[3];
+                }
+            }
+        } else {
+            const uint64_t k = k0 + (id >> 5), x = x0 + 4 * (id & 31);
+            if (k < K && x < X) {
+                const float* q = p + k * ld + x;
+                if (ALIGNED && x + 4 <= X) {
+                    v = *reinterpret_cast<const float4*>(q);
+                } else {
+                    v.x = q[0];
+                    if (x + 1 < X) v.y = q[1];
+                    if (x + 2 < X) v.z = q[2];
+                    if (x + 3 < X) v.w = q[3];
+                }
+            }
+        }
+        r[i] = v;
+    }
+}
+
+template <bool KMAJOR>
+__device__ __forceinline__ void store_tile(float* lds, int tid, const float4 (&r)[2]) {
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        const int id = tid + kThreads * i;
+        if (!KMAJOR)
+            *reinterpret_cast<float4*>(lds + (id >> 2) * kRowKStride + 4 * (id & 3)) = r[i];
+        else
+            *reinterpret_cast<float4*>(lds + (id >> 5) * kKRowStride + 4 * (id & 31)) = r[i];
+    }
+}
+
+// The 4 operand values (t = 0..3) of lane (x, h) for sub-step s.
+template <bool KMAJOR>
+__device__ __forceinline__ float4 read_frag(const float* lds, int x, int h, int s) {
+    if (!KMAJOR) return *reinterpret_cast<const float4*>(lds + x * kRowKStride + 8 * s + 4 * h);
+    const float* q = lds + (8 * s + 4 * h) * kKRowStride + x;
+    float4 v;
+    v.x = q[0];
+    v.y = q[kKRowStride];
+    v.z = q[2 * kKRowStride];
+    v.w = q[3 * kKRowStride];
+    return v;
+}
+
+template <bool AK, bool BK, bool ALIGNED>
+__global__ __launch_bounds__(kThreads, 2) void gemm_kernel(const float* __restrict__ A, uint64_t lda,
+                                                           const float* __restrict__ B, uint64_t ldb,
+                                                           float* __restrict__ C, uint64_t ldc, uint64_t M,
+                                                           uint64_t N, uint64_t K, float alpha, float beta,
+                                                           const float* __restrict__ row_scale,
+                                                           uint32_t tiles_n) {
+    __shared__ __attribute__((aligned(16))) float lds[2][2][kTileFloats];
+
+    const uint32_t tile_m = blockIdx.x / tiles_n, tile_n = blockIdx.x % tiles_n;
+    const uint64_t m0 = (uint64_t)tile_m * BM, n0 = (uint64_t)tile_n * BN;
+
+    const int tid = threadIdx.x;
+    const int wave = tid >> 6, lane = tid & 63;
+    const int wm = wave >> 1, wn = wave & 1;
+    const int x = lane & 31, h = lane >> 5;
+
+    floatx16 acc[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+    const uint64_t nk = (K + BKT - 1) / BKT;
+    float4 ra[2], rb[2];
+    if (nk) {
+        load_tile<AK, ALIGNED>(A, lda, m0, M, 0, K, tid, ra);
+        load_tile<BK, ALIGNED>(B, ldb, n0, N, 0, K, tid, rb);
+        store_tile<AK>(lds[0][0], tid, ra);
+        store_tile<BK>(lds[0][1], tid, rb);
+    }
+    __syncthreads();
+
+    for (uint64_t kt = 0; kt < nk; ++kt) {
+        const int cur = (int)(kt & 1);
+        if (kt + 1 < nk) {
+            load_tile<AK, ALIGNED>(A, lda, m0, M, (kt + 1) * BKT, K, tid, ra);
+            load_tile<BK, ALIGNED>(B, ldb, n0, N, (kt + 1) * BKT, K, tid, rb);
+        }
+        const float* as = lds[cur][0];
+        const float* bs = lds[cur][1];
+#pragma unroll
+        for (int s = 0; s < 2; ++s) {
+            float4 fa[2], fb[2];
+#pragma unroll
+            for (int i = 0; i < 2; ++i) fa[i] = read_frag<AK>(as, wm * 64 + 32 * i + x, h, s);
+#pragma unroll
+            for (int j = 0; j < 2; ++j) fb[j] = read_frag<BK>(bs, wn * 64 + 32 * j + x, h, s);
+#pragma unroll
+            for (int t = 0; t < 4; ++t)
+#pragma unroll
+                for (int i = 0; i < 2; ++i)
+#pragma unroll
+                    for (int j = 0; j < 2; ++j) {
+                        const float av = t == 0 ? fa[i].x : (t == 1 ? fa[i].y : (t == 2 ? fa[i].z : fa[i].w));
+                        const float bv = t == 0 ? fb[j].x : (t == 1 ? fb[j].y : (t == 2 ? fb[j].z : fb[j].w));
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(av, bv, acc[i][j], 0, 0, 0);
+                    }
+        }
+        if (kt + 1 < nk) {
+            store_tile<AK>(lds[cur ^ 1][0], tid, ra);
+            store_tile<BK>(lds[cur ^ 1][1], tid, rb);
+        }
+        __syncthreads();
+    }
+
+    // D[m][n] of a 32x32 MFMA: lane holds column n = lane % 32; register r holds row
+    // 8*(r/4) + 4*(lane/32) + r%4.
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const uint64_t row = m0 + wm * 64 + 32 * i + 8 * (r >> 2) + 4 * h + (r & 3);
+            if (row >= M) continue;
+            const float rs = row_scale ? row_scale[row] : 1.0f;
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                const uint64_t col = n0 + wn * 64 + 32 * j + x;
+                if (col >= N) continue;
+                float* c = C + row * ldc + col;
+                float v = alpha * acc[i][j][r];
+                if (beta != 0.0f) v += beta * *c;
+                *c = v * rs;
+            }
+        }
+    }
+}
+
+template <bool AK, bool BK>
+int launch(const float* A, uint64_t lda, const float* B, uint64_t ldb, float* C, uint64_t ldc, uint64_t M,
+           uint64_t N, uint64_t K, float alpha, float beta, const float* row_scale, hipStream_t s) {
+    if (M == 0 || N == 0) return TRAKHIP_OK;
+    if (!A || !B || !C) return TRAKHIP_ERR_NULL;
+    const uint64_t min_lda = AK ? M : K, min_ldb = BK ? N : K;
+    if (lda < min_lda || ldb < min_ldb || ldc < N) return TRAKHIP_ERR_SHAPE;
+    const uint64_t tm = (M + BM - 1) / BM, tn = (N + BN - 1) / BN;
+    if (tm * tn > 0x7FFFFFFFull) return TRAKHIP_ERR_SHAPE;
+    const bool aligned = (reinterpret_cast<uintptr_t>(A) % 16 == 0) && (reinterpret_cast<uintptr_t>(B) % 16 == 0) &&
+                         (lda % 4 == 0) && (ldb % 4 == 0);
+    const dim3 grid((uint32_t)(tm * tn)), block(kThreads);
+    if (aligned)
+        hipLaunchKernelGGL((gemm_kernel<AK, BK, true>), grid, block, 0, s, A, lda, B, ldb, C, ldc, M, N, K, alpha,
+                           beta, row_scale, (uint32_t)tn);
+    else
+        hipLaunchKernelGGL((gemm_kernel<AK, BK, false>), grid, block, 0, s, A, lda, B, ldb, C, ldc, M, N, K, alpha,
+                           beta, row_scale, (uint32_t)tn);
+    return hipGetLastError() == hipSuccess ? TRAKHIP_OK : TRAKHIP_ERR_LAUNCH;
+}
+
+}  // namespace
+
+namespace trakhip {
+
+int gemm_nt(const float* A, uint64_t lda, const float* B, uint64_t ldb, float* C, uint64_t ldc, uint64_t M,
+            uint64_t N, uint64_t K, float alpha, float beta, const float* row_scale, hipStream_t s) {
+    return launch<false, false>(A, lda, B, ldb, C, ldc, M, N, K, alpha, beta, row_scale, s);
+}
+
+int gemm_tn(const float* A, uint64_t lda, const float* B, uint64_t ldb, float* C, uint64_t ldc, uint64_t M,
+            uint64_t N, uint64_t K, float alpha, float beta, hipStream_t s) {
+    return launch<true, true>(A, lda, B, ldb, C, ldc, M, N, K, alpha, beta, nullptr, s);
+}
+
+int gemm_nn(const float* A, uint64_t lda, const float* B, uint64_t ldb, float* C, uint64_t ldc, uint64_t M,
+            uint64_t N, uint64_t K, float alpha, float beta, hipStream_t s) {
+    return launch<false, true>(A, lda, B, ldb, C, ldc, M, N, K, alpha, beta, nullptr, s);
+}
+
+}  // namespace trakhip

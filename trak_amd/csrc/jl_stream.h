@@ -1,0 +1,271 @@
+// Definition of the JL projection matrix S[f, c] as a counter-based random stream.
+//
+// Shared by the device kernels and the host-side materializer of this library.
+// (The CPU oracle used by the tests is written separately and does not include
+// this file.)
+//
+// What is kept from the reference kernel (fast_jl):
+//   * the feature axis is cut into T = min(P, num_feature_tiles) tiles of
+//     fts = ceil(P / T) features (fast_jl/fast_jl.cu:42, fast_jl/fast_jl_kernel.cuh:124);
+//   * every (JL column c, feature tile t) pair owns one random stream whose
+//     32-bit seed is  seed + 658105236*c + 359124577*t  with uint32 wrap-around
+//     (fast_jl/random.cuh:15-17);
+//   * entries are consumed in feature order inside a tile; a Rademacher entry
+//     costs one random bit, bit set -> +1 (fast_jl/random.cuh:33-37); a normal
+//     entry is a Box-Muller normal rounded to fp16 (fast_jl/random.cuh:50-60).
+//
+// What is new: the generator is Philox4x32-10 (the reference uses cuRAND XORWOW,
+// whose draws cannot be reproduced off an NVIDIA toolchain).  The stream of
+// (c, t) is the block sequence
+//       block(n) = Philox4x32-10(counter = (n, 0, 0, 0), key = (stream_seed, 0))
+// i.e. what curand_init(stream_seed, 0, 0) would address with a Philox state.
+//
+// Rademacher: feature offset o inside the tile uses block n = o / 128.  With
+//   j = o % 128, q = j / 8, i = j % 8  the entry is bit (15 - q + 16*(i & 1)) of
+//   word (i >> 1) of that block.  This places the 8 entries a lane feeds to one
+//   32x32x16 MFMA in bit 15 / bit 31 of (word << q), which is where the sign
+//   bits of a packed pair of 16-bit floats live.
+//
+// Normal: feature offset o uses block n = o / 4; words (0,1) give entries
+//   o%4 == 0 (cos branch) and 1 (sin branch), words (2,3) give 2 and 3.  The
+//   Box-Muller transform is spelled out below in IEEE binary32 operations
+//   (add, mul, fma, int<->float conversions of exactly representable values)
+//   so that any IEEE machine reproduces it bit for bit; the result is rounded
+//   to fp16 (round to nearest even).
+#pragma once
+#include <stdint.h>
+
+#if defined(__HIPCC__)
+#define JL_HD __host__ __device__ __forceinline__
+#else
+#define JL_HD inline
+#endif
+
+namespace jl {
+
+constexpr uint32_t kPhiloxM0 = 0xD2511F53u;
+constexpr uint32_t kPhiloxM1 = 0xCD9E8D57u;
+constexpr uint32_t kPhiloxW0 = 0x9E3779B9u;
+constexpr uint32_t kPhiloxW1 = 0xBB67AE85u;
+
+constexpr uint32_t kColumnStride = 658105236u;  // fast_jl/random.cuh:16
+constexpr uint32_t kTileStride = 359124577u;    // fast_jl/random.cuh:17
+
+struct u32x4 {
+    uint32_t x, y, z, w;
+};
+
+JL_HD uint32_t stream_seed(uint32_t seed, uint32_t column, uint32_t tile) {
+    return seed + kColumnStride * column + kTileStride * tile;
+}
+
+// Philox4x32-10, general counter and key.
+JL_HD u32x4 philox4x32_10(u32x4 c, uint32_t k0, uint32_t k1) {
+#pragma unroll
+    for (int r = 0; r < 10; ++r) {
+        const uint64_t p0 = (uint64_t)kPhiloxM0 * c.x;
+        const uint64_t p1 = (uint64_t)kPhiloxM1 * c.z;
+        u32x4 n;
+        n.x = (uint32_t)(p1 >> 32) ^ c.y ^ k0;
+        n.y = (uint32_t)p1;
+        n.z = (uint32_t)(p0 >> 32) ^ c.w ^ k1;
+        n.w = (uint32_t)p0;
+        c = n;
+        k0 += kPhiloxW0;
+        k1 += kPhiloxW1;
+    }
+    return c;
+}
+
+// Block n of the stream with seed s: counter (n, 0, 0, 0), key (s, 0).
+JL_HD u32x4 stream_block(uint32_t s, uint32_t n) {
+    u32x4 c = {n, 0u, 0u, 0u};
+    return philox4x32_10(c, s, 0u);
+}
+
+JL_HD uint32_t word_of(const u32x4& b, uint32_t i) {
+    return i == 0 ? b.x : (i == 1 ? b.y : (i == 2 ? b.z : b.w));
+}
+
+// Rademacher entry for offset j (0..127) inside a 128-entry block: 1 -> +1, 0 -> -1.
+JL_HD uint32_t rademacher_bit(const u32x4& b, uint32_t j) {
+    const uint32_t q = j >> 3, i = j & 7u;
+    return (word_of(b, i >> 1) >> (15u - q + 16u * (i & 1u))) & 1u;
+}
+
+// ---- Box-Muller in explicit binary32 arithmetic -------------------------------------------
+
+JL_HD float u2f(uint32_t u) {
+    union {
+        uint32_t u;
+        float f;
+    } v;
+    v.u = u;
+    return v.f;
+}
+JL_HD uint32_t f2u(float f) {
+    union {
+        uint32_t u;
+        float f;
+    } v;
+    v.f = f;
+    return v.u;
+}
+
+#if defined(__HIP_DEVICE_COMPILE__)
+#define JL_FMA(a, b, c) __builtin_fmaf((a), (b), (c))
+#define JL_MUL(a, b) __fmul_rn((a), (b))
+#define JL_ADD(a, b) __fadd_rn((a), (b))
+#else
+#define JL_FMA(a, b, c) __builtin_fmaf((a), (b), (c))
+JL_HD float jl_mul_(float a, float b) {
+    volatile float r = a * b;
+    return r;
+}
+JL_HD float jl_add_(float a, float b) {
+    volatile float r = a + b;
+    return r;
+}
+#define JL_MUL(a, b) jl::jl_mul_((a), (b))
+#define JL_ADD(a, b) jl::jl_add_((a), (b))
+#endif
+
+// Radius r = sqrt(-2 ln u), u = (2*(w >> 9) + 1) / 2^24 in (0, 1).
+JL_HD float bm_radius(uint32_t w) {
+    const uint32_t x = ((w >> 9) << 1) | 1u;  // odd, < 2^24: exact as float
+    const uint32_t xb = f2u((float)x);
+    int e = (int)(xb >> 23) - 127;
+    float m = u2f((xb & 0x007FFFFFu) | 0x3F800000u);  // [1, 2)
+    if (m > 1.41421354f) {
+        m = JL_MUL(m, 0.5f);
+        e += 1;
+    }
+    const float t = JL_ADD(m, -1.0f);
+    const float z = JL_MUL(t, t);
+    float p = 7.0376836292e-2f;
+    p = JL_FMA(p, t, -1.1514610310e-1f);
+    p = JL_FMA(p, t, 1.1676998740e-1f);
+    p = JL_FMA(p, t, -1.2420140846e-1f);
+    p = JL_FMA(p, t, 1.4249322787e-1f);
+    p = JL_FMA(p, t, -1.6668057665e-1f);
+    p = JL_FMA(p, t, 2.0000714765e-1f);
+    p = JL_FMA(p, t, -2.4999993993e-1f);
+    p = JL_FMA(p, t, 3.3333331174e-1f);
+    float y = JL_MUL(t, JL_MUL(z, p));
+    y = JL_FMA(-0.5f, z, y);
+    const float lnm = JL_ADD(t, y);
+    const float lnu = JL_FMA((float)(e - 24), 0.693147182f, lnm);
+    const float s = JL_MUL(-2.0f, lnu);
+    // sqrt(s) by three Newton steps on 1/sqrt(s) from an integer seed
+    float g = u2f(0x5f3759dfu - (f2u(s) >> 1));
+    const float h = JL_MUL(0.5f, s);
+#pragma unroll
+    for (int it = 0; it < 3; ++it) {
+        const float gg = JL_MUL(g, g);
+        const float c = JL_FMA(-h, gg, 1.5f);
+        g = JL_MUL(g, c);
+    }
+    return JL_MUL(s, g);
+}
+
+// cos and sin of the angle  (w >> 30) * pi/2 + (((w >> 6) & 0xFFFFFF) - 2^23) * (pi/2) / 2^24.
+JL_HD void bm_cossin(uint32_t w, float* c_out, float* s_out) {
+    const uint32_t qd = w >> 30;
+    const float fi = (float)((w >> 6) & 0x00FFFFFFu);
+    const float yv = JL_MUL(JL_ADD(fi, -8388608.0f), 9.36266447e-8f);  // (pi/2) * 2^-24
+    const float y2 = JL_MUL(yv, yv);
+    float ps = JL_FMA(-1.9515295891e-4f, y2, 8.3321608736e-3f);
+    ps = JL_FMA(ps, y2, -1.6666654611e-1f);
+    const float sn = JL_FMA(JL_MUL(ps, y2), yv, yv);
+    float pc = JL_FMA(2.443315711809948e-5f, y2, -1.388731625493765e-3f);
+    pc = JL_FMA(pc, y2, 4.166664568298827e-2f);
+    const float cs = JL_FMA(JL_MUL(pc, y2), y2, JL_FMA(-0.5f, y2, 1.0f));
+    const float c0 = (qd & 1u) ? sn : cs;
+    const float s0 = (qd & 1u) ? cs : sn;
+    const uint32_t negc = (((qd + 1u) >> 1) & 1u) << 31;
+    const uint32_t negs = (qd >> 1) << 31;
+    *c_out = u2f(f2u(c0) ^ negc);
+    *s_out = u2f(f2u(s0) ^ negs);
+}
+
+// The two binary32 normals of one word pair (before the rounding to fp16).
+JL_HD void bm_pair(uint32_t wa, uint32_t wb, float* z0, float* z1) {
+    const float r = bm_radius(wa);
+    float c, s;
+    bm_cossin(wb, &c, &s);
+    *z0 = JL_MUL(r, c);
+    *z1 = JL_MUL(r, s);
+}
+
+// binary32 -> binary16 bit pattern, round to nearest even (|v| < 65504 here, no NaN).
+JL_HD uint16_t f32_to_f16_rne(float v) {
+    const uint32_t b = f2u(v);
+    const uint32_t sign = (b >> 16) & 0x8000u;
+    const uint32_t a = b & 0x7FFFFFFFu;
+    if (a < 0x38800000u) {              // below the smallest normal half: subnormal or zero
+        if (a < 0x33000000u) return (uint16_t)sign;   // < 2^-25 rounds to zero
+        const uint32_t e = a >> 23;                    // 102..112
+        const uint32_t man = (a & 0x007FFFFFu) | 0x00800000u;
+        const uint32_t shift = 126u - e;               // 14..24
+        uint32_t hm = man >> shift;
+        const uint32_t rem = man & ((1u << shift) - 1u);
+        const uint32_t half = 1u << (shift - 1u);
+        if (rem > half || (rem == half && (hm & 1u))) hm += 1u;
+        return (uint16_t)(sign | hm);
+    }
+    uint32_t r = a - 0x38000000u;        // rebias exponent
+    const uint32_t rem = r & 0x1FFFu;
+    r >>= 13;
+    if (rem > 0x1000u || (rem == 0x1000u && (r & 1u))) r += 1u;
+    return (uint16_t)(sign | r);
+}
+
+JL_HD float f16_bits_to_f32(uint16_t hbits) {
+    const uint32_t sign = ((uint32_t)hbits & 0x8000u) << 16;
+    const uint32_t e = (hbits >> 10) & 0x1Fu;
+    const uint32_t m = hbits & 0x3FFu;
+    if (e == 0) {
+        // subnormal: m * 2^-24, exact in binary32
+        const float v = (float)m * 5.9604644775390625e-8f;
+        return u2f(f2u(v) | sign);
+    }
+    return u2f(sign | ((e + 112u) << 23) | (m << 13));
+}
+
+// ---- entry of the matrix --------------------------------------------------------------------
+
+// o = feature offset inside the tile.  Returns the value as binary32 (always exactly
+// representable in fp16).
+JL_HD float entry_rademacher(uint32_t sseed, uint32_t o) {
+    const u32x4 b = stream_block(sseed, o >> 7);
+    return rademacher_bit(b, o & 127u) ? 1.0f : -1.0f;
+}
+
+JL_HD uint16_t entry_normal_f16bits(uint32_t sseed, uint32_t o) {
+    const u32x4 b = stream_block(sseed, o >> 2);
+    const uint32_t e = o & 3u;
+    float z0, z1;
+    if (e < 2u)
+        bm_pair(b.x, b.y, &z0, &z1);
+    else
+        bm_pair(b.z, b.w, &z0, &z1);
+    return f32_to_f16_rne((e & 1u) ? z1 : z0);
+}
+
+JL_HD float entry_normal(uint32_t sseed, uint32_t o) {
+    return f16_bits_to_f32(entry_normal_f16bits(sseed, o));
+}
+
+// Tiling of the feature axis (fast_jl/fast_jl.cu:42, fast_jl/fast_jl_kernel.cuh:124).
+struct Tiling {
+    uint32_t tiles;      // T = min(P, num_feature_tiles)
+    uint64_t tile_size;  // fts = ceil(P / T)
+};
+JL_HD Tiling make_tiling(uint64_t P, uint32_t num_feature_tiles) {
+    Tiling t;
+    t.tiles = (uint64_t)num_feature_tiles < P ? num_feature_tiles : (uint32_t)P;
+    t.tile_size = (P - 1) / t.tiles + 1;
+    return t;
+}
+
+}  // namespace jl

@@ -1,0 +1,512 @@
+// JL projection  out[b, c] = sum_f G[b, f] * S[f, c]  for gfx950 (MI355X).
+//
+// Replaces project_kernel / project / fast_jl<> of the reference
+// (fast_jl/fast_jl_kernel.cuh:24-132, fast_jl/fast_jl.cu:29-79).  S is never
+// stored: every wave generates the entries it needs from the Philox stream
+// defined in jl_stream.h directly in the register layout of the B operand of
+// v_mfma_f32_32x32x16_{f16,bf16} and contracts them against gradient tiles that
+// the workgroup staged in LDS.
+//
+// Work decomposition
+//   workgroup = 4 waves = 512 JL columns x one feature tile (the reference's
+//               tile: fts = ceil(P / T) consecutive features);
+//   wave      = 4 groups of 32 columns (four 32x32 fp32 accumulators);
+//   lane      = (n = lane % 32, h = lane / 32): column n of each group, and the
+//               k-slots 8h..8h+7 of every MFMA.
+// The tile is walked in chunks of 256 features.  Lane half h owns features
+// [128h, 128h+128) of a chunk: MFMA number q (0..15) of the chunk contracts
+// features 128h + 8q + i (i = 0..7), so the 8 sign bits a lane needs for it sit
+// in bits 15/31 of (word_v << q), v = 0..3, of ONE Philox block per column per
+// chunk, and the A operand is 16 contiguous bytes of a gradient row.
+//
+// Partial sums of every feature tile go to a workspace [T, B, k] that a second
+// kernel adds up in tile order, so results do not depend on scheduling.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "jl_stream.h"
+#include "trakhip_internal.h"
+
+namespace {
+
+typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+
+constexpr int kWaves = 4;
+constexpr int kGroups = 4;                            // 32-column groups per wave
+constexpr int kThreads = kWaves * 64;                 // 256
+constexpr int kColsPerWG = kWaves * kGroups * 32;     // 512 (fast_jl_kernel.cuh:113)
+constexpr int kChunk = 256;                           // features per staged chunk
+constexpr int kLdsRow = kChunk + 8;                   // 16-bit elements; 528 B keeps b128 reads conflict free
+constexpr int kPlaneElems = 32 * kLdsRow;
+
+struct __attribute__((packed, aligned(2))) Raw16 {
+    uint32_t x, y, z, w;
+};
+struct __attribute__((packed, aligned(4))) Raw16f {
+    uint32_t x, y, z, w;
+};
+
+template <int IN>
+struct InTraits;
+template <>
+struct InTraits<TRAKHIP_F16> {
+    static constexpr int planes = 1;
+    static constexpr bool bf16 = false;
+};
+template <>
+struct InTraits<TRAKHIP_BF16> {
+    static constexpr int planes = 1;
+    static constexpr bool bf16 = true;
+};
+template <>
+struct InTraits<TRAKHIP_F32> {
+    static constexpr int planes = 3;  // x = b1 + b2 + b3 exactly, each a bf16
+    static constexpr bool bf16 = true;
+};
+
+__device__ __forceinline__ floatx16 mfma16(const uint4& a, const uint4& b, floatx16 c, bool bf16) {
+    if (bf16)
+        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a),
+                                                       __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8, a),
+                                                  __builtin_bit_cast(half8, b), c, 0, 0, 0);
+}
+
+// ---- staging of a [32 x 256] gradient chunk ------------------------------------------------
+
+// 16-bit inputs: every thread moves four 16-byte pieces.
+struct Stage16 {
+    uint4 v[4];
+
+    __device__ __forceinline__ void load(const uint16_t* __restrict__ g, uint64_t ld, uint32_t rows,
+                                         uint64_t f_begin, uint64_t f_end, int tid) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int id = tid + kThreads * i;
+            const uint32_t row = id >> 5, sg = id & 31;
+            const uint64_t f = f_begin + 8u * sg;
+            uint4 val = {0u, 0u, 0u, 0u};
+            if (row < rows && f < f_end) {
+                const uint16_t* p = g + (uint64_t)row * ld + f;
+                if (f + 8 <= f_end) {
+                    const Raw16 r = *reinterpret_cast<const Raw16*>(p);
+                    val = {r.x, r.y, r.z, r.w};
+                } else {
+                    uint32_t e[8];
+#pragma unroll
+                    for (int t = 0; t < 8; ++t) e[t] = (f + t < f_end) ? (uint32_t)p[t] : 0u;
+                    val = {e[0] | (e[1] << 16), e[2] | (e[3] << 16), e[4] | (e[5] << 16),
+                           e[6] | (e[7] << 16)};
+                }
+            }
+            v[i] = val;
+        }
+    }
+    __device__ __forceinline__ void store(uint16_t* lds, int tid) const {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int id = tid + kThreads * i;
+            const uint32_t row = id >> 5, sg = id & 31;
+            *reinterpret_cast<uint4*>(lds + row * kLdsRow + 8 * sg) = v[i];
+        }
+    }
+};
+
+// fp32 inputs: every thread moves eight pieces of 4 floats and splits each float into
+// three bf16 terms by truncation (x = b1 + b2 + b3 exactly).
+struct Stage32 {
+    uint4 v[8];
+
+    __device__ __forceinline__ void load(const float* __restrict__ g, uint64_t ld, uint32_t rows,
+                                         uint64_t f_begin, uint64_t f_end, int tid) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const int id = tid + kThreads * i;
+            const uint32_t row = id >> 6, sg = id & 63;
+            const uint64_t f = f_begin + 4u * sg;
+            uint4 val = {0u, 0u, 0u, 0u};
+            if (row < rows && f < f_end) {
+                const float* p = g + (uint64_t)row * ld + f;
+                if (f + 4 <= f_end) {
+                    const Raw16f r = *reinterpret_cast<const Raw16f*>(p);
+                    val = {r.x, r.y, r.z, r.w};
+                } else {
+                    val.x = __float_as_uint(p[0]);
+                    val.y = (f + 1 < f_end) ? __float_as_uint(p[1]) : 0u;
+                    val.z = (f + 2 < f_end) ? __float_as_uint(p[2]) : 0u;
+                    val.w = 0u;
+                }
+            }
+            v[i] = val;
+        }
+    }
+    __device__ __forceinline__ static void split(uint32_t xb, uint32_t& b1, uint32_t& b2, uint32_t& b3) {
+        const float x = __uint_as_float(xb);
+        const uint32_t h1 = xb & 0xFFFF0000u;
+        const float r1 = x - __uint_as_float(h1);
+        const uint32_t h2 = __float_as_uint(r1) & 0xFFFF0000u;
+        const float r2 = r1 - __uint_as_float(h2);
+        b1 = h1 >> 16;
+        b2 = h2 >> 16;
+        b3 = __float_as_uint(r2) >> 16;
+    }
+    __device__ __forceinline__ void store(uint16_t* lds, int tid) const {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const int id = tid + kThreads * i;
+            const uint32_t row = id >> 6, sg = id & 63;
+            uint32_t a[4][3];
+            split(v[i].x, a[0][0], a[0][1], a[0][2]);
+            split(v[i].y, a[1][0], a[1][1], a[1][2]);
+            split(v[i].z, a[2][0], a[2][1], a[2][2]);
+            split(v[i].w, a[3][0], a[3][1], a[3][2]);
+#pragma unroll
+            for (int pl = 0; pl < 3; ++pl) {
+                uint2 o = {a[0][pl] | (a[1][pl] << 16), a[2][pl] | (a[3][pl] << 16)};
+                *reinterpret_cast<uint2*>(lds + pl * kPlaneElems + row * kLdsRow + 4 * sg) = o;
+            }
+        }
+    }
+};
+
+template <int IN>
+struct StageOf {
+    typedef Stage16 type;
+    typedef uint16_t elem;
+};
+template <>
+struct StageOf<TRAKHIP_F32> {
+    typedef Stage32 type;
+    typedef float elem;
+};
+
+// ---- B operand generation --------------------------------------------------------------------
+
+// Packed pair of +-1 from bits 15 and 31 of m (bit set -> +1).  one = 0x3C003C00 (fp16) or
+// 0x3F803F80 (bf16).
+__device__ __forceinline__ uint32_t sign_pair(uint32_t m, uint32_t one) {
+    return (m & one) | (~m & (one | 0x80008000u));
+}
+
+__device__ __forceinline__ uint32_t pack_f16(float a, float b) {
+    return (uint32_t)jl::f32_to_f16_rne(a) | ((uint32_t)jl::f32_to_f16_rne(b) << 16);
+}
+
+// The 8 normal entries of offsets o0..o0+7 (o0 multiple of 8) as packed fp16.
+__device__ __forceinline__ uint4 normal_oct_f16(uint32_t sseed, uint32_t o0) {
+    const jl::u32x4 b0 = jl::stream_block(sseed, (o0 >> 2));
+    const jl::u32x4 b1 = jl::stream_block(sseed, (o0 >> 2) + 1u);
+    float z[8];
+    jl::bm_pair(b0.x, b0.y, &z[0], &z[1]);
+    jl::bm_pair(b0.z, b0.w, &z[2], &z[3]);
+    jl::bm_pair(b1.x, b1.y, &z[4], &z[5]);
+    jl::bm_pair(b1.z, b1.w, &z[6], &z[7]);
+    uint4 r;
+    r.x = pack_f16(z[0], z[1]);
+    r.y = pack_f16(z[2], z[3]);
+    r.z = pack_f16(z[4], z[5]);
+    r.w = pack_f16(z[6], z[7]);
+    return r;
+}
+
+// Split packed fp16 pairs into bf16 high and low terms (s = hi + lo exactly).
+__device__ __forceinline__ void f16pair_to_bf16_terms(uint32_t hp, uint32_t& hi, uint32_t& lo) {
+    const float a = jl::f16_bits_to_f32((uint16_t)(hp & 0xFFFFu));
+    const float b = jl::f16_bits_to_f32((uint16_t)(hp >> 16));
+    const uint32_t ah = __float_as_uint(a) & 0xFFFF0000u;
+    const uint32_t bh = __float_as_uint(b) & 0xFFFF0000u;
+    const float al = a - __uint_as_float(ah);
+    const float bl = b - __uint_as_float(bh);
+    hi = (ah >> 16) | bh;
+    lo = (__float_as_uint(al) >> 16) | (__float_as_uint(bl) & 0xFFFF0000u);
+}
+
+// Workgroup id -> (column block, tile).  Workgroups are handed to the 8 XCDs round-robin
+// by linear id; this puts the column blocks of one feature tile on the same XCD, next to
+// each other in time, so the tile is fetched from HBM once and then served by that XCD's L2.
+__device__ __forceinline__ void map_workgroup(uint32_t linear, uint32_t col_blocks, uint32_t& cb,
+                                              uint32_t& tile) {
+    const uint32_t xcd = linear & 7u;
+    const uint32_t idx = linear >> 3;
+    cb = idx % col_blocks;
+    tile = (idx / col_blocks) * 8u + xcd;
+}
+
+template <int IN, int PT>
+__global__ __launch_bounds__(kThreads, 2) void jl_project_kernel(
+    const void* __restrict__ g_in, uint64_t ld, uint32_t rows, uint64_t P, uint32_t k,
+    uint32_t seed, uint32_t tiles, uint64_t tile_size, float* __restrict__ partial) {
+    typedef InTraits<IN> Tr;
+    typedef typename StageOf<IN>::type Stage;
+    typedef typename StageOf<IN>::elem Elem;
+    constexpr bool kBf = Tr::bf16;
+    constexpr int kPlanes = Tr::planes;
+
+    __shared__ __attribute__((aligned(16))) uint16_t lds[kPlanes * kPlaneElems];
+
+    const uint32_t col_blocks = k / kColsPerWG;
+    uint32_t cb, tile;
+    map_workgroup(blockIdx.x, col_blocks, cb, tile);
+    if (tile >= tiles) return;  // padding of the tile count to a multiple of 8
+
+    const int tid = threadIdx.x;
+    const int wave = tid >> 6, lane = tid & 63;
+    const uint32_t n = lane & 31, h = lane >> 5;
+    const uint32_t col0 = cb * kColsPerWG + wave * (kGroups * 32) + n;
+
+    const uint64_t f_lo = (uint64_t)tile * tile_size;
+    const uint64_t f_hi = (f_lo + tile_size < P) ? f_lo + tile_size : P;  // may be <= f_lo
+    const uint32_t chunks = f_hi > f_lo ? (uint32_t)((f_hi - f_lo + kChunk - 1) / kChunk) : 0u;
+
+    uint32_t sseed[kGroups];
+#pragma unroll
+    for (int j = 0; j < kGroups; ++j) sseed[j] = jl::stream_seed(seed, col0 + 32u * j, tile);
+
+    floatx16 acc[kGroups];
+#pragma unroll
+    for (int j = 0; j < kGroups; ++j)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[j][r] = 0.0f;
+
+    const Elem* g = reinterpret_cast<const Elem*>(g_in);
+    Stage st;
+    if (chunks) st.load(g, ld, rows, f_lo, f_hi, tid);
+
+    const uint32_t one = kBf ? 0x3F803F80u : 0x3C003C00u;
+    const uint16_t* a_base = lds + n * kLdsRow + 128 * h;
+
+    for (uint32_t s = 0; s < chunks; ++s) {
+        __syncthreads();  // everyone is done reading the previous chunk
+        st.store(lds, tid);
+        __syncthreads();
+        if (s + 1 < chunks) st.load(g, ld, rows, f_lo + (uint64_t)(s + 1) * kChunk, f_hi, tid);
+
+        if (PT == TRAKHIP_RADEMACHER) {
+            jl::u32x4 w[kGroups];
+#pragma unroll
+            for (int j = 0; j < kGroups; ++j) w[j] = jl::stream_block(sseed[j], 2u * s + h);
+#pragma unroll
+            for (int q = 0; q < 16; ++q) {
+                uint4 a[kPlanes];
+#pragma unroll
+                for (int pl = 0; pl < kPlanes; ++pl)
+                    a[pl] = *reinterpret_cast<const uint4*>(a_base + pl * kPlaneElems + 8 * q);
+#pragma unroll
+                for (int j = 0; j < kGroups; ++j) {
+                    uint4 b;
+                    b.x = sign_pair(w[j].x << q, one);
+                    b.y = sign_pair(w[j].y << q, one);
+                    b.z = sign_pair(w[j].z << q, one);
+                    b.w = sign_pair(w[j].w << q, one);
+#pragma unroll
+                    for (int pl = 0; pl < kPlanes; ++pl) acc[j] = mfma16(a[pl], b, acc[j], kBf);
+                }
+            }
+        } else {
+            const uint32_t o_chunk = s * (uint32_t)kChunk + 128u * h;
+#pragma unroll 1
+            for (int q = 0; q < 16; ++q) {
+                uint4 a[kPlanes];
+#pragma unroll
+                for (int pl = 0; pl < kPlanes; ++pl)
+                    a[pl] = *reinterpret_cast<const uint4*>(a_base + pl * kPlaneElems + 8 * q);
+#pragma unroll
+                for (int j = 0; j < kGroups; ++j) {
+                    const uint4 bh = normal_oct_f16(sseed[j], o_chunk + 8u * q);
+                    if (!kBf) {
+                        acc[j] = mfma16(a[0], bh, acc[j], false);
+                    } else {
+                        uint4 hi, lo;
+                        f16pair_to_bf16_terms(bh.x, hi.x, lo.x);
+                        f16pair_to_bf16_terms(bh.y, hi.y, lo.y);
+                        f16pair_to_bf16_terms(bh.z, hi.z, lo.z);
+                        f16pair_to_bf16_terms(bh.w, hi.w, lo.w);
+#pragma unroll
+                        for (int pl = 0; pl < kPlanes; ++pl) {
+                            acc[j] = mfma16(a[pl], hi, acc[j], true);
+                            acc[j] = mfma16(a[pl], lo, acc[j], true);
+                        }
+                    }
+                }
+            }
+        }
+    }
+
+    // D[m][n] of a 32x32 MFMA: lane holds column n = lane % 32 and, in register r, row
+    // m = 8*(r/4) + 4*(lane/32) + r%4.
+    float* out = partial + (uint64_t)tile * rows * k;
+#pragma unroll
+    for (int j = 0; j < kGroups; ++j) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const uint32_t m = 8u * (r >> 2) + 4u * h + (r & 3);
+            if (m < rows) out[(uint64_t)m * k + col0 + 32u * j] = acc[j][r];
+        }
+    }
+}
+
+// out[b, c] = sum over tiles, in tile order.
+__global__ __launch_bounds__(256) void jl_reduce_kernel(const float* __restrict__ partial,
+                                                        uint32_t tiles, uint64_t n4, float scale,
+                                                        float* __restrict__ out) {
+    const uint64_t i = (uint64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= n4) return;
+    const float4* p = reinterpret_cast<const float4*>(partial) + i;
+    float4 s = {0.f, 0.f, 0.f, 0.f};
+    for (uint32_t t = 0; t < tiles; ++t) {
+        const float4 v = p[(uint64_t)t * n4];
+        s.x += v.x;
+        s.y += v.y;
+        s.z += v.z;
+        s.w += v.w;
+    }
+    s.x *= scale;
+    s.y *= scale;
+    s.z *= scale;
+    s.w *= scale;
+    reinterpret_cast<float4*>(out)[i] = s;
+}
+
+// S[f0 + i, c0 + j] for i < nf, j < nc, written as binary32, row-major [nf, nc].
+__global__ __launch_bounds__(256) void jl_materialize_kernel(uint32_t seed, uint32_t tiles,
+                                                             uint64_t tile_size, uint64_t f0,
+                                                             uint64_t nf, uint32_t c0, uint32_t nc,
+                                                             int proj_type, float* __restrict__ out) {
+    const uint64_t idx = (uint64_t)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= nf * nc) return;
+    const uint64_t f = f0 + idx / nc;
+    const uint32_t c = c0 + (uint32_t)(idx % nc);
+    const uint32_t tile = (uint32_t)(f / tile_size);
+    const uint32_t o = (uint32_t)(f % tile_size);
+    const uint32_t ss = jl::stream_seed(seed, c, tile);
+    out[idx] = proj_type == TRAKHIP_RADEMACHER ? jl::entry_rademacher(ss, o) : jl::entry_normal(ss, o);
+}
+
+template <int IN, int PT>
+hipError_t launch_one(const void* in, uint64_t ld, uint32_t rows, uint64_t P, uint32_t k,
+                      uint32_t seed, const jl::Tiling& tl, float* partial, hipStream_t s) {
+    const uint32_t col_blocks = k / kColsPerWG;
+    const uint32_t tiles8 = (tl.tiles + 7u) / 8u * 8u;
+    const uint64_t wgs = (uint64_t)tiles8 * col_blocks;
+    if (wgs > 0x7FFFFFFFull) return hipErrorInvalidValue;
+    hipLaunchKernelGGL((jl_project_kernel<IN, PT>), dim3((uint32_t)wgs), dim3(kThreads), 0, s, in, ld,
+                       rows, P, k, seed, tl.tiles, tl.tile_size, partial);
+    return hipGetLastError();
+}
+
+typedef hipError_t (*LaunchFn)(const void*, uint64_t, uint32_t, uint64_t, uint32_t, uint32_t,
+                               const jl::Tiling&, float*, hipStream_t);
+
+LaunchFn pick(int dtype, int proj_type) {
+    static const LaunchFn table[3][2] = {
+        {launch_one<TRAKHIP_F16, TRAKHIP_RADEMACHER>, launch_one<TRAKHIP_F16, TRAKHIP_NORMAL>},
+        {launch_one<TRAKHIP_BF16, TRAKHIP_RADEMACHER>, launch_one<TRAKHIP_BF16, TRAKHIP_NORMAL>},
+        {launch_one<TRAKHIP_F32, TRAKHIP_RADEMACHER>, launch_one<TRAKHIP_F32, TRAKHIP_NORMAL>},
+    };
+    return table[dtype][proj_type];
+}
+
+}  // namespace
+
+namespace trakhip {
+
+size_t project_workspace_bytes(uint64_t B, uint64_t P, uint32_t k, uint32_t num_feature_tiles) {
+    if (B == 0 || P == 0 || k == 0 || num_feature_tiles == 0) return 0;
+    const jl::Tiling tl = jl::make_tiling(P, num_feature_tiles);
+    const uint64_t rows = B < 32 ? B : 32;
+    return (size_t)tl.tiles * rows * k * sizeof(float);
+}
+
+static int check_project_args(const void* in, int dtype, uint64_t B, uint64_t P, uint64_t ld, const void* ws,
+                              size_t ws_bytes, uint32_t k, uint32_t num_feature_tiles, int proj_type) {
+    if (dtype < TRAKHIP_F16 || dtype > TRAKHIP_F32) return TRAKHIP_ERR_DTYPE;
+    if (proj_type != TRAKHIP_RADEMACHER && proj_type != TRAKHIP_NORMAL) return TRAKHIP_ERR_PROJ_TYPE;
+    if (k == 0 || k % kColsPerWG != 0) return TRAKHIP_ERR_PROJ_DIM;
+    if (B == 0 || P == 0 || P > 0xFFFFFFFFull || num_feature_tiles == 0) return TRAKHIP_ERR_SHAPE;
+    if (ld < P) return TRAKHIP_ERR_SHAPE;
+    if (!in || !ws) return TRAKHIP_ERR_NULL;
+    if (ws_bytes < project_workspace_bytes(B, P, k, num_feature_tiles)) return TRAKHIP_ERR_WORKSPACE;
+    const size_t esz = dtype == TRAKHIP_F32 ? 4 : 2;
+    if ((reinterpret_cast<uintptr_t>(in) % esz) || (reinterpret_cast<uintptr_t>(ws) % 16)) return TRAKHIP_ERR_ALIGN;
+    return TRAKHIP_OK;
+}
+
+int project_partials(const void* in, int dtype, uint64_t B, uint64_t P, uint64_t ld, void* ws, size_t ws_bytes,
+                     uint32_t k, uint32_t seed, uint32_t num_feature_tiles, int proj_type, hipStream_t s) {
+    const int e = check_project_args(in, dtype, B, P, ld, ws, ws_bytes, k, num_feature_tiles, proj_type);
+    if (e) return e;
+    if (B > 32) return TRAKHIP_ERR_SHAPE;
+    const jl::Tiling tl = jl::make_tiling(P, num_feature_tiles);
+    if (pick(dtype, proj_type)(in, ld, (uint32_t)B, P, k, seed, tl, static_cast<float*>(ws), s) != hipSuccess)
+        return TRAKHIP_ERR_LAUNCH;
+    return TRAKHIP_OK;
+}
+
+int project_reduce(const void* ws, uint64_t B, uint64_t P, uint32_t k, uint32_t num_feature_tiles, float scale,
+                   float* out, hipStream_t s) {
+    if (k == 0 || k % kColsPerWG != 0) return TRAKHIP_ERR_PROJ_DIM;
+    if (B == 0 || B > 32 || P == 0 || P > 0xFFFFFFFFull || num_feature_tiles == 0) return TRAKHIP_ERR_SHAPE;
+    if (!ws || !out) return TRAKHIP_ERR_NULL;
+    if ((reinterpret_cast<uintptr_t>(ws) % 16) || (reinterpret_cast<uintptr_t>(out) % 16)) return TRAKHIP_ERR_ALIGN;
+    const jl::Tiling tl = jl::make_tiling(P, num_feature_tiles);
+    const uint64_t n4 = B * k / 4;
+    hipLaunchKernelGGL(jl_reduce_kernel, dim3((uint32_t)((n4 + 255) / 256)), dim3(256), 0, s,
+                       static_cast<const float*>(ws), tl.tiles, n4, scale, out);
+    return hipGetLastError() == hipSuccess ? TRAKHIP_OK : TRAKHIP_ERR_LAUNCH;
+}
+
+int project(const void* in, int dtype, uint64_t B, uint64_t P, uint64_t ld, float* out, void* ws,
+            size_t ws_bytes, uint32_t k, uint32_t seed, uint32_t num_feature_tiles, int proj_type,
+            hipStream_t s) {
+    const int e = check_project_args(in, dtype, B, P, ld, ws, ws_bytes, k, num_feature_tiles, proj_type);
+    if (e) return e;
+    if (!out) return TRAKHIP_ERR_NULL;
+    if (reinterpret_cast<uintptr_t>(out) % 16) return TRAKHIP_ERR_ALIGN;
+    const size_t esz = dtype == TRAKHIP_F32 ? 4 : 2;
+    // rows are walked 32 at a time (the reference walks 8, 16 or 32 at a time: fast_jl/fast_jl.cu:44-76)
+    for (uint64_t b0 = 0; b0 < B; b0 += 32) {
+        const uint64_t rows = (B - b0) < 32 ? (B - b0) : 32;
+        const char* src = static_cast<const char*>(in) + b0 * ld * esz;
+        int r = project_partials(src, dtype, rows, P, ld, ws, ws_bytes, k, seed, num_feature_tiles, proj_type, s);
+        if (!r) r = project_reduce(ws, rows, P, k, num_feature_tiles, 1.0f, out + b0 * k, s);
+        if (r) return r;
+    }
+    return TRAKHIP_OK;
+}
+
+int materialize_device(uint32_t seed, uint32_t num_feature_tiles, uint64_t P, uint64_t f0, uint64_t nf,
+                       uint32_t c0, uint32_t nc, int proj_type, float* out, hipStream_t s) {
+    if (proj_type != TRAKHIP_RADEMACHER && proj_type != TRAKHIP_NORMAL) return TRAKHIP_ERR_PROJ_TYPE;
+    if (P == 0 || P > 0xFFFFFFFFull || num_feature_tiles == 0 || f0 + nf > P) return TRAKHIP_ERR_SHAPE;
+    if (nf == 0 || nc == 0) return TRAKHIP_OK;
+    if (!out) return TRAKHIP_ERR_NULL;
+    const jl::Tiling tl = jl::make_tiling(P, num_feature_tiles);
+    const uint64_t total = nf * nc;
+    if ((total + 255) / 256 > 0x7FFFFFFFull) return TRAKHIP_ERR_SHAPE;
+    hipLaunchKernelGGL(jl_materialize_kernel, dim3((uint32_t)((total + 255) / 256)), dim3(256), 0, s, seed,
+                       tl.tiles, tl.tile_size, f0, nf, c0, nc, proj_type, out);
+    return hipGetLastError() == hipSuccess ? TRAKHIP_OK : TRAKHIP_ERR_LAUNCH;
+}
+
+int materialize_host(uint32_t seed, uint32_t num_feature_tiles, uint64_t P, uint64_t f0, uint64_t nf,
+                     uint32_t c0, uint32_t nc, int proj_type, float* out) {
+    if (proj_type != TRAKHIP_RADEMACHER && proj_type != TRAKHIP_NORMAL) return TRAKHIP_ERR_PROJ_TYPE;
+    if (P == 0 || P > 0xFFFFFFFFull || num_feature_tiles == 0 || f0 + nf > P) return TRAKHIP_ERR_SHAPE;
+    if (nf == 0 || nc == 0) return TRAKHIP_OK;
+    if (!out) return TRAKHIP_ERR_NULL;
+    const jl::Tiling tl = jl::make_tiling(P, num_feature_tiles);
+    for (uint64_t i = 0; i < nf; ++i) {
+        const uint64_t f = f0 + i;
+        const uint32_t tile = (uint32_t)(f / tl.tile_size), o = (uint32_t)(f % tl.tile_size);
+        for (uint32_t j = 0; j < nc; ++j) {
+            const uint32_t ss = jl::stream_seed(seed, c0 + j, tile);
+            out[i * nc + j] =
+                proj_type == TRAKHIP_RADEMACHER ? jl::entry_rademacher(ss, o) : jl::entry_normal(ss, o);
+        }
+    }
+    return TRAKHIP_OK;
+}
+
+}  // namespace trakhip

@@ -1,0 +1,241 @@
+// (A + lambda I)^-1 for a symmetric positive definite fp32 matrix on one GPU, plus the
+// "divide by the mean absolute entry" step of the reference.
+//
+// Stands in for  xtx_inv = torch.linalg.inv(xtx + lambda_reg * eye);  xtx_inv /= xtx_inv.abs().mean()
+// (trak/score_computers.py:160-166).  The reference inverts with LU; the matrix here is a Gram
+// matrix plus a ridge, so this file uses a blocked Cholesky factorization instead:
+//
+//   1. W = A + lambda I, padded with an identity block up to a multiple of 128;
+//   2. for every 128-block column j:  one workgroup factors the diagonal block in LDS
+//      (L_jj) and inverts it; the panel below it is  W[j+1:, j] * L_jj^-T  and the trailing
+//      matrix gets  W -= panel * panel^T   (both MFMA GEMMs from gemm.hip);
+//   3. L^-1 by recursive halving: inv([[A,0],[B,C]]) = [[A^-1,0],[-C^-1 B A^-1, C^-1]]
+//      (two GEMMs per node of the recursion tree);
+//   4. inverse = L^-T L^-1 (one GEMM), then the mean of |.| by a two-stage reduction in a
+//      fixed order and a scaling pass.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "trakhip_internal.h"
+
+namespace {
+
+constexpr int NB = 128;
+constexpr int kLd = NB + 1;
+constexpr int kSumBlocks = 1024;
+
+__global__ __launch_bounds__(256) void spd_init_kernel(const float* __restrict__ A, uint64_t lda, float lambda,
+                                                       uint64_t n, uint64_t np, float* __restrict__ W,
+                                                       float* __restrict__ L, float* __restrict__ Li,
+                                                       int32_t* __restrict__ status) {
+    const uint64_t idx = (uint64_t)blockIdx.x * 256 + threadIdx.x;
+    if (idx == 0 && status) *status = 0;
+    if (idx >= np * np) return;
+    const uint64_t i = idx / np, j = idx % np;
+    float v;
+    if (i < n && j < n)
+        v = A[i * lda + j] + (i == j ? lambda : 0.0f);
+    else
+        v = (i == j) ? 1.0f : 0.0f;
+    W[idx] = v;
+    L[idx] = 0.0f;
+    Li[idx] = 0.0f;
+}
+
+// One workgroup: Cholesky of the 128x128 diagonal block at W (lower triangle used), L block to
+// Lout (upper part zero), its inverse to Linv_out.
+__global__ __launch_bounds__(256) void spd_diag_kernel(const float* __restrict__ W, uint64_t ldw,
+                                                       float* __restrict__ Lout, float* __restrict__ Linv_out,
+                                                       uint64_t ldl, int32_t block_index,
+                                                       int32_t* __restrict__ status) {
+    __shared__ float Ls[NB * kLd];
+    __shared__ float Xs[NB * kLd];
+    const int tid = threadIdx.x;
+
+    for (int e = tid; e < NB * NB; e += 256) {
+        const int i = e / NB, j = e % NB;
+        Ls[i * kLd + j] = (j <= i) ? W[(uint64_t)i * ldw + j] : 0.0f;
+        Xs[i * kLd + j] = 0.0f;
+    }
+    __syncthreads();
+
+    const int row = tid & (NB - 1), cpar = tid >> 7;  // row handled in the trailing update, column parity
+    for (int j = 0; j < NB; ++j) {
+        __syncthreads();  // the trailing update of the previous column is complete
+        float d = Ls[j * kLd + j];
+        if (!(d > 0.0f)) {
+            if (tid == 0 && status) {
+                if (*status == 0) *status = 1 + block_index * NB + j;
+            }
+            d = 1.0f;
+        }
+        const float sd = sqrtf(d);
+        const float inv_sd = 1.0f / sd;
+        __syncthreads();  // every thread has read the pivot
+        if (tid == 0) Ls[j * kLd + j] = sd;
+        if (tid > j && tid < NB) Ls[tid * kLd + j] *= inv_sd;
+        __syncthreads();
+        if (row > j) {
+            const float lij = Ls[row * kLd + j];
+            for (int c = j + 1 + cpar; c <= row; c += 2) Ls[row * kLd + c] -= lij * Ls[c * kLd + j];
+        }
+    }
+    __syncthreads();
+
+    // X = L^-1, one column per thread: forward substitution of the unit vectors.
+    if (tid < NB) {
+        const int c = tid;
+        Xs[c * kLd + c] = 1.0f / Ls[c * kLd + c];
+        for (int i = c + 1; i < NB; ++i) {
+            float sum = 0.0f;
+            for (int m = c; m < i; ++m) sum += Ls[i * kLd + m] * Xs[m * kLd + c];
+            Xs[i * kLd + c] = -sum / Ls[i * kLd + i];
+        }
+    }
+    __syncthreads();
+
+    for (int e = tid; e < NB * NB; e += 256) {
+        const int i = e / NB, j = e % NB;
+        Lout[(uint64_t)i * ldl + j] = Ls[i * kLd + j];
+        Linv_out[(uint64_t)i * ldl + j] = Xs[i * kLd + j];
+    }
+}
+
+__global__ __launch_bounds__(256) void abs_sum_kernel(const float* __restrict__ M, uint64_t ld, uint64_t n,
+                                                      float* __restrict__ partial) {
+    __shared__ float red[256];
+    const uint64_t total = n * n;
+    const uint64_t per = (total + kSumBlocks - 1) / kSumBlocks;
+    const uint64_t lo = (uint64_t)blockIdx.x * per;
+    const uint64_t hi = lo + per < total ? lo + per : total;
+    float s = 0.0f;
+    for (uint64_t e = lo + threadIdx.x; e < hi; e += 256) s += fabsf(M[(e / n) * ld + (e % n)]);
+    red[threadIdx.x] = s;
+    __syncthreads();
+    for (int w = 128; w > 0; w >>= 1) {
+        if ((int)threadIdx.x < w) red[threadIdx.x] += red[threadIdx.x + w];
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) partial[blockIdx.x] = red[0];
+}
+
+__global__ __launch_bounds__(256) void mean_kernel(const float* __restrict__ partial, uint64_t n,
+                                                   float* __restrict__ mean_out, float* __restrict__ mean_user) {
+    __shared__ float red[256];
+    float s = 0.0f;
+    for (int e = threadIdx.x; e < kSumBlocks; e += 256) s += partial[e];
+    red[threadIdx.x] = s;
+    __syncthreads();
+    for (int w = 128; w > 0; w >>= 1) {
+        if ((int)threadIdx.x < w) red[threadIdx.x] += red[threadIdx.x + w];
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) {
+        const float mean = red[0] / ((float)n * (float)n);
+        *mean_out = mean;
+        if (mean_user) *mean_user = mean;
+    }
+}
+
+__global__ __launch_bounds__(256) void scale_kernel(float* __restrict__ M, uint64_t ld, uint64_t n,
+                                                    const float* __restrict__ mean) {
+    const uint64_t idx = (uint64_t)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= n * n) return;
+    const float inv = 1.0f / *mean;
+    M[(idx / n) * ld + (idx % n)] *= inv;
+}
+
+struct Ctx {
+    float* W;
+    float* L;
+    float* Li;
+    uint64_t np;
+    hipStream_t s;
+    int err;
+};
+
+// Li[lo:hi, lo:hi] (block units) becomes the inverse of L[lo:hi, lo:hi]; diagonal blocks are
+// already inverted.
+void tri_inverse(Ctx& c, uint64_t lo, uint64_t hi) {
+    if (c.err || hi - lo <= 1) return;
+    const uint64_t mid = lo + (hi - lo) / 2;
+    tri_inverse(c, lo, mid);
+    tri_inverse(c, mid, hi);
+    const uint64_t r = (hi - mid) * NB, q = (mid - lo) * NB;
+    const uint64_t np = c.np;
+    const float* B = c.L + mid * NB * np + lo * NB;
+    const float* Ainv = c.Li + lo * NB * np + lo * NB;
+    const float* Cinv = c.Li + mid * NB * np + mid * NB;
+    float* T = c.W + mid * NB * np + lo * NB;  // W is free once the factorization is done
+    float* out = c.Li + mid * NB * np + lo * NB;
+    int e = trakhip::gemm_nn(B, np, Ainv, np, T, np, r, q, q, 1.0f, 0.0f, c.s);
+    if (!e) e = trakhip::gemm_nn(Cinv, np, T, np, out, np, r, q, r, -1.0f, 0.0f, c.s);
+    if (e) c.err = e;
+}
+
+}  // namespace
+
+namespace trakhip {
+
+size_t spd_inverse_workspace_bytes(uint64_t n) {
+    if (n == 0) return 0;
+    const uint64_t np = (n + NB - 1) / NB * NB;
+    return (size_t)(3 * np * np + kSumBlocks + 4) * sizeof(float);
+}
+
+int spd_inverse(const float* A, uint64_t lda, float lambda, float* inv, uint64_t ldi, uint64_t n, int normalize,
+                float* mean_abs, int32_t* status, void* ws, size_t ws_bytes, hipStream_t s) {
+    if (n == 0) return TRAKHIP_OK;
+    if (!A || !inv || !ws) return TRAKHIP_ERR_NULL;
+    if (lda < n || ldi < n || n > 0x40000) return TRAKHIP_ERR_SHAPE;
+    if (ws_bytes < spd_inverse_workspace_bytes(n)) return TRAKHIP_ERR_WORKSPACE;
+    if (reinterpret_cast<uintptr_t>(ws) % 16) return TRAKHIP_ERR_ALIGN;
+    const uint64_t np = (n + NB - 1) / NB * NB, nblk = np / NB;
+    float* W = static_cast<float*>(ws);
+    float* L = W + np * np;
+    float* Li = L + np * np;
+    float* partial = Li + np * np;
+    float* mean_dev = partial + kSumBlocks;
+
+    const uint64_t total = np * np;
+    hipLaunchKernelGGL(spd_init_kernel, dim3((uint32_t)((total + 255) / 256)), dim3(256), 0, s, A, lda, lambda, n,
+                       np, W, L, Li, status);
+    if (hipGetLastError() != hipSuccess) return TRAKHIP_ERR_LAUNCH;
+
+    for (uint64_t j = 0; j < nblk; ++j) {
+        const uint64_t off = j * NB * np + j * NB;
+        hipLaunchKernelGGL(spd_diag_kernel, dim3(1), dim3(256), 0, s, W + off, np, L + off, Li + off, np,
+                           (int32_t)j, status);
+        if (hipGetLastError() != hipSuccess) return TRAKHIP_ERR_LAUNCH;
+        if (j + 1 == nblk) break;
+        const uint64_t rows = np - (j + 1) * NB;
+        const uint64_t below = (j + 1) * NB * np + j * NB;
+        // panel = W[j+1:, j] * (L_jj^-1)^T
+        int e = gemm_nt(W + below, np, Li + off, np, L + below, np, rows, NB, NB, 1.0f, 0.0f, nullptr, s);
+        if (e) return e;
+        // trailing matrix -= panel * panel^T
+        const uint64_t tr = (j + 1) * NB * np + (j + 1) * NB;
+        e = gemm_nt(L + below, np, L + below, np, W + tr, np, rows, rows, NB, -1.0f, 1.0f, nullptr, s);
+        if (e) return e;
+    }
+
+    Ctx c = {W, L, Li, np, s, 0};
+    tri_inverse(c, 0, nblk);
+    if (c.err) return c.err;
+
+    // inverse = Li^T * Li (rows of Li at or beyond n do not reach the leading n x n block)
+    int e = gemm_tn(Li, np, Li, np, inv, ldi, n, n, n, 1.0f, 0.0f, s);
+    if (e) return e;
+
+    if (normalize || mean_abs) {
+        hipLaunchKernelGGL(abs_sum_kernel, dim3(kSumBlocks), dim3(256), 0, s, inv, ldi, n, partial);
+        hipLaunchKernelGGL(mean_kernel, dim3(1), dim3(256), 0, s, partial, n, mean_dev, mean_abs);
+        if (normalize)
+            hipLaunchKernelGGL(scale_kernel, dim3((uint32_t)((n * n + 255) / 256)), dim3(256), 0, s, inv, ldi, n,
+                               mean_dev);
+        if (hipGetLastError() != hipSuccess) return TRAKHIP_ERR_LAUNCH;
+    }
+    return TRAKHIP_OK;
+}
+
+}  // namespace trakhip

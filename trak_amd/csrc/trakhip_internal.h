@@ -1,0 +1,34 @@
+// Internal C++ interface between the C ABI (capi.hip) and the kernel files.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+#include <stdint.h>
+
+#include "../../include/trakhip.h"
+
+namespace trakhip {
+
+size_t project_workspace_bytes(uint64_t B, uint64_t P, uint32_t k, uint32_t num_feature_tiles);
+int project(const void* in, int dtype, uint64_t B, uint64_t P, uint64_t ld, float* out, void* ws,
+            size_t ws_bytes, uint32_t k, uint32_t seed, uint32_t num_feature_tiles, int proj_type,
+            hipStream_t s);
+int project_partials(const void* in, int dtype, uint64_t B, uint64_t P, uint64_t ld, void* ws, size_t ws_bytes,
+                     uint32_t k, uint32_t seed, uint32_t num_feature_tiles, int proj_type, hipStream_t s);
+int project_reduce(const void* ws, uint64_t B, uint64_t P, uint32_t k, uint32_t num_feature_tiles, float scale,
+                   float* out, hipStream_t s);
+int materialize_device(uint32_t seed, uint32_t num_feature_tiles, uint64_t P, uint64_t f0, uint64_t nf,
+                       uint32_t c0, uint32_t nc, int proj_type, float* out, hipStream_t s);
+int materialize_host(uint32_t seed, uint32_t num_feature_tiles, uint64_t P, uint64_t f0, uint64_t nf,
+                     uint32_t c0, uint32_t nc, int proj_type, float* out);
+
+int gemm_nt(const float* A, uint64_t lda, const float* B, uint64_t ldb, float* C, uint64_t ldc, uint64_t M,
+            uint64_t N, uint64_t K, float alpha, float beta, const float* row_scale, hipStream_t s);
+int gemm_tn(const float* A, uint64_t lda, const float* B, uint64_t ldb, float* C, uint64_t ldc, uint64_t M,
+            uint64_t N, uint64_t K, float alpha, float beta, hipStream_t s);
+int gemm_nn(const float* A, uint64_t lda, const float* B, uint64_t ldb, float* C, uint64_t ldc, uint64_t M,
+            uint64_t N, uint64_t K, float alpha, float beta, hipStream_t s);
+size_t spd_inverse_workspace_bytes(uint64_t n);
+int spd_inverse(const float* A, uint64_t lda, float lambda, float* inv, uint64_t ldi, uint64_t n,
+                int normalize, float* mean_abs, int32_t* status, void* ws, size_t ws_bytes, hipStream_t s);
+
+}  // namespace trakhip

@@ -1,0 +1,206 @@
+"""Helpers on either side of the projection and scoring kernels.
+
+Mirrors the hot-path part of the reference's trak/utils.py: `vectorize` (:80-110),
+`get_parameter_chunk_sizes` (:297-331) and `get_matrix_mult` (:248-294).
+"""
+import ctypes
+
+import numpy as np
+import torch
+
+from . import _lib
+
+
+def vectorize(g, arr=None, device="cuda"):
+    """Flattens a dict {name: grad[batch, ...]} to one [batch, num_params] tensor, in dict
+    order (trak/utils.py:80-110).  Gradients with fewer than two dims count as one column."""
+    if arr is None:
+        first = next(iter(g.values()))
+        batch_size = first.shape[0]
+        num_params = 0
+        for param in g.values():
+            assert param.shape[0] == batch_size
+            num_params += int(param.numel() / batch_size)
+        arr = torch.empty(size=(batch_size, num_params), dtype=first.dtype, device=device)
+
+    pointer = 0
+    for param in g.values():
+        if param.dim() < 2:
+            width = 1
+            flat = param.data.reshape(-1, 1)
+        else:
+            width = param[0].numel()
+            flat = param.flatten(start_dim=1).data
+        arr[:, pointer : pointer + width] = flat.to(device)
+        pointer += width
+    return arr
+
+
+def chunk_sizes_from_numels(numels, batch_size):
+    """Greedy grouping of parameter sizes into chunks whose element count times the batch
+    size stays below 2^32 (trak/utils.py:312-331).  Returns (max_chunk_size, params_per_chunk)."""
+    numels = np.array([int(n) for n in numels], dtype=np.int64)
+    max_chunk_size = int(np.iinfo(np.uint32).max // batch_size)
+    params_per_chunk = []
+    chunk_sum = 0
+    for ps in numels:
+        if chunk_sum + ps >= max_chunk_size:
+            params_per_chunk.append(int(chunk_sum))
+            chunk_sum = 0
+        chunk_sum += int(ps)
+    rest = int(numels.sum()) - int(np.sum(params_per_chunk))
+    if rest > 0:
+        params_per_chunk.append(rest)
+    return max_chunk_size, params_per_chunk
+
+
+def get_parameter_chunk_sizes(model, batch_size):
+    """(max_chunk_size, params_per_chunk) for a torch module (trak/utils.py:297-331)."""
+    return chunk_sizes_from_numels([p.numel() for p in model.parameters()], batch_size)
+
+
+def _as_f32_rows(t, name):
+    if t.dim() != 2:
+        raise RuntimeError(f"{name} must be 2D")
+    if t.dtype != torch.float32:
+        t = t.float()
+    if t.stride(1) != 1 or (t.shape[0] > 1 and t.stride(0) < t.shape[1]):
+        t = t.contiguous()
+    return t
+
+
+def _ld(t):
+    return t.stride(0) if t.shape[0] > 1 else max(t.shape[1], 1)
+
+
+def gemm_nt(a, b, out=None, alpha=1.0, beta=0.0, row_scale=None):
+    """out[M, N] = alpha * a[M, K] @ b[N, K].T + beta * out (fp32 on the GPU), rows optionally
+    scaled by row_scale[M]."""
+    a = _as_f32_rows(a, "a")
+    b = _as_f32_rows(b, "b")
+    if not a.is_cuda or b.device != a.device:
+        raise RuntimeError("gemm_nt needs both operands on the same GPU")
+    M, K = a.shape
+    N, K2 = b.shape
+    if K != K2:
+        raise RuntimeError(f"inner dimensions differ: {K} vs {K2}")
+    if out is None:
+        out = torch.empty((M, N), dtype=torch.float32, device=a.device)
+        beta = 0.0
+    if out.dtype != torch.float32 or out.shape != (M, N) or out.stride(1) != 1:
+        raise RuntimeError("out must be an fp32 [M, N] tensor with unit column stride")
+    rs = None
+    if row_scale is not None:
+        rs = row_scale.to(device=a.device, dtype=torch.float32).contiguous().reshape(-1)
+        if rs.numel() != M:
+            raise RuntimeError("row_scale must have M elements")
+    lib = _lib.load()
+    with torch.cuda.device(a.device):
+        stream = torch.cuda.current_stream(a.device).cuda_stream
+        code = lib.trakhip_gemm_nt(
+            ctypes.c_void_p(a.data_ptr()),
+            _ld(a),
+            ctypes.c_void_p(b.data_ptr()),
+            _ld(b),
+            ctypes.c_void_p(out.data_ptr()),
+            _ld(out),
+            M,
+            N,
+            K,
+            float(alpha),
+            float(beta),
+            ctypes.c_void_p(rs.data_ptr()) if rs is not None else None,
+            ctypes.c_void_p(stream),
+        )
+    _lib.check(code)
+    return out
+
+
+def gemm_tn(a, b, out=None, alpha=1.0, beta=0.0):
+    """out[M, N] = alpha * a[K, M].T @ b[K, N] + beta * out (fp32 on the GPU)."""
+    a = _as_f32_rows(a, "a")
+    b = _as_f32_rows(b, "b")
+    if not a.is_cuda or b.device != a.device:
+        raise RuntimeError("gemm_tn needs both operands on the same GPU")
+    K, M = a.shape
+    K2, N = b.shape
+    if K != K2:
+        raise RuntimeError(f"inner dimensions differ: {K} vs {K2}")
+    if out is None:
+        out = torch.empty((M, N), dtype=torch.float32, device=a.device)
+        beta = 0.0
+    if out.dtype != torch.float32 or out.shape != (M, N) or out.stride(1) != 1:
+        raise RuntimeError("out must be an fp32 [M, N] tensor with unit column stride")
+    lib = _lib.load()
+    with torch.cuda.device(a.device):
+        stream = torch.cuda.current_stream(a.device).cuda_stream
+        code = lib.trakhip_gemm_tn(
+            ctypes.c_void_p(a.data_ptr()),
+            _ld(a),
+            ctypes.c_void_p(b.data_ptr()),
+            _ld(b),
+            ctypes.c_void_p(out.data_ptr()),
+            _ld(out),
+            M,
+            N,
+            K,
+            float(alpha),
+            float(beta),
+            ctypes.c_void_p(stream),
+        )
+    _lib.check(code)
+    return out
+
+
+def spd_inverse(a, lambda_reg=0.0, normalize=False):
+    """(a + lambda*I)^-1 for a symmetric positive definite fp32 matrix on the GPU; with
+    normalize=True the result is divided by mean(|inverse|) (trak/score_computers.py:160-166).
+    Returns (inverse, mean_abs tensor of 1 element)."""
+    if a.dim() != 2 or a.shape[0] != a.shape[1]:
+        raise RuntimeError("spd_inverse needs a square matrix")
+    a = _as_f32_rows(a, "a")
+    if not a.is_cuda:
+        raise RuntimeError("spd_inverse needs a GPU tensor")
+    n = a.shape[0]
+    lib = _lib.load()
+    with torch.cuda.device(a.device):
+        inv = torch.empty((n, n), dtype=torch.float32, device=a.device)
+        mean_abs = torch.zeros(1, dtype=torch.float32, device=a.device)
+        status = torch.zeros(1, dtype=torch.int32, device=a.device)
+        nbytes = lib.trakhip_spd_inverse_workspace(n)
+        ws = torch.empty(max(nbytes, 1), dtype=torch.uint8, device=a.device)
+        stream = torch.cuda.current_stream(a.device).cuda_stream
+        code = lib.trakhip_spd_inverse(
+            ctypes.c_void_p(a.data_ptr()),
+            _ld(a),
+            float(lambda_reg),
+            ctypes.c_void_p(inv.data_ptr()),
+            n,
+            n,
+            int(bool(normalize)),
+            ctypes.c_void_p(mean_abs.data_ptr()),
+            ctypes.c_void_p(status.data_ptr()),
+            ctypes.c_void_p(ws.data_ptr()),
+            ws.numel(),
+            ctypes.c_void_p(stream),
+        )
+        _lib.check(code)
+        bad = int(status.item())  # also orders the workspace's lifetime after the kernels
+    if bad != 0:
+        raise torch.linalg.LinAlgError(
+            f"spd_inverse: the matrix is not positive definite (pivot {bad - 1} is not positive)"
+        )
+    return inv, mean_abs
+
+
+def get_matrix_mult(features, target_grads, target_dtype=None, batch_size=8096, use_blockwise=False):
+    """features @ target_grads.T (trak/utils.py:248-294).  On the GPU this is one fp32 MFMA GEMM;
+    CPU inputs take torch's matmul as in the reference (trak/utils.py:128-132).  The reference's
+    blockwise host-staged variant exists to fit small GPU memories; `use_blockwise` and
+    `batch_size` are accepted for signature compatibility and ignored."""
+    if target_dtype is None:
+        target_dtype = features.dtype
+    if features.device.type == "cpu":
+        return (features @ target_grads.t()).clone().to(target_dtype)
+    out = gemm_nt(features, target_grads.to(features.device))
+    return out.to(target_dtype)
