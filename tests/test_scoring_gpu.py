@@ -1,6 +1,6 @@
 """GPU parity tests of the scoring path (fp32 MFMA GEMMs + SPD inverse) against the float64
 oracle.  Tolerance: 1e-4 relative (to the largest magnitude of the result) as stated for the
-scores; GEMMs alone are held to 2e-6."""
+scores; GEMMs alone are held to the fp32 accumulation bound 1e-6 + 2e-7*sqrt(K)."""
 import math
 
 import numpy as np
@@ -12,6 +12,10 @@ from trak_amd import BasicScoreComputer, get_matrix_mult
 from trak_amd.utils import gemm_nt, gemm_tn, spd_inverse
 
 pytestmark = pytest.mark.gpu
+
+
+def gemm_tol(K):
+    return 1e-6 + 2e-7 * math.sqrt(K)
 
 
 def rel_max(got, want):
@@ -26,13 +30,13 @@ def test_gemm_nt(gpu, M, N, K):
     a, b = torch.randn(M, K, generator=gen), torch.randn(N, K, generator=gen)
     want = a.double().numpy() @ b.double().numpy().T
     got = gemm_nt(a.to(gpu), b.to(gpu))
-    assert got.shape == (M, N) and rel_max(got.cpu().numpy(), want) < 2e-6
+    assert got.shape == (M, N) and rel_max(got.cpu().numpy(), want) < gemm_tol(K)
     # alpha, beta and the row scale epilogue
     c0 = torch.randn(M, N, generator=gen)
     rs = torch.rand(M, generator=gen)
     got = gemm_nt(a.to(gpu), b.to(gpu), out=c0.clone().to(gpu), alpha=0.5, beta=-2.0, row_scale=rs.to(gpu))
     want2 = (0.5 * want - 2.0 * c0.double().numpy()) * rs.double().numpy()[:, None]
-    assert rel_max(got.cpu().numpy(), want2) < 2e-6
+    assert rel_max(got.cpu().numpy(), want2) < gemm_tol(K)
 
 
 @pytest.mark.parametrize("M,N,K", [(128, 128, 16), (96, 200, 1000), (33, 17, 5), (512, 512, 2050)])
@@ -41,9 +45,9 @@ def test_gemm_tn(gpu, M, N, K):
     a, b = torch.randn(K, M, generator=gen), torch.randn(K, N, generator=gen)
     want = a.double().numpy().T @ b.double().numpy()
     got = gemm_tn(a.to(gpu), b.to(gpu))
-    assert rel_max(got.cpu().numpy(), want) < 2e-6
+    assert rel_max(got.cpu().numpy(), want) < gemm_tol(K)
     acc = gemm_tn(a.to(gpu), b.to(gpu), out=got.clone(), beta=1.0)
-    assert rel_max(acc.cpu().numpy(), 2 * want) < 2e-6
+    assert rel_max(acc.cpu().numpy(), 2 * want) < gemm_tol(K)
 
 
 def test_gemm_on_strided_views(gpu):
@@ -53,7 +57,7 @@ def test_gemm_on_strided_views(gpu):
     out = torch.zeros(256, 160, device=gpu)
     gemm_nt(a, b, out=out[20:220, 7:107])
     want = a.double().cpu().numpy() @ b.double().cpu().numpy().T
-    assert rel_max(out[20:220, 7:107].cpu().numpy(), want) < 2e-6
+    assert rel_max(out[20:220, 7:107].cpu().numpy(), want) < gemm_tol(128)
     assert out[:20].abs().max() == 0 and out[:, :7].abs().max() == 0 and out[:, 107:].abs().max() == 0
 
 
