@@ -207,6 +207,8 @@ def main():
     ap.add_argument("--batches", type=int, default=16, help="distinct resident batches cycled through")
     ap.add_argument("--no-scoring", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run one 1 GiB device-to-device copy (reference point for rocprofv3 byte counters)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (see DESIGN.md, sharding note); "
@@ -219,6 +221,12 @@ def main():
         print("bench.py needs a GPU", file=sys.stderr)
         sys.exit(1)
     dev = torch.device("cuda:0")
+    if args.copy_calibration:
+        src = torch.ones(1 << 29, dtype=torch.float16, device=dev)
+        dst = torch.empty_like(src)
+        dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
     proj = bench_projection(torch, dev, args.steps, args.warmup, args.batches)
     torch.cuda.empty_cache()
     scoring = None if args.no_scoring else bench_scoring(torch, dev)

@@ -59,6 +59,15 @@ JL_HD uint32_t stream_seed(uint32_t seed, uint32_t column, uint32_t tile) {
     return seed + kColumnStride * column + kTileStride * tile;
 }
 
+// a ^ b ^ c: one v_bitop3_b32 (truth table 0x96) on the device.
+JL_HD uint32_t xor3(uint32_t a, uint32_t b, uint32_t c) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    return __builtin_amdgcn_bitop3_b32(a, b, c, 0x96);
+#else
+    return a ^ b ^ c;
+#endif
+}
+
 // Philox4x32-10, general counter and key.
 JL_HD u32x4 philox4x32_10(u32x4 c, uint32_t k0, uint32_t k1) {
 #pragma unroll
@@ -66,9 +75,9 @@ JL_HD u32x4 philox4x32_10(u32x4 c, uint32_t k0, uint32_t k1) {
         const uint64_t p0 = (uint64_t)kPhiloxM0 * c.x;
         const uint64_t p1 = (uint64_t)kPhiloxM1 * c.z;
         u32x4 n;
-        n.x = (uint32_t)(p1 >> 32) ^ c.y ^ k0;
+        n.x = xor3((uint32_t)(p1 >> 32), c.y, k0);
         n.y = (uint32_t)p1;
-        n.z = (uint32_t)(p0 >> 32) ^ c.w ^ k1;
+        n.z = xor3((uint32_t)(p0 >> 32), c.w, k1);
         n.w = (uint32_t)p0;
         c = n;
         k0 += kPhiloxW0;

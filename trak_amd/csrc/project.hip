@@ -82,6 +82,16 @@ struct Stage16 {
 
     __device__ __forceinline__ void load(const uint16_t* __restrict__ g, uint64_t ld, uint32_t rows,
                                          uint64_t f_begin, uint64_t f_end, int tid) {
+        if (rows == 32 && f_begin + kChunk <= f_end) {
+            // whole chunk in range (uniform test): four unguarded 16-byte loads
+            const uint16_t* p = g + (uint64_t)(tid >> 5) * ld + f_begin + 8u * (tid & 31);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const Raw16 r = *reinterpret_cast<const Raw16*>(p + (uint64_t)(8 * i) * ld);
+                v[i] = {r.x, r.y, r.z, r.w};
+            }
+            return;
+        }
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             const int id = tid + kThreads * i;
@@ -184,10 +194,19 @@ struct StageOf<TRAKHIP_F32> {
 
 // ---- B operand generation --------------------------------------------------------------------
 
-// Packed pair of +-1 from bits 15 and 31 of m (bit set -> +1).  one = 0x3C003C00 (fp16) or
-// 0x3F803F80 (bf16).
+// Packed pair of +-1 from bits 15 and 31 of m (bit set -> +1), every other bit of m ignored:
+// (m & one) | (~m & (one | 0x80008000)) as ONE v_bitop3_b32 (truth table 0xCA = a ? b : c).
+// one = 0x3C003C00 (fp16) or 0x3F803F80 (bf16).
 __device__ __forceinline__ uint32_t sign_pair(uint32_t m, uint32_t one) {
-    return (m & one) | (~m & (one | 0x80008000u));
+    return __builtin_amdgcn_bitop3_b32(m, one, one | 0x80008000u, 0xCA);
+}
+
+// Both words of a pair shifted left by q with one full-rate v_lshlrev_b64.  Bits that cross
+// from the low into the high word land below bit 15 (q <= 15) where sign_pair ignores them.
+__device__ __forceinline__ uint64_t shl_pair(uint64_t v, uint32_t q) {
+    uint64_t r;
+    asm("v_lshlrev_b64 %0, %1, %2" : "=v"(r) : "s"(q), "v"(v));
+    return r;
 }
 
 __device__ __forceinline__ uint32_t pack_f16(float a, float b) {
@@ -284,9 +303,13 @@ __global__ __launch_bounds__(kThreads, 2) void jl_project_kernel(
         if (s + 1 < chunks) st.load(g, ld, rows, f_lo + (uint64_t)(s + 1) * kChunk, f_hi, tid);
 
         if (PT == TRAKHIP_RADEMACHER) {
-            jl::u32x4 w[kGroups];
+            uint64_t w01[kGroups], w23[kGroups];
 #pragma unroll
-            for (int j = 0; j < kGroups; ++j) w[j] = jl::stream_block(sseed[j], 2u * s + h);
+            for (int j = 0; j < kGroups; ++j) {
+                const jl::u32x4 w = jl::stream_block(sseed[j], 2u * s + h);
+                w01[j] = ((uint64_t)w.y << 32) | w.x;
+                w23[j] = ((uint64_t)w.w << 32) | w.z;
+            }
 #pragma unroll
             for (int q = 0; q < 16; ++q) {
                 uint4 a[kPlanes];
@@ -295,11 +318,13 @@ __global__ __launch_bounds__(kThreads, 2) void jl_project_kernel(
                     a[pl] = *reinterpret_cast<const uint4*>(a_base + pl * kPlaneElems + 8 * q);
 #pragma unroll
                 for (int j = 0; j < kGroups; ++j) {
+                    const uint64_t m01 = q ? shl_pair(w01[j], q) : w01[j];
+                    const uint64_t m23 = q ? shl_pair(w23[j], q) : w23[j];
                     uint4 b;
-                    b.x = sign_pair(w[j].x << q, one);
-                    b.y = sign_pair(w[j].y << q, one);
-                    b.z = sign_pair(w[j].z << q, one);
-                    b.w = sign_pair(w[j].w << q, one);
+                    b.x = sign_pair((uint32_t)m01, one);
+                    b.y = sign_pair((uint32_t)(m01 >> 32), one);
+                    b.z = sign_pair((uint32_t)m23, one);
+                    b.w = sign_pair((uint32_t)(m23 >> 32), one);
 #pragma unroll
                     for (int pl = 0; pl < kPlanes; ++pl) acc[j] = mfma16(a[pl], b, acc[j], kBf);
                 }
