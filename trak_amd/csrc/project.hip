@@ -19,10 +19,12 @@
 // in bits 15/31 of (word_v << q), v = 0..3, of ONE Philox block per column per
 // chunk, and the A operand is 16 contiguous bytes of a gradient row.
 //
-// Partial sums of every feature tile go to a workspace [T, B, k] that a second
-// kernel adds up in tile order, so results do not depend on scheduling.
+// A workgroup walks a group of consecutive feature tiles (adding them up in its
+// accumulators) and writes one partial [B, 512] block; a second kernel adds the
+// groups up in order, so results do not depend on scheduling.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+#include <stdlib.h>
 
 #include "jl_stream.h"
 #include "trakhip_internal.h"
@@ -201,14 +203,6 @@ __device__ __forceinline__ uint32_t sign_pair(uint32_t m, uint32_t one) {
     return __builtin_amdgcn_bitop3_b32(m, one, one | 0x80008000u, 0xCA);
 }
 
-// Both words of a pair shifted left by q with one full-rate v_lshlrev_b64.  Bits that cross
-// from the low into the high word land below bit 15 (q <= 15) where sign_pair ignores them.
-__device__ __forceinline__ uint64_t shl_pair(uint64_t v, uint32_t q) {
-    uint64_t r;
-    asm("v_lshlrev_b64 %0, %1, %2" : "=v"(r) : "s"(q), "v"(v));
-    return r;
-}
-
 __device__ __forceinline__ uint32_t pack_f16(float a, float b) {
     return (uint32_t)jl::f32_to_f16_rne(a) | ((uint32_t)jl::f32_to_f16_rne(b) << 16);
 }
@@ -253,35 +247,52 @@ __device__ __forceinline__ void map_workgroup(uint32_t linear, uint32_t col_bloc
     tile = (idx / col_blocks) * 8u + xcd;
 }
 
+// Rademacher B operand of MFMA number q of the chunk for one column group: the two word pairs
+// shifted left by q, then one v_bitop3 per register.
+__device__ __forceinline__ uint4 rademacher_operand(uint64_t w01, uint64_t w23, int q, uint32_t one) {
+    // one full-rate v_lshlrev_b64 per pair (the compiler would split a plain 64-bit shift into
+    // two 32-bit ones); bits crossing into the high word stay below bit 15, which sign_pair ignores
+    uint64_t m01 = w01, m23 = w23;
+    if (q) {
+        asm("v_lshlrev_b64 %0, %1, %2" : "=v"(m01) : "s"(q), "v"(w01));
+        asm("v_lshlrev_b64 %0, %1, %2" : "=v"(m23) : "s"(q), "v"(w23));
+    }
+    uint4 b;
+    b.x = sign_pair((uint32_t)m01, one);
+    b.y = sign_pair((uint32_t)(m01 >> 32), one);
+    b.z = sign_pair((uint32_t)m23, one);
+    b.w = sign_pair((uint32_t)(m23 >> 32), one);
+    return b;
+}
+
 template <int IN, int PT>
 __global__ __launch_bounds__(kThreads, 2) void jl_project_kernel(
     const void* __restrict__ g_in, uint64_t ld, uint32_t rows, uint64_t P, uint32_t k,
-    uint32_t seed, uint32_t tiles, uint64_t tile_size, float* __restrict__ partial) {
+    uint32_t seed, uint32_t tiles, uint64_t tile_size, uint32_t tiles_per_group,
+    float* __restrict__ partial) {
     typedef InTraits<IN> Tr;
     typedef typename StageOf<IN>::type Stage;
     typedef typename StageOf<IN>::elem Elem;
     constexpr bool kBf = Tr::bf16;
     constexpr int kPlanes = Tr::planes;
+    // 16-bit inputs: two LDS buffers, one barrier per chunk.  fp32 inputs (three planes) keep one
+    // buffer and two barriers so that two workgroups still fit on a CU.
+    constexpr int kBuffers = kPlanes == 1 ? 2 : 1;
+    constexpr int kBufElems = kPlanes * kPlaneElems;
 
-    __shared__ __attribute__((aligned(16))) uint16_t lds[kPlanes * kPlaneElems];
+    __shared__ __attribute__((aligned(16))) uint16_t lds[kBuffers * kBufElems];
 
     const uint32_t col_blocks = k / kColsPerWG;
-    uint32_t cb, tile;
-    map_workgroup(blockIdx.x, col_blocks, cb, tile);
-    if (tile >= tiles) return;  // padding of the tile count to a multiple of 8
+    uint32_t cb, group;
+    map_workgroup(blockIdx.x, col_blocks, cb, group);
+    const uint32_t t0 = group * tiles_per_group;
+    if (t0 >= tiles) return;  // padding of the group count to a multiple of 8
+    const uint32_t t1 = t0 + tiles_per_group < tiles ? t0 + tiles_per_group : tiles;
 
     const int tid = threadIdx.x;
     const int wave = tid >> 6, lane = tid & 63;
     const uint32_t n = lane & 31, h = lane >> 5;
     const uint32_t col0 = cb * kColsPerWG + wave * (kGroups * 32) + n;
-
-    const uint64_t f_lo = (uint64_t)tile * tile_size;
-    const uint64_t f_hi = (f_lo + tile_size < P) ? f_lo + tile_size : P;  // may be <= f_lo
-    const uint32_t chunks = f_hi > f_lo ? (uint32_t)((f_hi - f_lo + kChunk - 1) / kChunk) : 0u;
-
-    uint32_t sseed[kGroups];
-#pragma unroll
-    for (int j = 0; j < kGroups; ++j) sseed[j] = jl::stream_seed(seed, col0 + 32u * j, tile);
 
     floatx16 acc[kGroups];
 #pragma unroll
@@ -290,78 +301,107 @@ __global__ __launch_bounds__(kThreads, 2) void jl_project_kernel(
         for (int r = 0; r < 16; ++r) acc[j][r] = 0.0f;
 
     const Elem* g = reinterpret_cast<const Elem*>(g_in);
-    Stage st;
-    if (chunks) st.load(g, ld, rows, f_lo, f_hi, tid);
-
     const uint32_t one = kBf ? 0x3F803F80u : 0x3C003C00u;
-    const uint16_t* a_base = lds + n * kLdsRow + 128 * h;
+    const uint32_t a_off = n * kLdsRow + 128 * h;
 
-    for (uint32_t s = 0; s < chunks; ++s) {
-        __syncthreads();  // everyone is done reading the previous chunk
+    Stage st;
+    {
+        const uint64_t lo = (uint64_t)t0 * tile_size;
+        const uint64_t hi = (lo + tile_size < P) ? lo + tile_size : P;
+        st.load(g, ld, rows, lo, hi, tid);
+    }
+    int cur = 0;
+    if (kBuffers == 2) {
         st.store(lds, tid);
         __syncthreads();
-        if (s + 1 < chunks) st.load(g, ld, rows, f_lo + (uint64_t)(s + 1) * kChunk, f_hi, tid);
+    }
 
-        if (PT == TRAKHIP_RADEMACHER) {
-            uint64_t w01[kGroups], w23[kGroups];
+    for (uint32_t tile = t0; tile < t1; ++tile) {
+        const uint64_t f_lo = (uint64_t)tile * tile_size;
+        const uint64_t f_hi = (f_lo + tile_size < P) ? f_lo + tile_size : P;  // may be <= f_lo
+        const uint32_t chunks = f_hi > f_lo ? (uint32_t)((f_hi - f_lo + kChunk - 1) / kChunk) : 0u;
+        const uint64_t nf_lo = f_lo + tile_size;                               // next tile
+        const uint64_t nf_hi = (nf_lo + tile_size < P) ? nf_lo + tile_size : P;
+
+        uint32_t sseed[kGroups];
 #pragma unroll
-            for (int j = 0; j < kGroups; ++j) {
-                const jl::u32x4 w = jl::stream_block(sseed[j], 2u * s + h);
-                w01[j] = ((uint64_t)w.y << 32) | w.x;
-                w23[j] = ((uint64_t)w.w << 32) | w.z;
+        for (int j = 0; j < kGroups; ++j) sseed[j] = jl::stream_seed(seed, col0 + 32u * j, tile);
+
+        for (uint32_t s = 0; s < chunks; ++s) {
+            const bool more_here = s + 1 < chunks;
+            const bool more = more_here || tile + 1 < t1;
+            if (kBuffers == 1) {
+                __syncthreads();  // everyone is done reading the previous chunk
+                st.store(lds, tid);
+                __syncthreads();
             }
-#pragma unroll
-            for (int q = 0; q < 16; ++q) {
-                uint4 a[kPlanes];
-#pragma unroll
-                for (int pl = 0; pl < kPlanes; ++pl)
-                    a[pl] = *reinterpret_cast<const uint4*>(a_base + pl * kPlaneElems + 8 * q);
+            if (more)
+                st.load(g, ld, rows, more_here ? f_lo + (uint64_t)(s + 1) * kChunk : nf_lo, more_here ? f_hi : nf_hi,
+                        tid);
+            const uint16_t* a_base = lds + cur * kBufElems + a_off;
+
+            if (PT == TRAKHIP_RADEMACHER) {
+                uint64_t w01[kGroups], w23[kGroups];
 #pragma unroll
                 for (int j = 0; j < kGroups; ++j) {
-                    const uint64_t m01 = q ? shl_pair(w01[j], q) : w01[j];
-                    const uint64_t m23 = q ? shl_pair(w23[j], q) : w23[j];
-                    uint4 b;
-                    b.x = sign_pair((uint32_t)m01, one);
-                    b.y = sign_pair((uint32_t)(m01 >> 32), one);
-                    b.z = sign_pair((uint32_t)m23, one);
-                    b.w = sign_pair((uint32_t)(m23 >> 32), one);
-#pragma unroll
-                    for (int pl = 0; pl < kPlanes; ++pl) acc[j] = mfma16(a[pl], b, acc[j], kBf);
+                    const jl::u32x4 w = jl::stream_block(sseed[j], 2u * s + h);
+                    w01[j] = ((uint64_t)w.y << 32) | w.x;
+                    w23[j] = ((uint64_t)w.w << 32) | w.z;
                 }
-            }
-        } else {
-            const uint32_t o_chunk = s * (uint32_t)kChunk + 128u * h;
+#pragma unroll
+                for (int q = 0; q < 16; ++q) {
+                    uint4 a[kPlanes];
+#pragma unroll
+                    for (int pl = 0; pl < kPlanes; ++pl)
+                        a[pl] = *reinterpret_cast<const uint4*>(a_base + pl * kPlaneElems + 8 * q);
+#pragma unroll
+                    for (int j = 0; j < kGroups; ++j) {
+                        const uint4 b = rademacher_operand(w01[j], w23[j], q, one);
+#pragma unroll
+                        for (int pl = 0; pl < kPlanes; ++pl) acc[j] = mfma16(a[pl], b, acc[j], kBf);
+                    }
+                }
+            } else {
+                const uint32_t o_chunk = s * (uint32_t)kChunk + 128u * h;
 #pragma unroll 1
-            for (int q = 0; q < 16; ++q) {
-                uint4 a[kPlanes];
+                for (int q = 0; q < 16; ++q) {
+                    uint4 a[kPlanes];
 #pragma unroll
-                for (int pl = 0; pl < kPlanes; ++pl)
-                    a[pl] = *reinterpret_cast<const uint4*>(a_base + pl * kPlaneElems + 8 * q);
+                    for (int pl = 0; pl < kPlanes; ++pl)
+                        a[pl] = *reinterpret_cast<const uint4*>(a_base + pl * kPlaneElems + 8 * q);
 #pragma unroll
-                for (int j = 0; j < kGroups; ++j) {
-                    const uint4 bh = normal_oct_f16(sseed[j], o_chunk + 8u * q);
-                    if (!kBf) {
-                        acc[j] = mfma16(a[0], bh, acc[j], false);
-                    } else {
-                        uint4 hi, lo;
-                        f16pair_to_bf16_terms(bh.x, hi.x, lo.x);
-                        f16pair_to_bf16_terms(bh.y, hi.y, lo.y);
-                        f16pair_to_bf16_terms(bh.z, hi.z, lo.z);
-                        f16pair_to_bf16_terms(bh.w, hi.w, lo.w);
+                    for (int j = 0; j < kGroups; ++j) {
+                        const uint4 bh = normal_oct_f16(sseed[j], o_chunk + 8u * q);
+                        if (!kBf) {
+                            acc[j] = mfma16(a[0], bh, acc[j], false);
+                        } else {
+                            uint4 hi, lo;
+                            f16pair_to_bf16_terms(bh.x, hi.x, lo.x);
+                            f16pair_to_bf16_terms(bh.y, hi.y, lo.y);
+                            f16pair_to_bf16_terms(bh.z, hi.z, lo.z);
+                            f16pair_to_bf16_terms(bh.w, hi.w, lo.w);
 #pragma unroll
-                        for (int pl = 0; pl < kPlanes; ++pl) {
-                            acc[j] = mfma16(a[pl], hi, acc[j], true);
-                            acc[j] = mfma16(a[pl], lo, acc[j], true);
+                            for (int pl = 0; pl < kPlanes; ++pl) {
+                                acc[j] = mfma16(a[pl], hi, acc[j], true);
+                                acc[j] = mfma16(a[pl], lo, acc[j], true);
+                            }
                         }
                     }
                 }
+            }
+
+            if (kBuffers == 2) {
+                // the other buffer was last read in the previous iteration, before its barrier
+                if (more) st.store(lds + (cur ^ 1) * kBufElems, tid);
+                __syncthreads();
+                cur ^= 1;
             }
         }
     }
 
     // D[m][n] of a 32x32 MFMA: lane holds column n = lane % 32 and, in register r, row
     // m = 8*(r/4) + 4*(lane/32) + r%4.
-    float* out = partial + (uint64_t)tile * rows * k;
+    float* out = partial + (uint64_t)group * rows * k;
 #pragma unroll
     for (int j = 0; j < kGroups; ++j) {
 #pragma unroll
@@ -372,7 +412,7 @@ __global__ __launch_bounds__(kThreads, 2) void jl_project_kernel(
     }
 }
 
-// out[b, c] = sum over tiles, in tile order.
+// out[b, c] = scale * sum over tile groups, in group order.
 __global__ __launch_bounds__(256) void jl_reduce_kernel(const float* __restrict__ partial,
                                                         uint32_t tiles, uint64_t n4, float scale,
                                                         float* __restrict__ out) {
@@ -409,15 +449,28 @@ __global__ __launch_bounds__(256) void jl_materialize_kernel(uint32_t seed, uint
     out[idx] = proj_type == TRAKHIP_RADEMACHER ? jl::entry_rademacher(ss, o) : jl::entry_normal(ss, o);
 }
 
+// Feature tiles handled by one workgroup (their partial sums are added in registers).  Chosen
+// so that the launch has about two workgroups per compute unit; depends only on the shape.
+__host__ uint32_t tiles_per_group(uint32_t tiles, uint32_t col_blocks) {
+    uint64_t target_wgs = 512;  // 256 CUs x 2 resident workgroups
+    if (const char* e = getenv("TRAKHIP_TARGET_WGS")) target_wgs = strtoull(e, nullptr, 10);
+    uint64_t tpg = ((uint64_t)tiles * col_blocks + target_wgs - 1) / target_wgs;
+    if (tpg < 1) tpg = 1;
+    if (tpg > tiles) tpg = tiles;
+    return (uint32_t)tpg;
+}
+
 template <int IN, int PT>
 hipError_t launch_one(const void* in, uint64_t ld, uint32_t rows, uint64_t P, uint32_t k,
                       uint32_t seed, const jl::Tiling& tl, float* partial, hipStream_t s) {
     const uint32_t col_blocks = k / kColsPerWG;
-    const uint32_t tiles8 = (tl.tiles + 7u) / 8u * 8u;
-    const uint64_t wgs = (uint64_t)tiles8 * col_blocks;
+    const uint32_t tpg = tiles_per_group(tl.tiles, col_blocks);
+    const uint32_t groups = (tl.tiles + tpg - 1) / tpg;
+    const uint32_t groups8 = (groups + 7u) / 8u * 8u;
+    const uint64_t wgs = (uint64_t)groups8 * col_blocks;
     if (wgs > 0x7FFFFFFFull) return hipErrorInvalidValue;
     hipLaunchKernelGGL((jl_project_kernel<IN, PT>), dim3((uint32_t)wgs), dim3(kThreads), 0, s, in, ld,
-                       rows, P, k, seed, tl.tiles, tl.tile_size, partial);
+                       rows, P, k, seed, tl.tiles, tl.tile_size, tpg, partial);
     return hipGetLastError();
 }
 
@@ -476,9 +529,11 @@ int project_reduce(const void* ws, uint64_t B, uint64_t P, uint32_t k, uint32_t 
     if (!ws || !out) return TRAKHIP_ERR_NULL;
     if ((reinterpret_cast<uintptr_t>(ws) % 16) || (reinterpret_cast<uintptr_t>(out) % 16)) return TRAKHIP_ERR_ALIGN;
     const jl::Tiling tl = jl::make_tiling(P, num_feature_tiles);
+    const uint32_t tpg = tiles_per_group(tl.tiles, k / kColsPerWG);
+    const uint32_t groups = (tl.tiles + tpg - 1) / tpg;
     const uint64_t n4 = B * k / 4;
     hipLaunchKernelGGL(jl_reduce_kernel, dim3((uint32_t)((n4 + 255) / 256)), dim3(256), 0, s,
-                       static_cast<const float*>(ws), tl.tiles, n4, scale, out);
+                       static_cast<const float*>(ws), groups, n4, scale, out);
     return hipGetLastError() == hipSuccess ? TRAKHIP_OK : TRAKHIP_ERR_LAUNCH;
 }
 
