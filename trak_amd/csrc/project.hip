@@ -247,16 +247,24 @@ __device__ __forceinline__ void map_workgroup(uint32_t linear, uint32_t col_bloc
     tile = (idx / col_blocks) * 8u + xcd;
 }
 
-// Rademacher B operand of MFMA number q of the chunk for one column group: the two word pairs
-// shifted left by q, then one v_bitop3 per register.
-__device__ __forceinline__ uint4 rademacher_operand(uint64_t w01, uint64_t w23, int q, uint32_t one) {
-    // one full-rate v_lshlrev_b64 per pair (the compiler would split a plain 64-bit shift into
-    // two 32-bit ones); bits crossing into the high word stay below bit 15, which sign_pair ignores
-    uint64_t m01 = w01, m23 = w23;
+// Rademacher B operand of MFMA number q of the chunk for one column group, in two halves so the
+// caller can put the MFMA of the previous step between them:
+//   shifted_pairs: both word pairs shifted left by q, one full-rate v_lshlrev_b64 each (for a
+//     constant count the compiler would emit two 32-bit instructions per pair); bits crossing into
+//     the high word stay below bit 15, which sign_pair ignores;
+//   signs_of: one v_bitop3 per operand register.
+__device__ __forceinline__ void shifted_pairs(uint64_t w01, uint64_t w23, int q, uint64_t& m01, uint64_t& m23) {
+    m01 = w01;
+    m23 = w23;
     if (q) {
-        asm("v_lshlrev_b64 %0, %1, %2" : "=v"(m01) : "s"(q), "v"(w01));
-        asm("v_lshlrev_b64 %0, %1, %2" : "=v"(m23) : "s"(q), "v"(w23));
+        // a shift count the compiler cannot see through keeps the 64-bit shift one instruction
+        int qq = q;
+        asm("" : "+s"(qq));
+        m01 = w01 << qq;
+        m23 = w23 << qq;
     }
+}
+__device__ __forceinline__ uint4 signs_of(uint64_t m01, uint64_t m23, uint32_t one) {
     uint4 b;
     b.x = sign_pair((uint32_t)m01, one);
     b.y = sign_pair((uint32_t)(m01 >> 32), one);
@@ -348,17 +356,36 @@ __global__ __launch_bounds__(kThreads, 2) void jl_project_kernel(
                     w01[j] = ((uint64_t)w.y << 32) | w.x;
                     w23[j] = ((uint64_t)w.w << 32) | w.z;
                 }
+                // 64 steps (q, j).  Issue order per step: shifts of the NEXT operand, MFMA of this
+                // step, sign expansion of the next operand.  The MFMA then never directly follows
+                // the VALU instructions that wrote its operand (no wait states to pad).
+                uint64_t m01, m23;
+                shifted_pairs(w01[0], w23[0], 0, m01, m23);
+                uint4 b = signs_of(m01, m23, one);
+                uint4 a[2][kPlanes];  // A operands of this q and of the next one (read one q ahead)
+#pragma unroll
+                for (int pl = 0; pl < kPlanes; ++pl)
+                    a[0][pl] = *reinterpret_cast<const uint4*>(a_base + pl * kPlaneElems);
 #pragma unroll
                 for (int q = 0; q < 16; ++q) {
-                    uint4 a[kPlanes];
-#pragma unroll
-                    for (int pl = 0; pl < kPlanes; ++pl)
-                        a[pl] = *reinterpret_cast<const uint4*>(a_base + pl * kPlaneElems + 8 * q);
 #pragma unroll
                     for (int j = 0; j < kGroups; ++j) {
-                        const uint4 b = rademacher_operand(w01[j], w23[j], q, one);
+                        const int step = q * kGroups + j;
+                        const bool last = step + 1 == 16 * kGroups;
+                        if (!last) shifted_pairs(w01[(step + 1) % kGroups], w23[(step + 1) % kGroups],
+                                                 (step + 1) / kGroups, m01, m23);
+                        if (j == 0 && q + 1 < 16) {
 #pragma unroll
-                        for (int pl = 0; pl < kPlanes; ++pl) acc[j] = mfma16(a[pl], b, acc[j], kBf);
+                            for (int pl = 0; pl < kPlanes; ++pl)
+                                a[(q + 1) & 1][pl] =
+                                    *reinterpret_cast<const uint4*>(a_base + pl * kPlaneElems + 8 * (q + 1));
+                        }
+                        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                        for (int pl = 0; pl < kPlanes; ++pl) acc[j] = mfma16(a[q & 1][pl], b, acc[j], kBf);
+                        __builtin_amdgcn_sched_barrier(0);
+                        if (!last) b = signs_of(m01, m23, one);
+                        __builtin_amdgcn_sched_barrier(0);
                     }
                 }
             } else {
