@@ -24,7 +24,6 @@
 // groups up in order, so results do not depend on scheduling.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
-#include <stdlib.h>
 
 #include "jl_stream.h"
 #include "trakhip_internal.h"
@@ -441,24 +440,49 @@ __global__ __launch_bounds__(kThreads, 2) void jl_project_kernel(
 
 // out[b, c] = scale * sum over tile groups, in group order.
 __global__ __launch_bounds__(256) void jl_reduce_kernel(const float* __restrict__ partial,
-                                                        uint32_t tiles, uint64_t n4, float scale,
+                                                        uint32_t groups, uint64_t n4, float scale,
                                                         float* __restrict__ out) {
     const uint64_t i = (uint64_t)blockIdx.x * 256 + threadIdx.x;
     if (i >= n4) return;
     const float4* p = reinterpret_cast<const float4*>(partial) + i;
-    float4 s = {0.f, 0.f, 0.f, 0.f};
-    for (uint32_t t = 0; t < tiles; ++t) {
-        const float4 v = p[(uint64_t)t * n4];
-        s.x += v.x;
-        s.y += v.y;
-        s.z += v.z;
-        s.w += v.w;
+    // eight running sums over groups g = u (mod 8) keep eight loads in flight; they are combined
+    // in a fixed order, so the result depends only on the shape
+    float4 s[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) s[u] = {0.f, 0.f, 0.f, 0.f};
+    uint32_t g = 0;
+    for (; g + 8 <= groups; g += 8) {
+        float4 v[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) v[u] = p[(uint64_t)(g + u) * n4];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            s[u].x += v[u].x;
+            s[u].y += v[u].y;
+            s[u].z += v[u].z;
+            s[u].w += v[u].w;
+        }
     }
-    s.x *= scale;
-    s.y *= scale;
-    s.z *= scale;
-    s.w *= scale;
-    reinterpret_cast<float4*>(out)[i] = s;
+#pragma unroll
+    for (int u = 0; u < 7; ++u) {
+        if (g + u < groups) {
+            const float4 v = p[(uint64_t)(g + u) * n4];
+            s[u].x += v.x;
+            s[u].y += v.y;
+            s[u].z += v.z;
+            s[u].w += v.w;
+        }
+    }
+    float4 r;
+    r.x = ((s[0].x + s[1].x) + (s[2].x + s[3].x)) + ((s[4].x + s[5].x) + (s[6].x + s[7].x));
+    r.y = ((s[0].y + s[1].y) + (s[2].y + s[3].y)) + ((s[4].y + s[5].y) + (s[6].y + s[7].y));
+    r.z = ((s[0].z + s[1].z) + (s[2].z + s[3].z)) + ((s[4].z + s[5].z) + (s[6].z + s[7].z));
+    r.w = ((s[0].w + s[1].w) + (s[2].w + s[3].w)) + ((s[4].w + s[5].w) + (s[6].w + s[7].w));
+    r.x *= scale;
+    r.y *= scale;
+    r.z *= scale;
+    r.w *= scale;
+    reinterpret_cast<float4*>(out)[i] = r;
 }
 
 // S[f0 + i, c0 + j] for i < nf, j < nc, written as binary32, row-major [nf, nc].
@@ -479,8 +503,7 @@ __global__ __launch_bounds__(256) void jl_materialize_kernel(uint32_t seed, uint
 // Feature tiles handled by one workgroup (their partial sums are added in registers).  Chosen
 // so that the launch has about two workgroups per compute unit; depends only on the shape.
 __host__ uint32_t tiles_per_group(uint32_t tiles, uint32_t col_blocks) {
-    uint64_t target_wgs = 512;  // 256 CUs x 2 resident workgroups
-    if (const char* e = getenv("TRAKHIP_TARGET_WGS")) target_wgs = strtoull(e, nullptr, 10);
+    const uint64_t target_wgs = 512;  // 256 CUs x 2 resident workgroups
     uint64_t tpg = ((uint64_t)tiles * col_blocks + target_wgs - 1) / target_wgs;
     if (tpg < 1) tpg = 1;
     if (tpg > tiles) tpg = tiles;
