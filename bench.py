@@ -27,6 +27,10 @@ sys.path.insert(0, ROOT)
 
 PEAK_FP16_TFLOPS = 2500.0   # MI355X dense fp16/bf16 MFMA
 PEAK_FP32_TFLOPS = 157.3    # MI355X fp32 MFMA
+# HBM bytes of one projection-kernel launch at the benchmark shape, from rocprofv3 --pmc FETCH_SIZE and
+# WRITE_SIZE (profiles/jl_project_f16_rademacher_resnet18_hbm_counters.txt): 365528 KiB x 2.0 (the factor
+# a 1 GiB copy needs for the same counter) fetched + 32768 KiB x 1.0 written.
+PROJECT_KERNEL_HBM_BYTES = (365528 * 2.0 + 32768 * 1.0) * 1024
 METRIC = "JL proj TFLOP/s & % MFMA peak at P=11.7M,k=4096,B=32; scoring TFLOP/s"
 
 
@@ -202,8 +206,8 @@ def cpu_baseline(torch):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--steps", type=int, default=30)
+    ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--batches", type=int, default=16, help="distinct resident batches cycled through")
     ap.add_argument("--no-scoring", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
@@ -259,7 +263,8 @@ def main():
             "peak": PEAK_FP16_TFLOPS,
             "unit": "TFLOP/s",
             "frac": round(proj["kernel_tflops"] / PEAK_FP16_TFLOPS, 4),
-            "traffic": None,
+            "traffic": PROJECT_KERNEL_HBM_BYTES,
+            "traffic_unit": "bytes per launch (algorithmic input+output: %d)" % (32 * 11_689_512 * 2 + 32 * 4096 * 4),
             "kernel": "jl_project_kernel<f16, rademacher>",
             "kernel_ms_avg": round(proj["kernel_ms_avg"], 4),
             "kernel_ms_min": round(proj["kernel_ms_min"], 4),
