@@ -128,6 +128,53 @@ def bench_projection(torch, dev, steps, warmup, n_batches):
     }
 
 
+def bench_other_configs(torch, dev):
+    """Throughput of the other projection configurations of BASELINE.json (not part of the default
+    line; `--all-configs` prints them to stderr for the design notes)."""
+    from trak_amd import ChunkedCudaProjector, CudaProjector, ProjectionType
+
+    res = {}
+
+    def timed(fn, reps):
+        fn()
+        torch.cuda.synchronize()
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        for _ in range(reps):
+            fn()
+        b.record()
+        torch.cuda.synchronize()
+        return a.elapsed_time(b) / reps
+
+    gen = torch.Generator(device=dev).manual_seed(20_001)
+    g1 = torch.randn(16, 1_048_576, generator=gen, device=dev) * 1e-3
+    p1 = CudaProjector(1_048_576, 512, 42, ProjectionType.rademacher, dev, 32)
+    ms = timed(lambda: p1.project(g1, 0), 50)
+    res["c1_fp32_rademacher_[16,1048576]_k512"] = {"ms": ms, "tflops": 2.0 * 16 * 1_048_576 * 512 / ms / 1e9}
+
+    g2 = (torch.randn(32, 4_825_610, generator=gen, device=dev) * 5e-4).half()
+    g2[torch.rand(32, 4_825_610, generator=gen, device=dev) < 0.01] = 0
+    p2 = CudaProjector(4_825_610, 2048, 0, ProjectionType.rademacher, dev, 32)
+    ms = timed(lambda: p2.project(g2, 0), 30)
+    res["c2_fp16_rademacher_[32,4825610]_k2048"] = {"ms": ms, "tflops": 2.0 * 32 * 4_825_610 * 2048 / ms / 1e9}
+    del g1, g2
+
+    import numpy as np
+
+    chunk = 27_370_560
+    seeds = np.random.default_rng(123).integers(0, 500, size=4)
+    grads = {i: (torch.randn(32, chunk, generator=gen, device=dev) * 1e-4).bfloat16() for i in range(4)}
+    per = [CudaProjector(chunk, 4096, int(seeds[i]), ProjectionType.normal, dev, 32) for i in range(4)]
+    p4 = ChunkedCudaProjector(per, chunk, [chunk] * 4, 32, dev, torch.bfloat16)
+    ms = timed(lambda: p4.project(grads, 0), 2)
+    res["c4_bf16_normal_chunked_[32,109482240]_k4096"] = {"ms": ms, "tflops": 2.0 * 32 * 4 * chunk * 4096 / ms / 1e9}
+    per_r = [CudaProjector(chunk, 4096, int(seeds[i]), ProjectionType.rademacher, dev, 32) for i in range(4)]
+    p4r = ChunkedCudaProjector(per_r, chunk, [chunk] * 4, 32, dev, torch.bfloat16)
+    ms = timed(lambda: p4r.project(grads, 0), 5)
+    res["c4_shape_bf16_rademacher_chunked"] = {"ms": ms, "tflops": 2.0 * 32 * 4 * chunk * 4096 / ms / 1e9}
+    return res
+
+
 def bench_scoring(torch, dev, reps=3):
     from trak_amd import BasicScoreComputer
 
@@ -211,6 +258,8 @@ def main():
     ap.add_argument("--batches", type=int, default=16, help="distinct resident batches cycled through")
     ap.add_argument("--no-scoring", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--all-configs", action="store_true",
+                    help="also time the other projection configurations and print them to stderr")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run one 1 GiB device-to-device copy (reference point for rocprofv3 byte counters)")
     args = ap.parse_args()
@@ -233,6 +282,9 @@ def main():
         del src, dst
     proj = bench_projection(torch, dev, args.steps, args.warmup, args.batches)
     torch.cuda.empty_cache()
+    if args.all_configs:
+        print(json.dumps(bench_other_configs(torch, dev), indent=1), file=sys.stderr)
+        torch.cuda.empty_cache()
     scoring = None if args.no_scoring else bench_scoring(torch, dev)
     torch.cuda.empty_cache()
     cpu = None if args.no_cpu else cpu_baseline(torch)

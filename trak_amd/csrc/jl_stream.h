@@ -206,8 +206,16 @@ JL_HD void bm_pair(uint32_t wa, uint32_t wb, float* z0, float* z1) {
     *z1 = JL_MUL(r, s);
 }
 
-// binary32 -> binary16 bit pattern, round to nearest even (|v| < 65504 here, no NaN).
+// binary32 -> binary16 bit pattern, round to nearest even (|v| < 65504 here, no NaN).  On the
+// device this is the hardware conversion (v_cvt_f16_f32, IEEE round-to-nearest-even with
+// subnormals); the host spells the same rounding out in integer arithmetic.
 JL_HD uint16_t f32_to_f16_rne(float v) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    // the empty asm keeps the binary32 value a separate, already rounded operand: without it the
+    // compiler folds a preceding multiply into a mixed-precision FMA that rounds only once
+    asm("" : "+v"(v));
+    return __builtin_bit_cast(uint16_t, (_Float16)v);
+#else
     const uint32_t b = f2u(v);
     const uint32_t sign = (b >> 16) & 0x8000u;
     const uint32_t a = b & 0x7FFFFFFFu;
@@ -227,9 +235,13 @@ JL_HD uint16_t f32_to_f16_rne(float v) {
     r >>= 13;
     if (rem > 0x1000u || (rem == 0x1000u && (r & 1u))) r += 1u;
     return (uint16_t)(sign | r);
+#endif
 }
 
 JL_HD float f16_bits_to_f32(uint16_t hbits) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    return (float)__builtin_bit_cast(_Float16, hbits);  // exact
+#else
     const uint32_t sign = ((uint32_t)hbits & 0x8000u) << 16;
     const uint32_t e = (hbits >> 10) & 0x1Fu;
     const uint32_t m = hbits & 0x3FFu;
@@ -239,6 +251,7 @@ JL_HD float f16_bits_to_f32(uint16_t hbits) {
         return u2f(f2u(v) | sign);
     }
     return u2f(sign | ((e + 112u) << 23) | (m << 13));
+#endif
 }
 
 // ---- entry of the matrix --------------------------------------------------------------------
