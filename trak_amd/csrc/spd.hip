@@ -42,63 +42,136 @@ __global__ __launch_bounds__(256) void spd_init_kernel(const float* __restrict__
     Li[idx] = 0.0f;
 }
 
-// One workgroup: Cholesky of the 128x128 diagonal block at W (lower triangle used), L block to
-// Lout (upper part zero), its inverse to Linv_out.
-__global__ __launch_bounds__(256) void spd_diag_kernel(const float* __restrict__ W, uint64_t ldw,
-                                                       float* __restrict__ Lout, float* __restrict__ Linv_out,
-                                                       uint64_t ldl, int32_t block_index,
-                                                       int32_t* __restrict__ status) {
-    __shared__ float Ls[NB * kLd];
-    __shared__ float Xs[NB * kLd];
+// One workgroup of 1024 threads: Cholesky of the 128x128 diagonal block at W (lower triangle
+// used), L block to Lout (upper part zero), its inverse to Linv_out.
+//
+// Thread (ty, tx) of a 32 x 32 grid keeps the elements (ty + 32 i, tx + 32 j), i, j < 4, of the
+// block in registers (cyclic ownership keeps every thread busy as the active part shrinks; four
+// waves per SIMD hide the issue latency of this strictly sequential algorithm).  Step k of the
+// right-looking factorization broadcasts column k of L through LDS and applies the rank-1 update
+// A -= l l^T from registers; the inverse runs the same way on B = I:
+// X[k, :] = B[k, :] / L[k, k], then B[r, :] -= L[r, k] X[k, :] for r > k.
+constexpr int kDiagGrid = 32;              // threads per side
+constexpr int kDiagTile = NB / kDiagGrid;  // 4 elements per side per thread
+
+__global__ __launch_bounds__(1024) void spd_diag_kernel(const float* __restrict__ W, uint64_t ldw,
+                                                        float* __restrict__ Lout, float* __restrict__ Linv_out,
+                                                        uint64_t ldl, int32_t block_index,
+                                                        int32_t* __restrict__ status) {
+    constexpr int G = kDiagGrid, T = kDiagTile;
+    __shared__ float Ls[NB * kLd];   // the finished factor, column k valid after step k
+    __shared__ float vec[2][NB];     // broadcast buffers (two, so the steps can overlap safely)
+    __shared__ float pivot[2];
     const int tid = threadIdx.x;
+    const int ty = tid / G, tx = tid % G;
 
-    for (int e = tid; e < NB * NB; e += 256) {
-        const int i = e / NB, j = e % NB;
-        Ls[i * kLd + j] = (j <= i) ? W[(uint64_t)i * ldw + j] : 0.0f;
-        Xs[i * kLd + j] = 0.0f;
-    }
-    __syncthreads();
+    float a[T][T];
+#pragma unroll
+    for (int i = 0; i < T; ++i)
+#pragma unroll
+        for (int j = 0; j < T; ++j) {
+            const int r = ty + G * i, c = tx + G * j;
+            a[i][j] = (c <= r) ? W[(uint64_t)r * ldw + c] : 0.0f;
+        }
 
-    const int row = tid & (NB - 1), cpar = tid >> 7;  // row handled in the trailing update, column parity
-    for (int j = 0; j < NB; ++j) {
-        __syncthreads();  // the trailing update of the previous column is complete
-        float d = Ls[j * kLd + j];
-        if (!(d > 0.0f)) {
-            if (tid == 0 && status) {
-                if (*status == 0) *status = 1 + block_index * NB + j;
+    // ---- factorization -------------------------------------------------------------------
+    for (int k = 0; k < NB; ++k) {
+        const int buf = k & 1;
+        const int ki = k / G, kt = k % G;  // element (k, k) lives in thread (kt, kt), slot [ki][ki]
+        if (ty == kt && tx == kt) {
+            float d = 0.0f;
+#pragma unroll
+            for (int i = 0; i < T; ++i)
+                if (i == ki) d = a[i][i];
+            if (!(d > 0.0f)) {
+                if (status && *status == 0) *status = 1 + block_index * NB + k;
+                d = 1.0f;
             }
-            d = 1.0f;
+            pivot[buf] = sqrtf(d);
         }
-        const float sd = sqrtf(d);
-        const float inv_sd = 1.0f / sd;
-        __syncthreads();  // every thread has read the pivot
-        if (tid == 0) Ls[j * kLd + j] = sd;
-        if (tid > j && tid < NB) Ls[tid * kLd + j] *= inv_sd;
         __syncthreads();
-        if (row > j) {
-            const float lij = Ls[row * kLd + j];
-            for (int c = j + 1 + cpar; c <= row; c += 2) Ls[row * kLd + c] -= lij * Ls[c * kLd + j];
+        const float sd = pivot[buf];
+        if (tx == kt) {  // owners of column k: scale and publish it
+            const float inv_sd = 1.0f / sd;
+#pragma unroll
+            for (int i = 0; i < T; ++i) {
+                const int r = ty + G * i;
+                float v = 0.0f;
+#pragma unroll
+                for (int j = 0; j < T; ++j)
+                    if (j == ki) v = a[i][j];
+                const float l = (r > k) ? v * inv_sd : (r == k ? sd : 0.0f);
+                vec[buf][r] = l;
+                Ls[r * kLd + k] = l;
+            }
         }
+        __syncthreads();
+        float lr[T], lc[T];
+#pragma unroll
+        for (int i = 0; i < T; ++i) {
+            const int r = ty + G * i;
+            lr[i] = (r > k) ? vec[buf][r] : 0.0f;
+        }
+#pragma unroll
+        for (int j = 0; j < T; ++j) {
+            const int c = tx + G * j;
+            lc[j] = (c > k) ? vec[buf][c] : 0.0f;
+        }
+#pragma unroll
+        for (int i = 0; i < T; ++i)
+#pragma unroll
+            for (int j = 0; j < T; ++j) a[i][j] -= lr[i] * lc[j];
     }
     __syncthreads();
 
-    // X = L^-1, one column per thread: forward substitution of the unit vectors.
-    if (tid < NB) {
-        const int c = tid;
-        Xs[c * kLd + c] = 1.0f / Ls[c * kLd + c];
-        for (int i = c + 1; i < NB; ++i) {
-            float sum = 0.0f;
-            for (int m = c; m < i; ++m) sum += Ls[i * kLd + m] * Xs[m * kLd + c];
-            Xs[i * kLd + c] = -sum / Ls[i * kLd + i];
-        }
-    }
-    __syncthreads();
+    // ---- inverse of L ---------------------------------------------------------------------
+    float b[T][T];
+#pragma unroll
+    for (int i = 0; i < T; ++i)
+#pragma unroll
+        for (int j = 0; j < T; ++j) b[i][j] = (ty + G * i == tx + G * j) ? 1.0f : 0.0f;
 
-    for (int e = tid; e < NB * NB; e += 256) {
-        const int i = e / NB, j = e % NB;
-        Lout[(uint64_t)i * ldl + j] = Ls[i * kLd + j];
-        Linv_out[(uint64_t)i * ldl + j] = Xs[i * kLd + j];
+    for (int k = 0; k < NB; ++k) {
+        const int buf = k & 1;
+        const int ki = k / G, kt = k % G;
+        if (ty == kt) {  // owners of row k: X[k, c] = B[k, c] / L[k, k]
+            const float inv_d = 1.0f / Ls[k * kLd + k];
+#pragma unroll
+            for (int j = 0; j < T; ++j) {
+                float v = 0.0f;
+#pragma unroll
+                for (int i = 0; i < T; ++i)
+                    if (i == ki) v = b[i][j];
+                v *= inv_d;
+#pragma unroll
+                for (int i = 0; i < T; ++i)
+                    if (i == ki) b[i][j] = v;
+                vec[buf][tx + G * j] = v;
+            }
+        }
+        __syncthreads();
+        float lr[T], xc[T];
+#pragma unroll
+        for (int i = 0; i < T; ++i) {
+            const int r = ty + G * i;
+            lr[i] = (r > k) ? Ls[r * kLd + k] : 0.0f;
+        }
+#pragma unroll
+        for (int j = 0; j < T; ++j) xc[j] = vec[buf][tx + G * j];
+#pragma unroll
+        for (int i = 0; i < T; ++i)
+#pragma unroll
+            for (int j = 0; j < T; ++j) b[i][j] -= lr[i] * xc[j];
     }
+
+#pragma unroll
+    for (int i = 0; i < T; ++i)
+#pragma unroll
+        for (int j = 0; j < T; ++j) {
+            const int r = ty + G * i, c = tx + G * j;
+            Lout[(uint64_t)r * ldl + c] = (c <= r) ? Ls[r * kLd + c] : 0.0f;
+            Linv_out[(uint64_t)r * ldl + c] = (c <= r) ? b[i][j] : 0.0f;
+        }
 }
 
 __global__ __launch_bounds__(256) void abs_sum_kernel(const float* __restrict__ M, uint64_t ld, uint64_t n,
@@ -204,7 +277,7 @@ int spd_inverse(const float* A, uint64_t lda, float lambda, float* inv, uint64_t
 
     for (uint64_t j = 0; j < nblk; ++j) {
         const uint64_t off = j * NB * np + j * NB;
-        hipLaunchKernelGGL(spd_diag_kernel, dim3(1), dim3(256), 0, s, W + off, np, L + off, Li + off, np,
+        hipLaunchKernelGGL(spd_diag_kernel, dim3(1), dim3(1024), 0, s, W + off, np, L + off, Li + off, np,
                            (int32_t)j, status);
         if (hipGetLastError() != hipSuccess) return TRAKHIP_ERR_LAUNCH;
         if (j + 1 == nblk) break;
