@@ -301,3 +301,45 @@ def test_full_size_resnet18_shape(gpu, c_oracle):
         want = c_oracle.project(g32, seed, tiles, c, 1, R)[:, 0]
         got = out[:, c].cpu().numpy().astype(np.float64)
         assert np.linalg.norm(got - want) / np.linalg.norm(want) < 1e-3
+
+
+# ---- the reference's uint32-overflow shapes (tests/test_jl.py:59-73, tests/test_jl_additional.py:11-44) ----
+
+
+@pytest.mark.parametrize("shape", [(8, 180_645_096), (31, 180_645_096), (2, 780_645_096)])
+def test_uint32_overflow_shapes_through_chunks(gpu, c_oracle, shape):
+    # B * P >= 2^31 / 2^32: the reference's kernel indexes with uint32 `row * features`
+    # (fast_jl/data_loading.cuh:37-41) and therefore chunks P; here addressing is 64-bit, and the
+    # chunked path is exercised exactly as the reference's tests do.
+    B, P = shape
+    k, seed, dtype = 15_360, 123, torch.float32
+    max_chunk_size = int(np.iinfo(np.uint32).max // B)
+    num_chunks = int(np.ceil(P / max_chunk_size))
+    g = torch.zeros(B, P, device=gpu, dtype=dtype)
+    g[:, 0] = 1.0
+    g[:, -1] = 2.0
+    g[0, 12_345_678] = 3.0
+    g[-1] = g[0]
+    chunks = {i: x for i, x in enumerate(torch.chunk(g, num_chunks, dim=1))}
+    sizes = [v.size(1) for v in chunks.values()]
+    seeds = np.random.default_rng(seed).integers(low=0, high=500, size=len(chunks))
+    per_chunk = [_projector(sz, k, int(seeds[i]), ProjectionType.rademacher, dtype) for i, sz in enumerate(sizes)]
+    proj = ChunkedCudaProjector(per_chunk, max_chunk_size, sizes, B, "cuda:0", dtype)
+    p = proj.project(chunks, model_id=0)
+    assert p.shape == (B, k)
+    assert torch.equal(p, proj.project(chunks, model_id=0))                  # seed consistency
+    assert torch.equal(p[0], p[-1])                                          # same rows, same features
+    # exact expectation from the oracle: row b = 1*S0[0,:] + 2*S_last[last,:] (+ 3*S[f,:] for rows 0 and B-1)
+    tiles = per_chunk[0].num_sms
+    first = c_oracle.materialize(int(seeds[0]), tiles, sizes[0], 0, 1, 0, k, R)[0]
+    last = c_oracle.materialize(int(seeds[-1]), tiles, sizes[-1], sizes[-1] - 1, 1, 0, k, R)[0]
+    ci, off = divmod(12_345_678, sizes[0]) if sizes[0] * (len(sizes) - 1) > 12_345_678 else (0, 12_345_678)
+    mid = c_oracle.materialize(int(seeds[ci]), tiles, sizes[ci], off, 1, 0, k, R)[0]
+    want_plain = first + 2.0 * last
+    got = p.cpu().numpy()
+    if B > 2:
+        assert np.array_equal(got[1], want_plain)
+    assert np.array_equal(got[0], want_plain + 3.0 * mid)
+    proj.free_memory()
+    del g, chunks
+    torch.cuda.empty_cache()
