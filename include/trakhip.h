@@ -67,10 +67,10 @@ int trakhip_project(const void* in_dev, int in_dtype, uint64_t B, uint64_t P, ui
                     float* out_dev, void* workspace_dev, size_t workspace_bytes, uint32_t proj_dim,
                     uint32_t seed, uint32_t num_feature_tiles, int proj_type, void* stream);
 
-/* The two phases of trakhip_project as separate calls, for B <= 32 rows: phase 1 writes the
- * per-feature-tile partial sums [T, B, proj_dim] (T = min(P, num_feature_tiles)) to the workspace
- * (the kernel of fast_jl/fast_jl_kernel.cuh:24-105 writing `output[row][tile][col]`), phase 2 adds
- * them up in tile order into out_dev (the `.sum(1)` of fast_jl/fast_jl.cu:78), multiplied by
+/* The two phases of trakhip_project as separate calls, for B <= 32 rows: phase 1 writes partial
+ * sums [G, B, proj_dim] over G runs of consecutive features to the workspace (the kernel of
+ * fast_jl/fast_jl_kernel.cuh:24-105 writing `output[row][tile][col]`; G depends only on the shape),
+ * phase 2 adds them up in order into out_dev (the `.sum(1)` of fast_jl/fast_jl.cu:78), multiplied by
  * `scale` (1.0f for the plain sum; 1/sqrt(P) gives the `grads /= normalize_factor` of
  * trak/traker.py:426 for free).  A caller can time the phases or put its own epilogue between. */
 int trakhip_project_partials(const void* in_dev, int in_dtype, uint64_t B, uint64_t P, uint64_t ld_in,

@@ -19,9 +19,9 @@
 // in bits 15/31 of (word_v << q), v = 0..3, of ONE Philox block per column per
 // chunk, and the A operand is 16 contiguous bytes of a gradient row.
 //
-// A workgroup walks a group of consecutive feature tiles (adding them up in its
-// accumulators) and writes one partial [B, 512] block; a second kernel adds the
-// groups up in order, so results do not depend on scheduling.
+// A workgroup walks a run of consecutive chunks (across tile boundaries, adding the
+// products up in its accumulators) and writes one partial [B, 512] block; a second
+// kernel adds the runs up in order, so results do not depend on scheduling.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
@@ -275,8 +275,8 @@ __device__ __forceinline__ uint4 signs_of(uint64_t m01, uint64_t m23, uint32_t o
 template <int IN, int PT>
 __global__ __launch_bounds__(kThreads, 2) void jl_project_kernel(
     const void* __restrict__ g_in, uint64_t ld, uint32_t rows, uint64_t P, uint32_t k,
-    uint32_t seed, uint32_t tiles, uint64_t tile_size, uint32_t tiles_per_group,
-    float* __restrict__ partial) {
+    uint32_t seed, uint32_t tiles, uint64_t tile_size, uint32_t chunks_per_tile,
+    uint32_t chunks_per_group, float* __restrict__ partial) {
     typedef InTraits<IN> Tr;
     typedef typename StageOf<IN>::type Stage;
     typedef typename StageOf<IN>::elem Elem;
@@ -292,9 +292,15 @@ __global__ __launch_bounds__(kThreads, 2) void jl_project_kernel(
     const uint32_t col_blocks = k / kColsPerWG;
     uint32_t cb, group;
     map_workgroup(blockIdx.x, col_blocks, cb, group);
-    const uint32_t t0 = group * tiles_per_group;
-    if (t0 >= tiles) return;  // padding of the group count to a multiple of 8
-    const uint32_t t1 = t0 + tiles_per_group < tiles ? t0 + tiles_per_group : tiles;
+    // this workgroup's share of the flattened (tile, chunk) sequence; the streams are counter
+    // based, so a workgroup can start in the middle of a tile
+    const uint64_t total_chunks = (uint64_t)tiles * chunks_per_tile;
+    const uint64_t c_begin = (uint64_t)group * chunks_per_group;
+    if (c_begin >= total_chunks) return;  // padding of the group count to a multiple of 8
+    const uint64_t c_end = c_begin + chunks_per_group < total_chunks ? c_begin + chunks_per_group : total_chunks;
+    const uint32_t t0 = (uint32_t)(c_begin / chunks_per_tile), s0 = (uint32_t)(c_begin % chunks_per_tile);
+    const uint32_t t_last = (uint32_t)((c_end - 1) / chunks_per_tile);
+    const uint32_t s_last_end = (uint32_t)((c_end - 1) % chunks_per_tile) + 1;
 
     const int tid = threadIdx.x;
     const int wave = tid >> 6, lane = tid & 63;
@@ -315,7 +321,7 @@ __global__ __launch_bounds__(kThreads, 2) void jl_project_kernel(
     {
         const uint64_t lo = (uint64_t)t0 * tile_size;
         const uint64_t hi = (lo + tile_size < P) ? lo + tile_size : P;
-        st.load(g, ld, rows, lo, hi, tid);
+        st.load(g, ld, rows, lo + (uint64_t)s0 * kChunk, hi, tid);
     }
     int cur = 0;
     if (kBuffers == 2) {
@@ -323,10 +329,11 @@ __global__ __launch_bounds__(kThreads, 2) void jl_project_kernel(
         __syncthreads();
     }
 
-    for (uint32_t tile = t0; tile < t1; ++tile) {
+    for (uint32_t tile = t0; tile <= t_last; ++tile) {
         const uint64_t f_lo = (uint64_t)tile * tile_size;
-        const uint64_t f_hi = (f_lo + tile_size < P) ? f_lo + tile_size : P;  // may be <= f_lo
-        const uint32_t chunks = f_hi > f_lo ? (uint32_t)((f_hi - f_lo + kChunk - 1) / kChunk) : 0u;
+        const uint64_t f_hi = (f_lo + tile_size < P) ? f_lo + tile_size : P;  // may be <= f_lo (loads give zeros)
+        const uint32_t s_begin = tile == t0 ? s0 : 0u;
+        const uint32_t chunks = tile == t_last ? s_last_end : chunks_per_tile;
         const uint64_t nf_lo = f_lo + tile_size;                               // next tile
         const uint64_t nf_hi = (nf_lo + tile_size < P) ? nf_lo + tile_size : P;
 
@@ -334,9 +341,9 @@ __global__ __launch_bounds__(kThreads, 2) void jl_project_kernel(
 #pragma unroll
         for (int j = 0; j < kGroups; ++j) sseed[j] = jl::stream_seed(seed, col0 + 32u * j, tile);
 
-        for (uint32_t s = 0; s < chunks; ++s) {
+        for (uint32_t s = s_begin; s < chunks; ++s) {
             const bool more_here = s + 1 < chunks;
-            const bool more = more_here || tile + 1 < t1;
+            const bool more = more_here || tile < t_last;
             if (kBuffers == 1) {
                 __syncthreads();  // everyone is done reading the previous chunk
                 st.store(lds, tid);
@@ -500,32 +507,44 @@ __global__ __launch_bounds__(256) void jl_materialize_kernel(uint32_t seed, uint
     out[idx] = proj_type == TRAKHIP_RADEMACHER ? jl::entry_rademacher(ss, o) : jl::entry_normal(ss, o);
 }
 
-// Feature tiles handled by one workgroup (their partial sums are added in registers).  Chosen
-// so that the launch has about two workgroups per compute unit; depends only on the shape.
-__host__ uint32_t tiles_per_group(uint32_t tiles, uint32_t col_blocks) {
+// How a launch is cut into workgroups.  The (tile, chunk) pairs of all feature tiles form one
+// sequence of tiles * chunks_per_tile chunks; every workgroup takes chunks_per_group consecutive
+// ones (adding their products in its accumulators) for one block of 512 columns.  The split
+// depends only on the shape, so results are reproducible; it aims at two workgroups per CU.
+struct Plan {
+    jl::Tiling tl;
+    uint32_t col_blocks, chunks_per_tile, chunks_per_group, groups;
+};
+
+Plan make_plan(uint64_t P, uint32_t k, uint32_t num_feature_tiles) {
+    Plan p;
+    p.tl = jl::make_tiling(P, num_feature_tiles);
+    p.col_blocks = k / kColsPerWG;
+    p.chunks_per_tile = (uint32_t)((p.tl.tile_size + kChunk - 1) / kChunk);
+    const uint64_t total = (uint64_t)p.tl.tiles * p.chunks_per_tile;
     const uint64_t target_wgs = 512;  // 256 CUs x 2 resident workgroups
-    uint64_t tpg = ((uint64_t)tiles * col_blocks + target_wgs - 1) / target_wgs;
-    if (tpg < 1) tpg = 1;
-    if (tpg > tiles) tpg = tiles;
-    return (uint32_t)tpg;
+    uint64_t groups = (target_wgs + p.col_blocks - 1) / p.col_blocks;
+    if (groups > total) groups = total;
+    if (groups < 1) groups = 1;
+    p.chunks_per_group = (uint32_t)((total + groups - 1) / groups);
+    p.groups = (uint32_t)((total + p.chunks_per_group - 1) / p.chunks_per_group);
+    return p;
 }
 
 template <int IN, int PT>
 hipError_t launch_one(const void* in, uint64_t ld, uint32_t rows, uint64_t P, uint32_t k,
-                      uint32_t seed, const jl::Tiling& tl, float* partial, hipStream_t s) {
-    const uint32_t col_blocks = k / kColsPerWG;
-    const uint32_t tpg = tiles_per_group(tl.tiles, col_blocks);
-    const uint32_t groups = (tl.tiles + tpg - 1) / tpg;
-    const uint32_t groups8 = (groups + 7u) / 8u * 8u;
-    const uint64_t wgs = (uint64_t)groups8 * col_blocks;
+                      uint32_t seed, const Plan& pl, float* partial, hipStream_t s) {
+    const uint32_t groups8 = (pl.groups + 7u) / 8u * 8u;
+    const uint64_t wgs = (uint64_t)groups8 * pl.col_blocks;
     if (wgs > 0x7FFFFFFFull) return hipErrorInvalidValue;
     hipLaunchKernelGGL((jl_project_kernel<IN, PT>), dim3((uint32_t)wgs), dim3(kThreads), 0, s, in, ld,
-                       rows, P, k, seed, tl.tiles, tl.tile_size, tpg, partial);
+                       rows, P, k, seed, pl.tl.tiles, pl.tl.tile_size, pl.chunks_per_tile,
+                       pl.chunks_per_group, partial);
     return hipGetLastError();
 }
 
 typedef hipError_t (*LaunchFn)(const void*, uint64_t, uint32_t, uint64_t, uint32_t, uint32_t,
-                               const jl::Tiling&, float*, hipStream_t);
+                               const Plan&, float*, hipStream_t);
 
 LaunchFn pick(int dtype, int proj_type) {
     static const LaunchFn table[3][2] = {
@@ -542,9 +561,10 @@ namespace trakhip {
 
 size_t project_workspace_bytes(uint64_t B, uint64_t P, uint32_t k, uint32_t num_feature_tiles) {
     if (B == 0 || P == 0 || k == 0 || num_feature_tiles == 0) return 0;
-    const jl::Tiling tl = jl::make_tiling(P, num_feature_tiles);
+    if (k % kColsPerWG != 0 || P > 0xFFFFFFFFull) return 0;
+    const Plan pl = make_plan(P, k, num_feature_tiles);
     const uint64_t rows = B < 32 ? B : 32;
-    return (size_t)tl.tiles * rows * k * sizeof(float);
+    return (size_t)pl.groups * rows * k * sizeof(float);
 }
 
 static int check_project_args(const void* in, int dtype, uint64_t B, uint64_t P, uint64_t ld, const void* ws,
@@ -566,8 +586,8 @@ int project_partials(const void* in, int dtype, uint64_t B, uint64_t P, uint64_t
     const int e = check_project_args(in, dtype, B, P, ld, ws, ws_bytes, k, num_feature_tiles, proj_type);
     if (e) return e;
     if (B > 32) return TRAKHIP_ERR_SHAPE;
-    const jl::Tiling tl = jl::make_tiling(P, num_feature_tiles);
-    if (pick(dtype, proj_type)(in, ld, (uint32_t)B, P, k, seed, tl, static_cast<float*>(ws), s) != hipSuccess)
+    const Plan pl = make_plan(P, k, num_feature_tiles);
+    if (pick(dtype, proj_type)(in, ld, (uint32_t)B, P, k, seed, pl, static_cast<float*>(ws), s) != hipSuccess)
         return TRAKHIP_ERR_LAUNCH;
     return TRAKHIP_OK;
 }
@@ -578,9 +598,7 @@ int project_reduce(const void* ws, uint64_t B, uint64_t P, uint32_t k, uint32_t 
     if (B == 0 || B > 32 || P == 0 || P > 0xFFFFFFFFull || num_feature_tiles == 0) return TRAKHIP_ERR_SHAPE;
     if (!ws || !out) return TRAKHIP_ERR_NULL;
     if ((reinterpret_cast<uintptr_t>(ws) % 16) || (reinterpret_cast<uintptr_t>(out) % 16)) return TRAKHIP_ERR_ALIGN;
-    const jl::Tiling tl = jl::make_tiling(P, num_feature_tiles);
-    const uint32_t tpg = tiles_per_group(tl.tiles, k / kColsPerWG);
-    const uint32_t groups = (tl.tiles + tpg - 1) / tpg;
+    const uint32_t groups = make_plan(P, k, num_feature_tiles).groups;
     const uint64_t n4 = B * k / 4;
     hipLaunchKernelGGL(jl_reduce_kernel, dim3((uint32_t)((n4 + 255) / 256)), dim3(256), 0, s,
                        static_cast<const float*>(ws), groups, n4, scale, out);
