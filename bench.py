@@ -128,9 +128,57 @@ def bench_projection(torch, dev, steps, warmup, n_batches):
     }
 
 
+def resnet18_param_shapes():
+    """Parameter shapes of torchvision's resnet18 in `named_parameters()` order (62 tensors,
+    11 689 512 elements)."""
+    shapes = [(64, 3, 7, 7), (64,), (64,)]
+    inp = 64
+    for out, stride in ((64, 1), (128, 2), (256, 2), (512, 2)):
+        for block in range(2):
+            cin = inp if block == 0 else out
+            shapes += [(out, cin, 3, 3), (out,), (out,), (out, out, 3, 3), (out,), (out,)]
+            if block == 0 and (stride != 1 or inp != out):
+                shapes += [(out, inp, 1, 1), (out,), (out,)]
+        inp = out
+    shapes += [(1000, 512), (1000,)]
+    return shapes
+
+
+def bench_featurize_path(torch, dev, reps=20):
+    """The projector call of TRAKer.featurize on a ResNet-18 gradient dict: flatten-and-copy then
+    project (what the reference does) against projecting the dict in place."""
+    import math
+
+    from trak_amd import CudaProjector, ProjectionType, vectorize
+
+    shapes = resnet18_param_shapes()
+    P = sum(math.prod(sh) for sh in shapes)
+    assert P == 11_689_512 and len(shapes) == 62
+    gen = torch.Generator(device=dev).manual_seed(20_006)
+    grads = {i: (torch.randn(32, *sh, generator=gen, device=dev) * 1e-3).half() for i, sh in enumerate(shapes)}
+    proj = CudaProjector(P, 4096, 7, ProjectionType.rademacher, dev, 32)
+
+    def timed(fn):
+        for _ in range(5):
+            fn()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            fn()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) * 1e3 / reps
+
+    flat_ms = timed(lambda: proj.project(vectorize(grads, device=dev), 0))
+    gather_ms = timed(lambda: proj.project(grads, 0))
+    same = bool(torch.equal(proj.project(vectorize(grads, device=dev), 0), proj.project(grads, 0)))
+    return {"vectorize_then_project_ms": flat_ms, "project_dict_in_place_ms": gather_ms, "bit_identical": same,
+            "tflops_in_place": 2.0 * 32 * P * 4096 / gather_ms / 1e9}
+
+
 def bench_other_configs(torch, dev):
-    """Throughput of the other projection configurations of BASELINE.json (not part of the default
-    line; `--all-configs` prints them to stderr for the design notes)."""
+    """Throughput of the other projection configurations (the CPU-runnable fp32 case, the
+    ResNet-9-sized case and the BERT-sized chunked normal case); not part of the default line,
+    `--all-configs` prints them to stderr."""
     from trak_amd import ChunkedCudaProjector, CudaProjector, ProjectionType
 
     res = {}
@@ -235,7 +283,7 @@ def cpu_baseline(torch):
         "value": flop / dt / 1e12, "unit": "TFLOP/s", "cores": cores, "kind": "port",
         "sample": f"BasicProjector restatement, full config [16,1048576] fp32 -> 512 rademacher, {dt:.2f} s",
     }
-    N, M, kk = 4000, 1000, 1024
+    N, M, kk = 20_000, 4_000, 2048
     X = torch.randn(N, kk, generator=gen) / 32
     Xt = torch.randn(M, kk, generator=gen) / 32
     sc = BasicScoreComputerCPU(lambda_reg=1e-3)
@@ -264,8 +312,8 @@ def main():
                     help="also run one 1 GiB device-to-device copy (reference point for rocprofv3 byte counters)")
     args = ap.parse_args()
     if args.gpus != 1:
-        print("bench.py measures one GPU: this build has no multi-GPU path (see DESIGN.md, sharding note); "
-              "run with --gpus 1", file=sys.stderr)
+        print("bench.py measures one GPU: this library has no multi-GPU path (the projection shards over rows, "
+              "columns or parameters without changing the kernel); run with --gpus 1", file=sys.stderr)
         sys.exit(2)
 
     import torch
@@ -284,6 +332,7 @@ def main():
     torch.cuda.empty_cache()
     if args.all_configs:
         print(json.dumps(bench_other_configs(torch, dev), indent=1), file=sys.stderr)
+        print(json.dumps({"featurize_path": bench_featurize_path(torch, dev)}, indent=1), file=sys.stderr)
         torch.cuda.empty_cache()
     scoring = None if args.no_scoring else bench_scoring(torch, dev)
     torch.cuda.empty_cache()

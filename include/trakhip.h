@@ -79,6 +79,25 @@ int trakhip_project_partials(const void* in_dev, int in_dtype, uint64_t B, uint6
 int trakhip_project_reduce(const void* workspace_dev, uint64_t B, uint64_t P, uint32_t proj_dim,
                            uint32_t num_feature_tiles, float scale, float* out_dev, void* stream);
 
+/* One piece of a gradient that is stored as a list of tensors (one per model parameter): features
+ * [first, first + numel) of every row live at ptr[row * ld + (feature - first)]. */
+typedef struct trakhip_segment {
+    const void* ptr; /* device memory, aligned to the element size */
+    uint64_t first;  /* first feature index of this piece */
+    uint64_t numel;  /* features in this piece (>= 1) */
+    uint64_t ld;     /* row pitch in elements (>= numel) */
+} trakhip_segment;
+
+/* Phase 1 of the projection reading the [B, P] gradient through a table of segments instead of one
+ * dense matrix: the flatten-and-copy of trak.utils.vectorize (trak/utils.py:80-110) and the chunk
+ * packing of ChunkedCudaProjector.project (trak/projectors.py:479-503) disappear.  segs_dev is a
+ * device array of n_segs segments, sorted by `first`, contiguous (first[i+1] = first[i] + numel[i])
+ * and covering [0, P); all of element type in_dtype; B <= 32.  Result and workspace as for
+ * trakhip_project_partials; finish with trakhip_project_reduce. */
+int trakhip_project_gather_partials(const trakhip_segment* segs_dev, uint32_t n_segs, int in_dtype, uint64_t B,
+                                    uint64_t P, void* workspace_dev, size_t workspace_bytes, uint32_t proj_dim,
+                                    uint32_t seed, uint32_t num_feature_tiles, int proj_type, void* stream);
+
 /* Writes the block S[f0 : f0+nf, c0 : c0+nc] of the projection matrix that trakhip_project uses
  * for (seed, num_feature_tiles, P) as fp32, row-major [nf, nc].  The reference never stores S
  * (it exists only inside fast_jl/random.cuh:27-60); this is the hook that lets a caller check

@@ -343,3 +343,49 @@ def test_uint32_overflow_shapes_through_chunks(gpu, c_oracle, shape):
     proj.free_memory()
     del g, chunks
     torch.cuda.empty_cache()
+
+
+# ---- gathered input: the gradient dict is projected in place -----------------------------------
+
+
+@pytest.mark.parametrize("proj_type", [R, G])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
+def test_gather_equals_vectorize_then_project(gpu, c_oracle, proj_type, dtype):
+    from trak_amd import vectorize
+
+    gen = torch.Generator(device="cpu").manual_seed(77)
+    B = 19
+    shapes = [(64, 3, 3, 3), (64,), (), (128, 64, 3, 3), (7,), (1,), (33, 5), (1000, 17), (2, 1, 1), (511,), (10, 10)]
+    grads = {}
+    for i, sh in enumerate(shapes):
+        grads[f"p{i}"] = (torch.randn(B, *sh, generator=gen) * 1e-2).to(dtype).to(gpu)
+    # one parameter arrives as a non-contiguous view (a column slice of a wider buffer)
+    wide = (torch.randn(B, 300, generator=gen) * 1e-2).to(dtype).to(gpu)
+    grads["view"] = wide[:, 10:210]
+    flat = vectorize(grads, device=gpu)
+    P, k, seed, tiles = flat.shape[1], 1024, 5, 256
+    dense = fn(proj_type)(flat, k, seed, tiles)
+    gathered = fast_jl.project_gather(list(grads.values()), k, seed, tiles, NAMES[proj_type])
+    assert torch.equal(dense, gathered)
+    # and against the oracle directly
+    want = c_oracle.project(to_f32_numpy(flat), seed, tiles, 0, 32, proj_type)
+    assert rel_l2_rows(gathered[:, :32].cpu().numpy(), want).max() < TOL[dtype]
+    # the scale of the featurize epilogue (trak/traker.py:426) is applied in the reduction
+    scaled = fast_jl.project_gather(list(grads.values()), k, seed, tiles, NAMES[proj_type], scale=1.0 / math.sqrt(P))
+    assert torch.allclose(scaled, dense / math.sqrt(P), rtol=1e-6, atol=0)
+    # CudaProjector takes the dict path
+    proj = _projector(P, k, seed, ProjectionType(NAMES[proj_type]), dtype)
+    assert torch.equal(proj.project(grads, model_id=0), dense)
+    assert torch.equal(proj.project(flat, model_id=0), dense)
+
+
+def test_gather_many_rows_and_tiny_segments(gpu):
+    # B > 32 walks the rows in blocks of 32; segments of one feature straddle every 16-byte piece
+    from trak_amd import vectorize
+
+    gen = torch.Generator(device="cpu").manual_seed(78)
+    B = 45
+    grads = {i: torch.randn(B, n, generator=gen).half().to(gpu) for i, n in enumerate([1, 1, 3, 1, 5, 2, 900, 1, 1, 7, 4000, 3])}
+    flat = vectorize(grads, device=gpu)
+    dense = fn(R)(flat, 512, 11, 256)
+    assert torch.equal(fast_jl.project_gather(list(grads.values()), 512, 11, 256, "rademacher"), dense)

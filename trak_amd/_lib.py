@@ -44,6 +44,8 @@ def load():
     lib.trakhip_project.restype = i32
     lib.trakhip_project_partials.argtypes = [vp, i32, u64, u64, u64, vp, sz, u32, u32, u32, i32, vp]
     lib.trakhip_project_partials.restype = i32
+    lib.trakhip_project_gather_partials.argtypes = [vp, u32, i32, u64, u64, vp, sz, u32, u32, u32, i32, vp]
+    lib.trakhip_project_gather_partials.restype = i32
     lib.trakhip_project_reduce.argtypes = [vp, u64, u64, u32, u32, f32, vp, vp]
     lib.trakhip_project_reduce.restype = i32
     lib.trakhip_materialize.argtypes = [u32, u32, u64, u64, u64, u32, u32, i32, vp, i32, vp]

@@ -41,6 +41,14 @@ int trakhip_project_partials(const void* in_dev, int in_dtype, uint64_t B, uint6
                                      num_feature_tiles, proj_type, static_cast<hipStream_t>(stream));
 }
 
+int trakhip_project_gather_partials(const trakhip_segment* segs_dev, uint32_t n_segs, int in_dtype, uint64_t B,
+                                    uint64_t P, void* workspace_dev, size_t workspace_bytes, uint32_t proj_dim,
+                                    uint32_t seed, uint32_t num_feature_tiles, int proj_type, void* stream) {
+    return trakhip::project_gather_partials(segs_dev, n_segs, in_dtype, B, P, workspace_dev, workspace_bytes,
+                                            proj_dim, seed, num_feature_tiles, proj_type,
+                                            static_cast<hipStream_t>(stream));
+}
+
 int trakhip_project_reduce(const void* workspace_dev, uint64_t B, uint64_t P, uint32_t proj_dim,
                            uint32_t num_feature_tiles, float scale, float* out_dev, void* stream) {
     return trakhip::project_reduce(workspace_dev, B, P, proj_dim, num_feature_tiles, scale, out_dev,

@@ -182,15 +182,159 @@ struct Stage32 {
     }
 };
 
-template <int IN>
+// ---- gathered input: the gradient is a list of per-parameter tensors --------------------
+//
+// Segment i holds features [first, first + numel) as a row-major [B, numel] tensor with row
+// pitch ld (what TRAK's gradient dict holds per parameter, trak/utils.py:80-110).  A thread's
+// pieces of one chunk all start at the same feature, and that feature only grows while the
+// workgroup walks its run, so the thread keeps the segment it is in and moves forward when needed.
+// ROWS = pieces per thread and chunk (all at the same feature, ROW_STEP rows apart).
+template <int ROWS>
+struct SegCursor {
+    uint32_t idx;
+    uint32_t first, end;         // feature range of segs[idx] (P < 2^32)
+    const char* base[ROWS];      // base[i] + feature * elem_size = address of (row_i, feature)
+
+    __device__ __forceinline__ void set(const trakhip_segment* segs, uint32_t i, uint32_t row0, uint32_t row_step,
+                                        uint32_t esz) {
+        const trakhip_segment sg = segs[i];
+        idx = i;
+        first = (uint32_t)sg.first;
+        end = (uint32_t)(sg.first + sg.numel);
+        const char* p = static_cast<const char*>(sg.ptr) - sg.first * esz;
+#pragma unroll
+        for (int r = 0; r < ROWS; ++r) base[r] = p + (uint64_t)(row0 + row_step * r) * sg.ld * esz;
+    }
+    // segment containing feature f (segments are sorted, contiguous and cover [0, P); f < P)
+    __device__ __forceinline__ void seek(const trakhip_segment* segs, uint32_t n, uint32_t f, uint32_t row0,
+                                         uint32_t row_step, uint32_t esz) {
+        uint32_t lo = 0, hi = n - 1;
+        while (lo < hi) {
+            const uint32_t mid = (lo + hi + 1) >> 1;
+            if (segs[mid].first <= f)
+                lo = mid;
+            else
+                hi = mid - 1;
+        }
+        set(segs, lo, row0, row_step, esz);
+    }
+    __device__ __forceinline__ void advance(const trakhip_segment* segs, uint32_t n, uint32_t f, uint32_t row0,
+                                            uint32_t row_step, uint32_t esz) {
+        while (f >= end && idx + 1 < n) set(segs, idx + 1, row0, row_step, esz);
+    }
+};
+
+// A piece of COUNT elements that straddles a segment boundary or the end of the tile (slow path,
+// kept out of line and rolled up so that the hot loop stays small).
+template <typename T, int COUNT>
+__device__ __noinline__ uint4 gather_piece(const trakhip_segment* segs, uint32_t n, uint32_t idx, uint32_t row,
+                                           uint64_t f, uint64_t f_end) {
+    uint32_t e[4] = {0u, 0u, 0u, 0u};
+#pragma unroll 1
+    for (int t = 0; t < COUNT; ++t) {
+        const uint64_t ff = f + t;
+        if (ff >= f_end) break;
+        while (idx + 1 < n && ff >= segs[idx + 1].first) ++idx;
+        const trakhip_segment sg = segs[idx];
+        const uint32_t val = (uint32_t) reinterpret_cast<const T*>(sg.ptr)[(uint64_t)row * sg.ld + (ff - sg.first)];
+        if (sizeof(T) == 2)
+            e[t >> 1] |= val << (16 * (t & 1));
+        else
+            e[t] = val;
+    }
+    return {e[0], e[1], e[2], e[3]};
+}
+
+struct Gather16 : Stage16 {
+    SegCursor<4> cur;
+    __device__ __forceinline__ void init(const trakhip_segment* segs, uint32_t n, uint64_t f_begin, uint64_t P,
+                                         int tid) {
+        const uint64_t f = f_begin + 8u * (tid & 31);
+        cur.seek(segs, n, (uint32_t)(f < P ? f : P - 1), tid >> 5, 8, 2);
+    }
+    __device__ __forceinline__ void load(const trakhip_segment* segs, uint64_t n64, uint32_t rows, uint64_t f_begin,
+                                         uint64_t f_end, int tid) {
+        const uint32_t n = (uint32_t)n64;
+        const uint64_t f64 = f_begin + 8u * (tid & 31);
+        const bool live = f64 < f_end;
+        const uint32_t f = (uint32_t)f64;
+        if (live) cur.advance(segs, n, f, tid >> 5, 8, 2);
+        const uint32_t lim = (uint32_t)f_end < cur.end ? (uint32_t)f_end : cur.end;  // f_end <= P < 2^32
+        const bool whole = live && f + 8u <= lim && f + 8u > f;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const uint32_t row = (tid >> 5) + 8 * i;
+            uint4 val = {0u, 0u, 0u, 0u};
+            if (live && row < rows) {
+                if (whole) {
+                    const Raw16 r = *reinterpret_cast<const Raw16*>(cur.base[i] + (uint64_t)f * 2);
+                    val = {r.x, r.y, r.z, r.w};
+                } else {
+                    val = gather_piece<uint16_t, 8>(segs, n, cur.idx, row, f64, f_end);
+                }
+            }
+            v[i] = val;
+        }
+    }
+};
+
+struct Gather32 : Stage32 {
+    SegCursor<8> cur;
+    __device__ __forceinline__ void init(const trakhip_segment* segs, uint32_t n, uint64_t f_begin, uint64_t P,
+                                         int tid) {
+        const uint64_t f = f_begin + 4u * (tid & 63);
+        cur.seek(segs, n, (uint32_t)(f < P ? f : P - 1), tid >> 6, 4, 4);
+    }
+    __device__ __forceinline__ void load(const trakhip_segment* segs, uint64_t n64, uint32_t rows, uint64_t f_begin,
+                                         uint64_t f_end, int tid) {
+        const uint32_t n = (uint32_t)n64;
+        const uint64_t f64 = f_begin + 4u * (tid & 63);
+        const bool live = f64 < f_end;
+        const uint32_t f = (uint32_t)f64;
+        if (live) cur.advance(segs, n, f, tid >> 6, 4, 4);
+        const uint32_t lim = (uint32_t)f_end < cur.end ? (uint32_t)f_end : cur.end;
+        const bool whole = live && f + 4u <= lim && f + 4u > f;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const uint32_t row = (tid >> 6) + 4 * i;
+            uint4 val = {0u, 0u, 0u, 0u};
+            if (live && row < rows) {
+                if (whole) {
+                    const Raw16f r = *reinterpret_cast<const Raw16f*>(cur.base[i] + (uint64_t)f * 4);
+                    val = {r.x, r.y, r.z, r.w};
+                } else {
+                    val = gather_piece<uint32_t, 4>(segs, n, cur.idx, row, f64, f_end);
+                }
+            }
+            v[i] = val;
+        }
+    }
+};
+
+template <int IN, bool GATHER>
 struct StageOf {
     typedef Stage16 type;
     typedef uint16_t elem;
 };
 template <>
-struct StageOf<TRAKHIP_F32> {
+struct StageOf<TRAKHIP_F32, false> {
     typedef Stage32 type;
     typedef float elem;
+};
+template <>
+struct StageOf<TRAKHIP_F16, true> {
+    typedef Gather16 type;
+    typedef trakhip_segment elem;
+};
+template <>
+struct StageOf<TRAKHIP_BF16, true> {
+    typedef Gather16 type;
+    typedef trakhip_segment elem;
+};
+template <>
+struct StageOf<TRAKHIP_F32, true> {
+    typedef Gather32 type;
+    typedef trakhip_segment elem;
 };
 
 // ---- B operand generation --------------------------------------------------------------------
@@ -272,14 +416,16 @@ __device__ __forceinline__ uint4 signs_of(uint64_t m01, uint64_t m23, uint32_t o
     return b;
 }
 
-template <int IN, int PT>
+// GATHER: g_in is a device array of trakhip_segment and ld their number; otherwise g_in is the
+// dense [rows, P] matrix with row pitch ld.
+template <int IN, int PT, bool GATHER>
 __global__ __launch_bounds__(kThreads, 2) void jl_project_kernel(
     const void* __restrict__ g_in, uint64_t ld, uint32_t rows, uint64_t P, uint32_t k,
     uint32_t seed, uint32_t tiles, uint64_t tile_size, uint32_t chunks_per_tile,
     uint32_t chunks_per_group, float* __restrict__ partial) {
     typedef InTraits<IN> Tr;
-    typedef typename StageOf<IN>::type Stage;
-    typedef typename StageOf<IN>::elem Elem;
+    typedef typename StageOf<IN, GATHER>::type Stage;
+    typedef typename StageOf<IN, GATHER>::elem Elem;
     constexpr bool kBf = Tr::bf16;
     constexpr int kPlanes = Tr::planes;
     // 16-bit inputs: two LDS buffers, one barrier per chunk.  fp32 inputs (three planes) keep one
@@ -321,6 +467,7 @@ __global__ __launch_bounds__(kThreads, 2) void jl_project_kernel(
     {
         const uint64_t lo = (uint64_t)t0 * tile_size;
         const uint64_t hi = (lo + tile_size < P) ? lo + tile_size : P;
+        if constexpr (GATHER) st.init(g, (uint32_t)ld, lo + (uint64_t)s0 * kChunk, P, tid);
         st.load(g, ld, rows, lo + (uint64_t)s0 * kChunk, hi, tid);
     }
     int cur = 0;
@@ -531,13 +678,13 @@ Plan make_plan(uint64_t P, uint32_t k, uint32_t num_feature_tiles) {
     return p;
 }
 
-template <int IN, int PT>
+template <int IN, int PT, bool GATHER>
 hipError_t launch_one(const void* in, uint64_t ld, uint32_t rows, uint64_t P, uint32_t k,
                       uint32_t seed, const Plan& pl, float* partial, hipStream_t s) {
     const uint32_t groups8 = (pl.groups + 7u) / 8u * 8u;
     const uint64_t wgs = (uint64_t)groups8 * pl.col_blocks;
     if (wgs > 0x7FFFFFFFull) return hipErrorInvalidValue;
-    hipLaunchKernelGGL((jl_project_kernel<IN, PT>), dim3((uint32_t)wgs), dim3(kThreads), 0, s, in, ld,
+    hipLaunchKernelGGL((jl_project_kernel<IN, PT, GATHER>), dim3((uint32_t)wgs), dim3(kThreads), 0, s, in, ld,
                        rows, P, k, seed, pl.tl.tiles, pl.tl.tile_size, pl.chunks_per_tile,
                        pl.chunks_per_group, partial);
     return hipGetLastError();
@@ -546,13 +693,16 @@ hipError_t launch_one(const void* in, uint64_t ld, uint32_t rows, uint64_t P, ui
 typedef hipError_t (*LaunchFn)(const void*, uint64_t, uint32_t, uint64_t, uint32_t, uint32_t,
                                const Plan&, float*, hipStream_t);
 
-LaunchFn pick(int dtype, int proj_type) {
-    static const LaunchFn table[3][2] = {
-        {launch_one<TRAKHIP_F16, TRAKHIP_RADEMACHER>, launch_one<TRAKHIP_F16, TRAKHIP_NORMAL>},
-        {launch_one<TRAKHIP_BF16, TRAKHIP_RADEMACHER>, launch_one<TRAKHIP_BF16, TRAKHIP_NORMAL>},
-        {launch_one<TRAKHIP_F32, TRAKHIP_RADEMACHER>, launch_one<TRAKHIP_F32, TRAKHIP_NORMAL>},
+LaunchFn pick(int dtype, int proj_type, bool gather) {
+    static const LaunchFn table[2][3][2] = {
+        {{launch_one<TRAKHIP_F16, TRAKHIP_RADEMACHER, false>, launch_one<TRAKHIP_F16, TRAKHIP_NORMAL, false>},
+         {launch_one<TRAKHIP_BF16, TRAKHIP_RADEMACHER, false>, launch_one<TRAKHIP_BF16, TRAKHIP_NORMAL, false>},
+         {launch_one<TRAKHIP_F32, TRAKHIP_RADEMACHER, false>, launch_one<TRAKHIP_F32, TRAKHIP_NORMAL, false>}},
+        {{launch_one<TRAKHIP_F16, TRAKHIP_RADEMACHER, true>, launch_one<TRAKHIP_F16, TRAKHIP_NORMAL, true>},
+         {launch_one<TRAKHIP_BF16, TRAKHIP_RADEMACHER, true>, launch_one<TRAKHIP_BF16, TRAKHIP_NORMAL, true>},
+         {launch_one<TRAKHIP_F32, TRAKHIP_RADEMACHER, true>, launch_one<TRAKHIP_F32, TRAKHIP_NORMAL, true>}},
     };
-    return table[dtype][proj_type];
+    return table[gather ? 1 : 0][dtype][proj_type];
 }
 
 }  // namespace
@@ -587,7 +737,22 @@ int project_partials(const void* in, int dtype, uint64_t B, uint64_t P, uint64_t
     if (e) return e;
     if (B > 32) return TRAKHIP_ERR_SHAPE;
     const Plan pl = make_plan(P, k, num_feature_tiles);
-    if (pick(dtype, proj_type)(in, ld, (uint32_t)B, P, k, seed, pl, static_cast<float*>(ws), s) != hipSuccess)
+    if (pick(dtype, proj_type, false)(in, ld, (uint32_t)B, P, k, seed, pl, static_cast<float*>(ws), s) != hipSuccess)
+        return TRAKHIP_ERR_LAUNCH;
+    return TRAKHIP_OK;
+}
+
+int project_gather_partials(const trakhip_segment* segs, uint32_t n_segs, int dtype, uint64_t B, uint64_t P,
+                            void* ws, size_t ws_bytes, uint32_t k, uint32_t seed, uint32_t num_feature_tiles,
+                            int proj_type, hipStream_t s) {
+    // segs is device memory: its contents (sorted, contiguous, covering [0, P)) are the caller's contract
+    const int e = check_project_args(segs, dtype, B, P, P, ws, ws_bytes, k, num_feature_tiles, proj_type);
+    if (e) return e;
+    if (B > 32 || n_segs == 0) return TRAKHIP_ERR_SHAPE;
+    if (reinterpret_cast<uintptr_t>(segs) % 8) return TRAKHIP_ERR_ALIGN;
+    const Plan pl = make_plan(P, k, num_feature_tiles);
+    if (pick(dtype, proj_type, true)(segs, n_segs, (uint32_t)B, P, k, seed, pl, static_cast<float*>(ws), s) !=
+        hipSuccess)
         return TRAKHIP_ERR_LAUNCH;
     return TRAKHIP_OK;
 }

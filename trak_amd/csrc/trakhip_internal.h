@@ -14,6 +14,9 @@ int project(const void* in, int dtype, uint64_t B, uint64_t P, uint64_t ld, floa
             hipStream_t s);
 int project_partials(const void* in, int dtype, uint64_t B, uint64_t P, uint64_t ld, void* ws, size_t ws_bytes,
                      uint32_t k, uint32_t seed, uint32_t num_feature_tiles, int proj_type, hipStream_t s);
+int project_gather_partials(const trakhip_segment* segs, uint32_t n_segs, int dtype, uint64_t B, uint64_t P,
+                            void* ws, size_t ws_bytes, uint32_t k, uint32_t seed, uint32_t num_feature_tiles,
+                            int proj_type, hipStream_t s);
 int project_reduce(const void* ws, uint64_t B, uint64_t P, uint32_t k, uint32_t num_feature_tiles, float scale,
                    float* out, hipStream_t s);
 int materialize_device(uint32_t seed, uint32_t num_feature_tiles, uint64_t P, uint64_t f0, uint64_t nf,

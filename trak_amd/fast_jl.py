@@ -13,6 +13,8 @@ from . import _lib
 
 _DTYPES = {torch.float16: _lib.F16, torch.bfloat16: _lib.BF16, torch.float32: _lib.F32}
 _workspaces = {}
+_segment_tables = {}  # (device, rows) -> device table; the key holds every pointer, so a hit is exact
+_SEGMENT_TABLE_CACHE = 16
 
 
 def _workspace(device, nbytes):
@@ -29,6 +31,23 @@ def _workspace(device, nbytes):
 
 def free_workspaces():
     _workspaces.clear()
+    _segment_tables.clear()
+
+
+def _segment_table(device, rows):
+    """Device array of trakhip_segment {ptr, first, numel, ld} for these rows.  Gradient buffers
+    come back at the same addresses batch after batch (caching allocator), so the upload is
+    usually skipped."""
+    key = (device, rows)
+    table = _segment_tables.get(key)
+    if table is None:
+        if len(_segment_tables) >= _SEGMENT_TABLE_CACHE:
+            _segment_tables.pop(next(iter(_segment_tables)))
+        host = torch.tensor(rows, dtype=torch.int64).pin_memory()
+        table = host.to(device, non_blocking=True)
+        _segment_tables[key] = table
+        table._host = host  # keeps the pinned source alive until the copy has certainly run
+    return table
 
 
 def _project(input, N, seed, num_feature_tiles, proj_type, ld=None):
@@ -73,6 +92,79 @@ def _project(input, N, seed, num_feature_tiles, proj_type, ld=None):
             ctypes.c_void_p(stream),
         )
     _lib.check(code)
+    return out
+
+
+def _flat_rows(p):
+    """[B, numel] view of one gradient tensor [B, ...] with unit inner stride (a copy only when the
+    tensor cannot be viewed that way); tensors with fewer than two dims count as one column
+    (trak/utils.py:99-104)."""
+    B = p.shape[0]
+    flat = p.reshape(B, 1) if p.dim() < 2 else p.flatten(start_dim=1)
+    if flat.shape[1] > 1 and flat.stride(1) != 1:
+        flat = flat.contiguous()
+    if B > 1 and flat.stride(0) < flat.shape[1]:
+        flat = flat.contiguous()
+    return flat
+
+
+def gather_supported(tensors):
+    """True when a list of gradient tensors can be projected in place (no flatten-and-copy): same
+    supported dtype, same CUDA device, same batch size."""
+    tensors = list(tensors)
+    if not tensors:
+        return False
+    t0 = tensors[0]
+    if not isinstance(t0, torch.Tensor) or not t0.is_cuda or t0.dtype not in _DTYPES or t0.dim() < 1:
+        return False
+    return all(
+        isinstance(t, torch.Tensor) and t.device == t0.device and t.dtype == t0.dtype and t.dim() >= 1
+        and t.shape[0] == t0.shape[0] and t.numel() > 0
+        for t in tensors
+    )
+
+
+def project_gather(tensors, N, seed, num_feature_tiles, proj_type, scale=1.0):
+    """Projects the gradient given as a list of per-parameter tensors [B, ...] (in order) without
+    materializing the [B, P] matrix: same result, bit for bit, as `project_*` on
+    `trak.utils.vectorize` of the same tensors.  Returns fp32 [B, N] times `scale`."""
+    tensors = list(tensors)
+    if not gather_supported(tensors):
+        raise RuntimeError("project_gather needs CUDA tensors of one supported dtype, device and batch size")
+    flats = [_flat_rows(t) for t in tensors]
+    device, dtype = flats[0].device, flats[0].dtype
+    B = flats[0].shape[0]
+    esz = flats[0].element_size()
+    N, seed, tiles = int(N), int(seed) & 0xFFFFFFFF, int(num_feature_tiles)
+    lib = _lib.load()
+    if N <= 0 or N % 512 != 0:
+        _lib.check(_lib.ERR_PROJ_DIM)
+    rows, first = [], 0
+    for f in flats:
+        numel = f.shape[1]
+        ld = f.stride(0) if B > 1 else numel
+        rows.append([f.data_ptr(), first, numel, ld])
+        first += numel
+    P = first
+    pt = _lib.NORMAL if str(getattr(proj_type, "value", proj_type)) in ("normal", "1") else _lib.RADEMACHER
+    with torch.cuda.device(device):
+        out = torch.empty((B, N), dtype=torch.float32, device=device)
+        nbytes = lib.trakhip_project_workspace(B, P, N, tiles)
+        ws = _workspace(device, nbytes)
+        stream = torch.cuda.current_stream(device).cuda_stream
+        for b0 in range(0, B, 32):
+            nb = min(32, B - b0)
+            table_dev = _segment_table(device, tuple((p + b0 * ld * esz, fi, n, ld) for p, fi, n, ld in rows))
+            code = lib.trakhip_project_gather_partials(
+                ctypes.c_void_p(table_dev.data_ptr()), len(rows), _DTYPES[dtype], nb, P,
+                ctypes.c_void_p(ws.data_ptr()), ws.numel(), N, seed, tiles, pt, ctypes.c_void_p(stream),
+            )
+            _lib.check(code)
+            code = lib.trakhip_project_reduce(
+                ctypes.c_void_p(ws.data_ptr()), nb, P, N, tiles, float(scale),
+                ctypes.c_void_p(out.data_ptr() + b0 * N * 4), ctypes.c_void_p(stream),
+            )
+            _lib.check(code)
     return out
 
 

@@ -122,6 +122,13 @@ class CudaProjector(AbstractProjector):
 
     def project(self, grads: Union[dict, Tensor], model_id: int) -> Tensor:
         if isinstance(grads, dict):
+            tensors = list(grads.values())
+            if fast_jl.gather_supported(tensors) and tensors[0].device == self._device:
+                # the kernel reads the per-parameter tensors in place: same result as projecting
+                # vectorize(grads) (trak/projectors.py:389-390) without building the [B, P] copy
+                return fast_jl.project_gather(
+                    tensors, self.proj_dim, self.seed + int(1e4) * model_id, self.num_sms, _type_name(self.proj_type)
+                )
             grads = vectorize(grads, device=self.device)
 
         batch_size = grads.shape[0]
