@@ -113,7 +113,11 @@ def test_score_computer_matches_float64_oracle(gpu, N, k, M, lam, max_dim):
         sc.get_scores(feats, Xt.to(gpu), accumulator=acc)     # [N_train, M_targets] (trak/score_computers.py:90)
         sc.get_scores(feats, Xt.to(gpu), accumulator=acc)
         assert rel_max(acc.numpy(), 2 * scores_want) < 1e-4
-    # lambda = 0 identity: features^T X = I / mean|inv|
+    # accumulator resident on the GPU: accumulated in the GEMM epilogue
+    dev_acc = torch.zeros(N, M, device=gpu)
+    sc.get_scores(feats, Xt.to(gpu), accumulator=dev_acc)
+    sc.get_scores(feats, Xt.to(gpu), accumulator=dev_acc)
+    assert rel_max(dev_acc.cpu().numpy(), 2 * scores_want) < 1e-4
     # fused finalize_scores epilogue (trak/traker.py:670-678) for one model
     fused = sc.get_scaled_scores(feats, Xt.to(gpu), otl.to(gpu))
     assert rel_max(fused.cpu().numpy(), so.finalize_scores_f64(scores_want, otl.numpy(), 1)) < 1e-4

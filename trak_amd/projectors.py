@@ -185,7 +185,32 @@ class ChunkedCudaProjector:
         del self.ch_input
         self.input_allocated = False
 
+    def _project_in_place(self, grads, model_id):
+        """Same grouping rule as the packing path below, but every chunk is handed to its projector
+        as a dict, which projects the parameter tensors where they are."""
+        groups, current, pointer = [], {}, 0
+        for name, p in grads.items():
+            param_size = 1 if len(p.shape) < 2 else p[0].numel()
+            if pointer + param_size > self.max_chunk_size:
+                groups.append((current, pointer))
+                current, pointer = {}, 0
+            current[name] = p
+            pointer += param_size
+        groups.append((current, pointer))
+        actual_bs = min(self.feat_bs, next(iter(grads.values())).shape[0])
+        acc = None
+        for index, (group, size) in enumerate(groups):
+            assert size == self.params_per_chunk[index]
+            if actual_bs != next(iter(group.values())).shape[0]:
+                group = {k: v[:actual_bs] for k, v in group.items()}
+            part = self.projector_per_chunk[index].project(group, model_id=model_id)
+            acc = part if acc is None else acc.add_(part)
+        return acc.to(self.dtype)
+
     def project(self, grads, model_id):
+        tensors = list(grads.values())
+        if fast_jl.gather_supported(tensors) and tensors[0].dtype == self.dtype:
+            return self._project_in_place(grads, model_id)
         self.allocate_input()
         acc = ch.zeros(size=(self.feat_bs, self.proj_dim), device=self.device, dtype=ch.float32)
         pointer = 0

@@ -96,7 +96,19 @@ class BasicScoreComputer(AbstractScoreComputer):
         train_dim = features.shape[0]
         target_dim = target_grads.shape[0]
         self.logger.debug(f"{train_dim=}, {target_dim=}")
-        scores = gemm_nt(features.to(self._dev), target_grads.to(self._dev))
+        f, t = features.to(self._dev), target_grads.to(self._dev)
+        if (
+            accumulator.is_cuda
+            and accumulator.device == f.device
+            and accumulator.dtype == ch.float32
+            and accumulator.dim() == 2
+            and accumulator.stride(1) == 1
+        ):
+            # accumulator on the GPU: the sum over checkpoints happens in the GEMM epilogue and the
+            # [N, M] matrix never crosses PCIe per checkpoint (trak/traker.py:641-668 moves it each time)
+            gemm_nt(f, t, out=accumulator, alpha=1.0, beta=1.0)
+            return
+        scores = gemm_nt(f, t)
         if accumulator.is_cuda:
             accumulator += scores.to(accumulator.dtype)
         else:
