@@ -175,6 +175,31 @@ def bench_featurize_path(torch, dev, reps=20):
             "tflops_in_place": 2.0 * 32 * P * 4096 / gather_ms / 1e9}
 
 
+def bench_batch_scaling(torch, dev):
+    """Projection throughput against the number of gradient rows per call at the ResNet-18 shape."""
+    from trak_amd import CudaProjector, ProjectionType
+
+    P, k = 11_689_512, 4096
+    proj = CudaProjector(P, k, 7, ProjectionType.rademacher, dev, 32)
+    gen = torch.Generator(device=dev).manual_seed(20_007)
+    res = {}
+    for B in (32, 64, 128):
+        g = (torch.randn(B, P, generator=gen, device=dev) * 1e-3).half()
+        for _ in range(8):
+            proj.project(g, 0)
+        torch.cuda.synchronize()
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        for _ in range(20):
+            proj.project(g, 0)
+        b.record()
+        torch.cuda.synchronize()
+        ms = a.elapsed_time(b) / 20
+        res[f"B={B}"] = {"ms": ms, "ms_per_32_rows": ms * 32 / B, "tflops": 2.0 * B * P * k / ms / 1e9}
+        del g
+    return res
+
+
 def bench_other_configs(torch, dev):
     """Throughput of the other projection configurations (the CPU-runnable fp32 case, the
     ResNet-9-sized case and the BERT-sized chunked normal case); not part of the default line,
@@ -333,6 +358,7 @@ def main():
     if args.all_configs:
         print(json.dumps(bench_other_configs(torch, dev), indent=1), file=sys.stderr)
         print(json.dumps({"featurize_path": bench_featurize_path(torch, dev)}, indent=1), file=sys.stderr)
+        print(json.dumps({"batch_scaling": bench_batch_scaling(torch, dev)}, indent=1), file=sys.stderr)
         torch.cuda.empty_cache()
     scoring = None if args.no_scoring else bench_scoring(torch, dev)
     torch.cuda.empty_cache()

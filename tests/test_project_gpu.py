@@ -389,3 +389,39 @@ def test_gather_many_rows_and_tiny_segments(gpu):
     flat = vectorize(grads, device=gpu)
     dense = fn(R)(flat, 512, 11, 256)
     assert torch.equal(fast_jl.project_gather(list(grads.values()), 512, 11, 256, "rademacher"), dense)
+
+
+# ---- more than 32 rows: the batch is walked 32 rows at a time ------------------------------------
+
+
+@pytest.mark.parametrize("proj_type", [R, G])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("B", [33, 64, 100, 129])
+def test_many_rows(gpu, c_oracle, proj_type, dtype, B):
+    P, k, tiles, seed = 9_001, 512, 256, 21
+    gen = torch.Generator(device="cpu").manual_seed(B)
+    g = (torch.randn(B, P, generator=gen) * 1e-2).to(dtype).to(gpu)
+    out = fn(proj_type)(g, k, seed, tiles)
+    assert out.shape == (B, k)
+    want = c_oracle.project(to_f32_numpy(g), seed, tiles, 480, 32, proj_type)
+    assert rel_l2_rows(out[:, 480:].cpu().numpy(), want).max() < TOL[dtype]
+    # every row is projected by the same matrix whichever pass it falls into: one-hot rows read it back
+    e = torch.zeros(B, P, dtype=dtype, device=gpu)
+    feats = [(37 * r) % P for r in range(B)]
+    e[torch.arange(B), torch.tensor(feats)] = 1.0
+    got = fn(proj_type)(e, k, seed, tiles).cpu().numpy()
+    for r in (0, 31, 32, 33, 63, B - 1):
+        if r < B:
+            assert np.array_equal(got[r], c_oracle.materialize(seed, tiles, P, feats[r], 1, 0, k, proj_type)[0]), r
+    # a batch and its first 32 rows agree
+    head = fn(proj_type)(g[:32].contiguous(), k, seed, tiles)
+    assert torch.allclose(out[:32], head, rtol=1e-4, atol=1e-5)
+
+
+def test_many_rows_gather(gpu):
+    from trak_amd import vectorize
+
+    gen = torch.Generator(device="cpu").manual_seed(5)
+    grads = {i: torch.randn(100, n, generator=gen).half().to(gpu) for i, n in enumerate([300, 1, 4097, 15, 2000])}
+    flat = vectorize(grads, device=gpu)
+    assert torch.equal(fast_jl.project_gather(list(grads.values()), 512, 3, 256, "rademacher"), fn(R)(flat, 512, 3, 256))
