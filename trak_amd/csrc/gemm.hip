@@ -11,10 +11,12 @@
 //   "k-row"  (KMAJOR = true):  element (x, k) at ptr[k * ld + x]   (x contiguous)
 // NT = (row-k, row-k), TN = (k-row, k-row), NN = (row-k, k-row).
 //
-// Workgroup = 256 threads = 4 waves in a 2x2 grid, 128x128 tile of C, k step 16, two LDS
-// buffers.  A wave owns 64x64 of C = 2x2 MFMA tiles (64 accumulator VGPRs).  The MFMA sums
-// over k in any order, so lane half h (= lane / 32) is given k = 8*s + 4*h + t for the t-th
-// MFMA of sub-step s: a row-k operand then needs ONE 16-byte LDS read per four MFMAs.
+// Workgroup = 256 threads = 4 waves in a 2x2 grid, 128 x BN tile of C (BN = 128 or 256), k step
+// 16, two LDS buffers.  A wave owns 64 x BN/2 of C = 2 x (2 or 4) MFMA tiles (64 or 128
+// accumulator VGPRs); the wide tile does twice the multiply-adds per LDS round trip and barrier
+// and is used when C has at least 256 columns.  The MFMA sums over k in any order, so lane half
+// h (= lane / 32) is given k = 8*s + 4*h + t for the t-th MFMA of sub-step s: a row-k operand
+// then needs ONE 16-byte LDS read per four MFMAs.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
@@ -24,19 +26,23 @@ namespace {
 
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 
-constexpr int BM = 128, BN = 128, BKT = 16;
+constexpr int BM = 128, BKT = 16;
 constexpr int kThreads = 256;
 constexpr int kRowKStride = BKT + 4;   // floats; 80 B rows keep 16-byte reads conflict free
-constexpr int kKRowStride = BM;        // floats
-constexpr int kTileFloats = BM * kRowKStride;  // 2560 >= BKT * kKRowStride (2048)
+// an operand tile has ROWS rows (128 or 256) and BKT k-values; k-row tiles use ROWS floats per k
+template <int ROWS>
+struct Tile {
+    static constexpr int pieces = ROWS * BKT / 4 / kThreads;  // 16-byte pieces per thread
+    static constexpr int floats = ROWS * kRowKStride;          // >= BKT * ROWS
+};
 
 // ---- global -> registers -------------------------------------------------------------------
 
-template <bool KMAJOR, bool ALIGNED>
+template <bool KMAJOR, bool ALIGNED, int ROWS>
 __device__ __forceinline__ void load_tile(const float* __restrict__ p, uint64_t ld, uint64_t x0, uint64_t X,
-                                          uint64_t k0, uint64_t K, int tid, float4 (&r)[2]) {
+                                          uint64_t k0, uint64_t K, int tid, float4 (&r)[Tile<ROWS>::pieces]) {
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
+    for (int i = 0; i < Tile<ROWS>::pieces; ++i) {
         const int id = tid + kThreads * i;
         float4 v = {0.f, 0.f, 0.f, 0.f};
         if (!KMAJOR) {
@@ -53,7 +59,7 @@ __device__ __forceinline__ void load_tile(const float* __restrict__ p, uint64_t 
                 }
             }
         } else {
-            const uint64_t k = k0 + (id >> 5), x = x0 + 4 * (id & 31);
+            const uint64_t k = k0 + id / (ROWS / 4), x = x0 + 4 * (id % (ROWS / 4));
             if (k < K && x < X) {
                 const float* q = p + k * ld + x;
                 if (ALIGNED && x + 4 <= X) {
@@ -70,39 +76,40 @@ __device__ __forceinline__ void load_tile(const float* __restrict__ p, uint64_t 
     }
 }
 
-template <bool KMAJOR>
-__device__ __forceinline__ void store_tile(float* lds, int tid, const float4 (&r)[2]) {
+template <bool KMAJOR, int ROWS>
+__device__ __forceinline__ void store_tile(float* lds, int tid, const float4 (&r)[Tile<ROWS>::pieces]) {
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
+    for (int i = 0; i < Tile<ROWS>::pieces; ++i) {
         const int id = tid + kThreads * i;
         if (!KMAJOR)
             *reinterpret_cast<float4*>(lds + (id >> 2) * kRowKStride + 4 * (id & 3)) = r[i];
         else
-            *reinterpret_cast<float4*>(lds + (id >> 5) * kKRowStride + 4 * (id & 31)) = r[i];
+            *reinterpret_cast<float4*>(lds + (id / (ROWS / 4)) * ROWS + 4 * (id % (ROWS / 4))) = r[i];
     }
 }
 
 // The 4 operand values (t = 0..3) of lane (x, h) for sub-step s.
-template <bool KMAJOR>
+template <bool KMAJOR, int ROWS>
 __device__ __forceinline__ float4 read_frag(const float* lds, int x, int h, int s) {
     if (!KMAJOR) return *reinterpret_cast<const float4*>(lds + x * kRowKStride + 8 * s + 4 * h);
-    const float* q = lds + (8 * s + 4 * h) * kKRowStride + x;
+    const float* q = lds + (8 * s + 4 * h) * ROWS + x;
     float4 v;
     v.x = q[0];
-    v.y = q[kKRowStride];
-    v.z = q[2 * kKRowStride];
-    v.w = q[3 * kKRowStride];
+    v.y = q[ROWS];
+    v.z = q[2 * ROWS];
+    v.w = q[3 * ROWS];
     return v;
 }
 
-template <bool AK, bool BK, bool ALIGNED>
+template <bool AK, bool BK, bool ALIGNED, int WN>
 __global__ __launch_bounds__(kThreads, 2) void gemm_kernel(const float* __restrict__ A, uint64_t lda,
                                                            const float* __restrict__ B, uint64_t ldb,
                                                            float* __restrict__ C, uint64_t ldc, uint64_t M,
                                                            uint64_t N, uint64_t K, float alpha, float beta,
                                                            const float* __restrict__ row_scale,
                                                            uint32_t tiles_n) {
-    __shared__ __attribute__((aligned(16))) float lds[2][2][kTileFloats];
+    constexpr int BN = 64 * WN;  // two waves side by side, WN 32-column MFMA tiles each
+    __shared__ __attribute__((aligned(16))) float lds[2][Tile<BM>::floats + Tile<BN>::floats];
 
     const uint32_t tile_m = blockIdx.x / tiles_n, tile_n = blockIdx.x % tiles_n;
     const uint64_t m0 = (uint64_t)tile_m * BM, n0 = (uint64_t)tile_n * BN;
@@ -112,53 +119,53 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_kernel(const float* __restri
     const int wm = wave >> 1, wn = wave & 1;
     const int x = lane & 31, h = lane >> 5;
 
-    floatx16 acc[2][2];
+    floatx16 acc[2][WN];
 #pragma unroll
     for (int i = 0; i < 2; ++i)
 #pragma unroll
-        for (int j = 0; j < 2; ++j)
+        for (int j = 0; j < WN; ++j)
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
     const uint64_t nk = (K + BKT - 1) / BKT;
-    float4 ra[2], rb[2];
+    float4 ra[Tile<BM>::pieces], rb[Tile<BN>::pieces];
     if (nk) {
-        load_tile<AK, ALIGNED>(A, lda, m0, M, 0, K, tid, ra);
-        load_tile<BK, ALIGNED>(B, ldb, n0, N, 0, K, tid, rb);
-        store_tile<AK>(lds[0][0], tid, ra);
-        store_tile<BK>(lds[0][1], tid, rb);
+        load_tile<AK, ALIGNED, BM>(A, lda, m0, M, 0, K, tid, ra);
+        load_tile<BK, ALIGNED, BN>(B, ldb, n0, N, 0, K, tid, rb);
+        store_tile<AK, BM>(lds[0], tid, ra);
+        store_tile<BK, BN>(lds[0] + Tile<BM>::floats, tid, rb);
     }
     __syncthreads();
 
     for (uint64_t kt = 0; kt < nk; ++kt) {
         const int cur = (int)(kt & 1);
         if (kt + 1 < nk) {
-            load_tile<AK, ALIGNED>(A, lda, m0, M, (kt + 1) * BKT, K, tid, ra);
-            load_tile<BK, ALIGNED>(B, ldb, n0, N, (kt + 1) * BKT, K, tid, rb);
+            load_tile<AK, ALIGNED, BM>(A, lda, m0, M, (kt + 1) * BKT, K, tid, ra);
+            load_tile<BK, ALIGNED, BN>(B, ldb, n0, N, (kt + 1) * BKT, K, tid, rb);
         }
-        const float* as = lds[cur][0];
-        const float* bs = lds[cur][1];
+        const float* as = lds[cur];
+        const float* bs = lds[cur] + Tile<BM>::floats;
 #pragma unroll
-        for (int s = 0; s < 2; ++s) {
-            float4 fa[2], fb[2];
+        for (int s = 0; s < BKT / 8; ++s) {
+            float4 fa[2], fb[WN];
 #pragma unroll
-            for (int i = 0; i < 2; ++i) fa[i] = read_frag<AK>(as, wm * 64 + 32 * i + x, h, s);
+            for (int i = 0; i < 2; ++i) fa[i] = read_frag<AK, BM>(as, wm * 64 + 32 * i + x, h, s);
 #pragma unroll
-            for (int j = 0; j < 2; ++j) fb[j] = read_frag<BK>(bs, wn * 64 + 32 * j + x, h, s);
+            for (int j = 0; j < WN; ++j) fb[j] = read_frag<BK, BN>(bs, wn * (32 * WN) + 32 * j + x, h, s);
 #pragma unroll
             for (int t = 0; t < 4; ++t)
 #pragma unroll
                 for (int i = 0; i < 2; ++i)
 #pragma unroll
-                    for (int j = 0; j < 2; ++j) {
+                    for (int j = 0; j < WN; ++j) {
                         const float av = t == 0 ? fa[i].x : (t == 1 ? fa[i].y : (t == 2 ? fa[i].z : fa[i].w));
                         const float bv = t == 0 ? fb[j].x : (t == 1 ? fb[j].y : (t == 2 ? fb[j].z : fb[j].w));
                         acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(av, bv, acc[i][j], 0, 0, 0);
                     }
         }
         if (kt + 1 < nk) {
-            store_tile<AK>(lds[cur ^ 1][0], tid, ra);
-            store_tile<BK>(lds[cur ^ 1][1], tid, rb);
+            store_tile<AK, BM>(lds[cur ^ 1], tid, ra);
+            store_tile<BK, BN>(lds[cur ^ 1] + Tile<BM>::floats, tid, rb);
         }
         __syncthreads();
     }
@@ -173,8 +180,8 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_kernel(const float* __restri
             if (row >= M) continue;
             const float rs = row_scale ? row_scale[row] : 1.0f;
 #pragma unroll
-            for (int j = 0; j < 2; ++j) {
-                const uint64_t col = n0 + wn * 64 + 32 * j + x;
+            for (int j = 0; j < WN; ++j) {
+                const uint64_t col = n0 + wn * (32 * WN) + 32 * j + x;
                 if (col >= N) continue;
                 float* c = C + row * ldc + col;
                 float v = alpha * acc[i][j][r];
@@ -185,6 +192,23 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_kernel(const float* __restri
     }
 }
 
+template <bool AK, bool BK, int WN>
+int launch_tiles(const float* A, uint64_t lda, const float* B, uint64_t ldb, float* C, uint64_t ldc, uint64_t M,
+                 uint64_t N, uint64_t K, float alpha, float beta, const float* row_scale, bool aligned,
+                 hipStream_t s) {
+    constexpr int BN = 64 * WN;
+    const uint64_t tm = (M + BM - 1) / BM, tn = (N + BN - 1) / BN;
+    if (tm * tn > 0x7FFFFFFFull) return TRAKHIP_ERR_SHAPE;
+    const dim3 grid((uint32_t)(tm * tn)), block(kThreads);
+    if (aligned)
+        hipLaunchKernelGGL((gemm_kernel<AK, BK, true, WN>), grid, block, 0, s, A, lda, B, ldb, C, ldc, M, N, K, alpha,
+                           beta, row_scale, (uint32_t)tn);
+    else
+        hipLaunchKernelGGL((gemm_kernel<AK, BK, false, WN>), grid, block, 0, s, A, lda, B, ldb, C, ldc, M, N, K,
+                           alpha, beta, row_scale, (uint32_t)tn);
+    return hipGetLastError() == hipSuccess ? TRAKHIP_OK : TRAKHIP_ERR_LAUNCH;
+}
+
 template <bool AK, bool BK>
 int launch(const float* A, uint64_t lda, const float* B, uint64_t ldb, float* C, uint64_t ldc, uint64_t M,
            uint64_t N, uint64_t K, float alpha, float beta, const float* row_scale, hipStream_t s) {
@@ -192,18 +216,12 @@ int launch(const float* A, uint64_t lda, const float* B, uint64_t ldb, float* C,
     if (!A || !B || !C) return TRAKHIP_ERR_NULL;
     const uint64_t min_lda = AK ? M : K, min_ldb = BK ? N : K;
     if (lda < min_lda || ldb < min_ldb || ldc < N) return TRAKHIP_ERR_SHAPE;
-    const uint64_t tm = (M + BM - 1) / BM, tn = (N + BN - 1) / BN;
-    if (tm * tn > 0x7FFFFFFFull) return TRAKHIP_ERR_SHAPE;
     const bool aligned = (reinterpret_cast<uintptr_t>(A) % 16 == 0) && (reinterpret_cast<uintptr_t>(B) % 16 == 0) &&
                          (lda % 4 == 0) && (ldb % 4 == 0);
-    const dim3 grid((uint32_t)(tm * tn)), block(kThreads);
-    if (aligned)
-        hipLaunchKernelGGL((gemm_kernel<AK, BK, true>), grid, block, 0, s, A, lda, B, ldb, C, ldc, M, N, K, alpha,
-                           beta, row_scale, (uint32_t)tn);
-    else
-        hipLaunchKernelGGL((gemm_kernel<AK, BK, false>), grid, block, 0, s, A, lda, B, ldb, C, ldc, M, N, K, alpha,
-                           beta, row_scale, (uint32_t)tn);
-    return hipGetLastError() == hipSuccess ? TRAKHIP_OK : TRAKHIP_ERR_LAUNCH;
+    // the wide tile pays off once C has a few hundred 128 x 256 tiles; narrow C keeps 128 x 128
+    const bool wide = N >= 256 && ((M + BM - 1) / BM) * ((N + 255) / 256) >= 256;
+    if (wide) return launch_tiles<AK, BK, 4>(A, lda, B, ldb, C, ldc, M, N, K, alpha, beta, row_scale, aligned, s);
+    return launch_tiles<AK, BK, 2>(A, lda, B, ldb, C, ldc, M, N, K, alpha, beta, row_scale, aligned, s);
 }
 
 }  // namespace
