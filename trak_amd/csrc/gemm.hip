@@ -107,12 +107,17 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_kernel(const float* __restri
                                                            float* __restrict__ C, uint64_t ldc, uint64_t M,
                                                            uint64_t N, uint64_t K, float alpha, float beta,
                                                            const float* __restrict__ row_scale,
-                                                           uint32_t tiles_n) {
+                                                           uint32_t tiles_n, uint32_t flags) {
     constexpr int BN = 64 * WN;  // two waves side by side, WN 32-column MFMA tiles each
     __shared__ __attribute__((aligned(16))) float lds[2][Tile<BM>::floats + Tile<BN>::floats];
 
     const uint32_t tile_m = blockIdx.x / tiles_n, tile_n = blockIdx.x % tiles_n;
     const uint64_t m0 = (uint64_t)tile_m * BM, n0 = (uint64_t)tile_n * BN;
+    // tiles strictly above the diagonal are not needed by a caller that reads the lower triangle
+    if ((flags & trakhip::kGemmLowerTilesOnly) && n0 > m0 + BM - 1) return;
+    // both operands vanish for k < their row/column index (lower-triangular factors stored k-row):
+    // the sum starts at the larger of the tile origins
+    const uint64_t k_first = (flags & trakhip::kGemmKFromDiagonal) ? ((m0 > n0 ? m0 : n0) / BKT) : 0;
 
     const int tid = threadIdx.x;
     const int wave = tid >> 6, lane = tid & 63;
@@ -129,16 +134,16 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_kernel(const float* __restri
 
     const uint64_t nk = (K + BKT - 1) / BKT;
     float4 ra[Tile<BM>::pieces], rb[Tile<BN>::pieces];
-    if (nk) {
-        load_tile<AK, ALIGNED, BM>(A, lda, m0, M, 0, K, tid, ra);
-        load_tile<BK, ALIGNED, BN>(B, ldb, n0, N, 0, K, tid, rb);
+    if (k_first < nk) {
+        load_tile<AK, ALIGNED, BM>(A, lda, m0, M, k_first * BKT, K, tid, ra);
+        load_tile<BK, ALIGNED, BN>(B, ldb, n0, N, k_first * BKT, K, tid, rb);
         store_tile<AK, BM>(lds[0], tid, ra);
         store_tile<BK, BN>(lds[0] + Tile<BM>::floats, tid, rb);
     }
     __syncthreads();
 
-    for (uint64_t kt = 0; kt < nk; ++kt) {
-        const int cur = (int)(kt & 1);
+    for (uint64_t kt = k_first; kt < nk; ++kt) {
+        const int cur = (int)((kt - k_first) & 1);
         if (kt + 1 < nk) {
             load_tile<AK, ALIGNED, BM>(A, lda, m0, M, (kt + 1) * BKT, K, tid, ra);
             load_tile<BK, ALIGNED, BN>(B, ldb, n0, N, (kt + 1) * BKT, K, tid, rb);
@@ -195,23 +200,23 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_kernel(const float* __restri
 template <bool AK, bool BK, int WN>
 int launch_tiles(const float* A, uint64_t lda, const float* B, uint64_t ldb, float* C, uint64_t ldc, uint64_t M,
                  uint64_t N, uint64_t K, float alpha, float beta, const float* row_scale, bool aligned,
-                 hipStream_t s) {
+                 uint32_t flags, hipStream_t s) {
     constexpr int BN = 64 * WN;
     const uint64_t tm = (M + BM - 1) / BM, tn = (N + BN - 1) / BN;
     if (tm * tn > 0x7FFFFFFFull) return TRAKHIP_ERR_SHAPE;
     const dim3 grid((uint32_t)(tm * tn)), block(kThreads);
     if (aligned)
         hipLaunchKernelGGL((gemm_kernel<AK, BK, true, WN>), grid, block, 0, s, A, lda, B, ldb, C, ldc, M, N, K, alpha,
-                           beta, row_scale, (uint32_t)tn);
+                           beta, row_scale, (uint32_t)tn, flags);
     else
         hipLaunchKernelGGL((gemm_kernel<AK, BK, false, WN>), grid, block, 0, s, A, lda, B, ldb, C, ldc, M, N, K,
-                           alpha, beta, row_scale, (uint32_t)tn);
+                           alpha, beta, row_scale, (uint32_t)tn, flags);
     return hipGetLastError() == hipSuccess ? TRAKHIP_OK : TRAKHIP_ERR_LAUNCH;
 }
 
 template <bool AK, bool BK>
 int launch(const float* A, uint64_t lda, const float* B, uint64_t ldb, float* C, uint64_t ldc, uint64_t M,
-           uint64_t N, uint64_t K, float alpha, float beta, const float* row_scale, hipStream_t s) {
+           uint64_t N, uint64_t K, float alpha, float beta, const float* row_scale, uint32_t flags, hipStream_t s) {
     if (M == 0 || N == 0) return TRAKHIP_OK;
     if (!A || !B || !C) return TRAKHIP_ERR_NULL;
     const uint64_t min_lda = AK ? M : K, min_ldb = BK ? N : K;
@@ -220,8 +225,9 @@ int launch(const float* A, uint64_t lda, const float* B, uint64_t ldb, float* C,
                          (lda % 4 == 0) && (ldb % 4 == 0);
     // the wide tile pays off once C has a few hundred 128 x 256 tiles; narrow C keeps 128 x 128
     const bool wide = N >= 256 && ((M + BM - 1) / BM) * ((N + 255) / 256) >= 256;
-    if (wide) return launch_tiles<AK, BK, 4>(A, lda, B, ldb, C, ldc, M, N, K, alpha, beta, row_scale, aligned, s);
-    return launch_tiles<AK, BK, 2>(A, lda, B, ldb, C, ldc, M, N, K, alpha, beta, row_scale, aligned, s);
+    if (wide)
+        return launch_tiles<AK, BK, 4>(A, lda, B, ldb, C, ldc, M, N, K, alpha, beta, row_scale, aligned, flags, s);
+    return launch_tiles<AK, BK, 2>(A, lda, B, ldb, C, ldc, M, N, K, alpha, beta, row_scale, aligned, flags, s);
 }
 
 }  // namespace
@@ -229,18 +235,18 @@ int launch(const float* A, uint64_t lda, const float* B, uint64_t ldb, float* C,
 namespace trakhip {
 
 int gemm_nt(const float* A, uint64_t lda, const float* B, uint64_t ldb, float* C, uint64_t ldc, uint64_t M,
-            uint64_t N, uint64_t K, float alpha, float beta, const float* row_scale, hipStream_t s) {
-    return launch<false, false>(A, lda, B, ldb, C, ldc, M, N, K, alpha, beta, row_scale, s);
+            uint64_t N, uint64_t K, float alpha, float beta, const float* row_scale, hipStream_t s, uint32_t flags) {
+    return launch<false, false>(A, lda, B, ldb, C, ldc, M, N, K, alpha, beta, row_scale, flags, s);
 }
 
 int gemm_tn(const float* A, uint64_t lda, const float* B, uint64_t ldb, float* C, uint64_t ldc, uint64_t M,
-            uint64_t N, uint64_t K, float alpha, float beta, hipStream_t s) {
-    return launch<true, true>(A, lda, B, ldb, C, ldc, M, N, K, alpha, beta, nullptr, s);
+            uint64_t N, uint64_t K, float alpha, float beta, hipStream_t s, uint32_t flags) {
+    return launch<true, true>(A, lda, B, ldb, C, ldc, M, N, K, alpha, beta, nullptr, flags, s);
 }
 
 int gemm_nn(const float* A, uint64_t lda, const float* B, uint64_t ldb, float* C, uint64_t ldc, uint64_t M,
-            uint64_t N, uint64_t K, float alpha, float beta, hipStream_t s) {
-    return launch<false, true>(A, lda, B, ldb, C, ldc, M, N, K, alpha, beta, nullptr, s);
+            uint64_t N, uint64_t K, float alpha, float beta, hipStream_t s, uint32_t flags) {
+    return launch<false, true>(A, lda, B, ldb, C, ldc, M, N, K, alpha, beta, nullptr, flags, s);
 }
 
 }  // namespace trakhip

@@ -45,12 +45,15 @@ __global__ __launch_bounds__(256) void spd_init_kernel(const float* __restrict__
 // One workgroup of 1024 threads: Cholesky of the 128x128 diagonal block at W (lower triangle
 // used), L block to Lout (upper part zero), its inverse to Linv_out.
 //
-// Thread (ty, tx) of a 32 x 32 grid keeps the elements (ty + 32 i, tx + 32 j), i, j < 4, of the
-// block in registers (cyclic ownership keeps every thread busy as the active part shrinks; four
-// waves per SIMD hide the issue latency of this strictly sequential algorithm).  Step k of the
-// right-looking factorization broadcasts column k of L through LDS and applies the rank-1 update
-// A -= l l^T from registers; the inverse runs the same way on B = I:
-// X[k, :] = B[k, :] / L[k, k], then B[r, :] -= L[r, k] X[k, :] for r > k.
+// The block lives in registers, 4 x 4 elements per thread, cyclically distributed so that every
+// thread stays busy as the active part shrinks (four waves per SIMD hide the issue latency of this
+// strictly sequential algorithm).  Step k of the right-looking factorization broadcasts column k
+// of L through LDS and applies the rank-1 update A -= l l^T from registers; the inverse runs the
+// same way on B = I:  X[k, :] = B[k, :] / L[k, k], then B[r, :] -= L[r, k] X[k, :] for r > k.
+// Ownership is chosen so that the threads that publish a column (factorization) or a row
+// (inverse) form half of ONE wave: thread t holds rows t % 32 + 32 i and columns t / 32 + 32 j
+// while factoring, and the transpose of that while inverting.  Updates are not masked: entries of
+// rows or columns <= k are never read again once step k is over, so what lands there is ignored.
 constexpr int kDiagGrid = 32;              // threads per side
 constexpr int kDiagTile = NB / kDiagGrid;  // 4 elements per side per thread
 
@@ -63,60 +66,61 @@ __global__ __launch_bounds__(1024) void spd_diag_kernel(const float* __restrict_
     __shared__ float vec[2][NB];     // broadcast buffers (two, so the steps can overlap safely)
     __shared__ float pivot[2];
     const int tid = threadIdx.x;
-    const int ty = tid / G, tx = tid % G;
+    const int p = tid % G, q = tid / G;  // p varies inside a half-wave, q selects the half-wave
 
+    // ---- factorization: rows p + G i, columns q + G j ------------------------------------------
     float a[T][T];
 #pragma unroll
     for (int i = 0; i < T; ++i)
 #pragma unroll
         for (int j = 0; j < T; ++j) {
-            const int r = ty + G * i, c = tx + G * j;
+            const int r = p + G * i, c = q + G * j;
             a[i][j] = (c <= r) ? W[(uint64_t)r * ldw + c] : 0.0f;
         }
 
-    // ---- factorization -------------------------------------------------------------------
     for (int k = 0; k < NB; ++k) {
         const int buf = k & 1;
-        const int ki = k / G, kt = k % G;  // element (k, k) lives in thread (kt, kt), slot [ki][ki]
-        if (ty == kt && tx == kt) {
-            float d = 0.0f;
-#pragma unroll
-            for (int i = 0; i < T; ++i)
-                if (i == ki) d = a[i][i];
-            if (!(d > 0.0f)) {
-                if (status && *status == 0) *status = 1 + block_index * NB + k;
-                d = 1.0f;
-            }
-            pivot[buf] = sqrtf(d);
-        }
-        __syncthreads();
-        const float sd = pivot[buf];
-        if (tx == kt) {  // owners of column k: scale and publish it
-            const float inv_sd = 1.0f / sd;
+        const int ks = k / G, kt = k % G;  // column k: threads with q == kt, slot [*][ks]
+        if (q == kt) {                     // one half-wave
+            float col[T];
 #pragma unroll
             for (int i = 0; i < T; ++i) {
-                const int r = ty + G * i;
-                float v = 0.0f;
+                col[i] = 0.0f;
 #pragma unroll
                 for (int j = 0; j < T; ++j)
-                    if (j == ki) v = a[i][j];
-                const float l = (r > k) ? v * inv_sd : (r == k ? sd : 0.0f);
-                vec[buf][r] = l;
-                Ls[r * kLd + k] = l;
+                    if (j == ks) col[i] = a[i][j];
             }
+            if (p == kt) {  // the diagonal element (k, k) is in slot [ks][ks] of this thread
+                float d = 0.0f;
+#pragma unroll
+                for (int i = 0; i < T; ++i)
+                    if (i == ks) d = col[i];
+                if (!(d > 0.0f)) {
+                    if (status && *status == 0) *status = 1 + block_index * NB + k;
+                    d = 1.0f;
+                }
+                pivot[buf] = d;
+            }
+#pragma unroll
+            for (int i = 0; i < T; ++i) vec[buf][p + G * i] = col[i];  // unscaled column
         }
         __syncthreads();
+        const float d = pivot[buf];
+        const float inv_d = 1.0f / d;
+        if (q == kt) {  // the finished column of L, off the critical path of the other waves
+            const float inv_sd = 1.0f / sqrtf(d);
+#pragma unroll
+            for (int i = 0; i < T; ++i) {
+                const int r = p + G * i;
+                Ls[r * kLd + k] = (r >= k) ? vec[buf][r] * inv_sd : 0.0f;  // L[k][k] = d / sqrt(d)
+            }
+        }
+        // A[r][c] -= raw[r] * raw[c] / d
         float lr[T], lc[T];
 #pragma unroll
-        for (int i = 0; i < T; ++i) {
-            const int r = ty + G * i;
-            lr[i] = (r > k) ? vec[buf][r] : 0.0f;
-        }
+        for (int i = 0; i < T; ++i) lr[i] = vec[buf][p + G * i];
 #pragma unroll
-        for (int j = 0; j < T; ++j) {
-            const int c = tx + G * j;
-            lc[j] = (c > k) ? vec[buf][c] : 0.0f;
-        }
+        for (int j = 0; j < T; ++j) lc[j] = vec[buf][q + G * j] * inv_d;
 #pragma unroll
         for (int i = 0; i < T; ++i)
 #pragma unroll
@@ -124,40 +128,41 @@ __global__ __launch_bounds__(1024) void spd_diag_kernel(const float* __restrict_
     }
     __syncthreads();
 
-    // ---- inverse of L ---------------------------------------------------------------------
+    // ---- inverse of L: rows q + G i, columns p + G j (transposed ownership) --------------------
     float b[T][T];
 #pragma unroll
     for (int i = 0; i < T; ++i)
 #pragma unroll
-        for (int j = 0; j < T; ++j) b[i][j] = (ty + G * i == tx + G * j) ? 1.0f : 0.0f;
+        for (int j = 0; j < T; ++j) b[i][j] = (q + G * i == p + G * j) ? 1.0f : 0.0f;
 
     for (int k = 0; k < NB; ++k) {
         const int buf = k & 1;
-        const int ki = k / G, kt = k % G;
-        if (ty == kt) {  // owners of row k: X[k, c] = B[k, c] / L[k, k]
+        const int ks = k / G, kt = k % G;  // row k: threads with q == kt, slot [ks][*]
+        if (q == kt) {
             const float inv_d = 1.0f / Ls[k * kLd + k];
 #pragma unroll
             for (int j = 0; j < T; ++j) {
                 float v = 0.0f;
 #pragma unroll
                 for (int i = 0; i < T; ++i)
-                    if (i == ki) v = b[i][j];
+                    if (i == ks) v = b[i][j];
                 v *= inv_d;
 #pragma unroll
                 for (int i = 0; i < T; ++i)
-                    if (i == ki) b[i][j] = v;
-                vec[buf][tx + G * j] = v;
+                    if (i == ks) b[i][j] = v;
+                vec[buf][p + G * j] = v;
             }
         }
         __syncthreads();
+        // B[r][c] -= L[r][k] * X[k][c] for r > k (rows <= k keep their finished values)
         float lr[T], xc[T];
 #pragma unroll
         for (int i = 0; i < T; ++i) {
-            const int r = ty + G * i;
+            const int r = q + G * i;
             lr[i] = (r > k) ? Ls[r * kLd + k] : 0.0f;
         }
 #pragma unroll
-        for (int j = 0; j < T; ++j) xc[j] = vec[buf][tx + G * j];
+        for (int j = 0; j < T; ++j) xc[j] = vec[buf][p + G * j];
 #pragma unroll
         for (int i = 0; i < T; ++i)
 #pragma unroll
@@ -168,7 +173,7 @@ __global__ __launch_bounds__(1024) void spd_diag_kernel(const float* __restrict_
     for (int i = 0; i < T; ++i)
 #pragma unroll
         for (int j = 0; j < T; ++j) {
-            const int r = ty + G * i, c = tx + G * j;
+            const int r = q + G * i, c = p + G * j;
             Lout[(uint64_t)r * ldl + c] = (c <= r) ? Ls[r * kLd + c] : 0.0f;
             Linv_out[(uint64_t)r * ldl + c] = (c <= r) ? b[i][j] : 0.0f;
         }
@@ -288,7 +293,8 @@ int spd_inverse(const float* A, uint64_t lda, float lambda, float* inv, uint64_t
         if (e) return e;
         // trailing matrix -= panel * panel^T
         const uint64_t tr = (j + 1) * NB * np + (j + 1) * NB;
-        e = gemm_nt(L + below, np, L + below, np, W + tr, np, rows, rows, NB, -1.0f, 1.0f, nullptr, s);
+        e = gemm_nt(L + below, np, L + below, np, W + tr, np, rows, rows, NB, -1.0f, 1.0f, nullptr, s,
+                    kGemmLowerTilesOnly);  // only the lower triangle of W is ever read
         if (e) return e;
     }
 
@@ -297,7 +303,8 @@ int spd_inverse(const float* A, uint64_t lda, float lambda, float* inv, uint64_t
     if (c.err) return c.err;
 
     // inverse = Li^T * Li (rows of Li at or beyond n do not reach the leading n x n block)
-    int e = gemm_tn(Li, np, Li, np, inv, ldi, n, n, n, 1.0f, 0.0f, s);
+    // Li is lower triangular: Li[k][m] = 0 for k < m, so the sum over k starts at max(m, n)
+    int e = gemm_tn(Li, np, Li, np, inv, ldi, n, n, n, 1.0f, 0.0f, s, kGemmKFromDiagonal);
     if (e) return e;
 
     if (normalize || mean_abs) {

@@ -24,12 +24,17 @@ int materialize_device(uint32_t seed, uint32_t num_feature_tiles, uint64_t P, ui
 int materialize_host(uint32_t seed, uint32_t num_feature_tiles, uint64_t P, uint64_t f0, uint64_t nf,
                      uint32_t c0, uint32_t nc, int proj_type, float* out);
 
+// internal GEMM options (spd.hip)
+constexpr uint32_t kGemmLowerTilesOnly = 1u;  // skip output tiles strictly above the diagonal
+constexpr uint32_t kGemmKFromDiagonal = 2u;   // start the k sum at max(tile row origin, tile column origin)
+
 int gemm_nt(const float* A, uint64_t lda, const float* B, uint64_t ldb, float* C, uint64_t ldc, uint64_t M,
-            uint64_t N, uint64_t K, float alpha, float beta, const float* row_scale, hipStream_t s);
+            uint64_t N, uint64_t K, float alpha, float beta, const float* row_scale, hipStream_t s,
+            uint32_t flags = 0);
 int gemm_tn(const float* A, uint64_t lda, const float* B, uint64_t ldb, float* C, uint64_t ldc, uint64_t M,
-            uint64_t N, uint64_t K, float alpha, float beta, hipStream_t s);
+            uint64_t N, uint64_t K, float alpha, float beta, hipStream_t s, uint32_t flags = 0);
 int gemm_nn(const float* A, uint64_t lda, const float* B, uint64_t ldb, float* C, uint64_t ldc, uint64_t M,
-            uint64_t N, uint64_t K, float alpha, float beta, hipStream_t s);
+            uint64_t N, uint64_t K, float alpha, float beta, hipStream_t s, uint32_t flags = 0);
 size_t spd_inverse_workspace_bytes(uint64_t n);
 int spd_inverse(const float* A, uint64_t lda, float lambda, float* inv, uint64_t ldi, uint64_t n,
                 int normalize, float* mean_abs, int32_t* status, void* ws, size_t ws_bytes, hipStream_t s);
