@@ -248,6 +248,81 @@ def bench_other_configs(torch, dev):
     return res
 
 
+def bench_store_paths(torch, dev):
+    """The store-side epilogues against the reference's sequences of passes: one featurize batch at
+    the ResNet-18 shape down to host memory (trak/traker.py:425-429), and the score sums of three
+    checkpoints at N=50 000, M=10 000 down to a host array (trak/traker.py:641-678)."""
+    import numpy as np
+
+    from trak_amd import BasicScoreComputer, CudaProjector, FeatureWriter, ProjectionType, ScoreAccumulator
+
+    res = {}
+    P, k, B = 11_689_512, 4096, 32
+    proj = CudaProjector(P, k, 7, ProjectionType.rademacher, dev, 32)
+    gen = torch.Generator(device=dev).manual_seed(20_008)
+    g = (torch.randn(B, P, generator=gen, device=dev) * 1e-3).half()
+    nf = torch.sqrt(torch.tensor(float(P)))
+    store = np.zeros((64 * B, k), dtype=np.float16)
+
+    def reference_batch(i):
+        x = proj.project(g, 0)
+        x /= nf
+        store[i * B:(i + 1) * B] = x.to(torch.float16).cpu().clone().detach()
+
+    writer = FeatureWriter(proj, k, nf, dtype=torch.float16, max_batch_size=B, depth=2)
+
+    def fused_batch(i):
+        writer.write(g, 0, store, np.arange(i * B, (i + 1) * B))
+
+    for name, fn, done in (("reference_sequence", reference_batch, lambda: None),
+                           ("feature_writer", fused_batch, writer.flush)):
+        for i in range(4):
+            fn(i)
+        done()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for i in range(64):
+            fn(i)
+        done()
+        torch.cuda.synchronize()
+        res[f"featurize_batch_to_host_ms[{name}]"] = (time.perf_counter() - t0) * 1e3 / 64
+    del g
+
+    N, M, kk, models = 50_000, 10_000, 4096, 3
+    sc = BasicScoreComputer(dtype=torch.float32, device=dev)
+    f = torch.randn(N, kk, generator=gen, device=dev) / 64
+    t = torch.randn(M, kk, generator=gen, device=dev) / 64
+    o = np.random.default_rng(0).random((N, 1)).astype(np.float32)
+    out = np.zeros((N, M), dtype=np.float32)
+    for _ in range(2):  # second pass timed: the first touches the host pages
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        acc = torch.zeros(N, M)
+        osum = np.zeros((N, 1), dtype=np.float32)
+        for _m in range(models):
+            sc.get_scores(f, t, accumulator=acc)
+            osum += o
+        out[:] = (acc.numpy() / float(models)) * (osum / float(models))
+        ref_s = time.perf_counter() - t0
+    del acc
+    for _ in range(2):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        sa = ScoreAccumulator(sc, N, M)
+        for _m in range(models):
+            sa.add(f, t, o)
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+        sa.finalize(out)
+        t2 = time.perf_counter()
+        del sa
+    res["finalize_scores_3_checkpoints_s[reference_sequence]"] = ref_s
+    res["finalize_scores_3_checkpoints_s[score_accumulator]"] = t2 - t0
+    res["score_accumulator_finalize_only_s"] = t2 - t1
+    res["score_accumulator_finalize_GBps"] = N * M * 4 / (t2 - t1) / 1e9
+    return res
+
+
 def bench_scoring(torch, dev, reps=3):
     from trak_amd import BasicScoreComputer
 
@@ -359,6 +434,8 @@ def main():
         print(json.dumps(bench_other_configs(torch, dev), indent=1), file=sys.stderr)
         print(json.dumps({"featurize_path": bench_featurize_path(torch, dev)}, indent=1), file=sys.stderr)
         print(json.dumps({"batch_scaling": bench_batch_scaling(torch, dev)}, indent=1), file=sys.stderr)
+        torch.cuda.empty_cache()
+        print(json.dumps({"store_paths": bench_store_paths(torch, dev)}, indent=1), file=sys.stderr)
         torch.cuda.empty_cache()
     scoring = None if args.no_scoring else bench_scoring(torch, dev)
     torch.cuda.empty_cache()

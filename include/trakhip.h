@@ -41,6 +41,7 @@ extern "C" {
 #define TRAKHIP_ERR_LAUNCH -8    /* HIP refused the launch (hipGetLastError != hipSuccess) */
 #define TRAKHIP_ERR_NOT_SPD -9   /* matrix handed to the SPD inverse is not positive definite */
 #define TRAKHIP_ERR_NO_DEVICE -10
+#define TRAKHIP_ERR_POINTER -11  /* destination is neither device memory nor page-locked host memory */
 
 const char* trakhip_strerror(int code);
 
@@ -78,6 +79,19 @@ int trakhip_project_partials(const void* in_dev, int in_dtype, uint64_t B, uint6
                              uint32_t num_feature_tiles, int proj_type, void* stream);
 int trakhip_project_reduce(const void* workspace_dev, uint64_t B, uint64_t P, uint32_t proj_dim,
                            uint32_t num_feature_tiles, float scale, float* out_dev, void* stream);
+
+/* Phase 2 with the rest of TRAKer.featurize's epilogue folded in: out[b, c] = cast((sum of the
+ * partials) * scale), i.e. `grads /= normalize_factor; grads.to(dtype)` of trak/traker.py:426-428
+ * (torch divides by a scalar as a multiplication by its fp32 reciprocal, so scale = 1.0f / sqrt(P)
+ * gives the same bits), written with row pitch ld_out (elements) either to device memory or
+ * straight into page-locked host memory (hipHostMalloc / torch pin_memory) - the staging buffer
+ * of the `grads` store rows of trak/savers.py:406-410, which replaces the `.cpu()` copy.
+ *   out_dtype   TRAKHIP_F16 | TRAKHIP_BF16 | TRAKHIP_F32 (round to nearest even)
+ *   out         aligned to four elements, ld_out >= proj_dim and a multiple of 4; pageable host
+ *               memory is refused with TRAKHIP_ERR_POINTER */
+int trakhip_project_reduce_store(const void* workspace_dev, uint64_t B, uint64_t P, uint32_t proj_dim,
+                                 uint32_t num_feature_tiles, float scale, int out_dtype, void* out,
+                                 uint64_t ld_out, void* stream);
 
 /* One piece of a gradient that is stored as a list of tensors (one per model parameter): features
  * [first, first + numel) of every row live at ptr[row * ld + (feature - first)]. */
@@ -121,6 +135,17 @@ int trakhip_gemm_nt(const float* A_dev, uint64_t lda, const float* B_dev, uint64
 int trakhip_gemm_tn(const float* A_dev, uint64_t lda, const float* B_dev, uint64_t ldb, float* C_dev,
                     uint64_t ldc, uint64_t M, uint64_t N, uint64_t K, float alpha, float beta,
                     void* stream);
+
+/* out[i, j] = cast((acc[i, j] / divisor) * row_factor[i]) for the [N, M] fp32 score sums that
+ * trakhip_gemm_nt accumulated over checkpoints (beta = 1): the closing expression of
+ * TRAKer.finalize_scores, `(_scores / n) * (_avg_out_to_losses / n)` (trak/traker.py:670-678), with
+ * divisor = n and row_factor[i] = the second factor, two correctly rounded fp32 operations in that
+ * order, then the cast to the store's type (TRAKHIP_F16 | TRAKHIP_BF16 | TRAKHIP_F32).  `out` is device
+ * memory or page-locked host memory (pageable host memory: TRAKHIP_ERR_POINTER), so the score
+ * matrix crosses PCIe once, after the last checkpoint.  row_factor_dev may be NULL (factor 1). */
+int trakhip_scores_finalize(const float* acc_dev, uint64_t ld_acc, uint64_t N, uint64_t M, float divisor,
+                            const float* row_factor_dev, int out_dtype, void* out, uint64_t ld_out,
+                            void* stream);
 
 /* Bytes of scratch trakhip_spd_inverse needs for an n x n matrix. */
 size_t trakhip_spd_inverse_workspace(uint64_t n);

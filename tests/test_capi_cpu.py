@@ -34,7 +34,7 @@ def test_abi_version_and_strerror():
     assert _lib.strerror(0) == "success"
     # the text the reference throws at fast_jl/fast_jl_kernel.cuh:113-115
     assert _lib.strerror(-1) == "Invalid Number of JL dimensions it has to be a multiple of 512"
-    for code in range(-10, 0):
+    for code in range(-11, 0):
         assert "unknown trakhip error" not in _lib.strerror(code)
     assert "unknown trakhip error" in _lib.strerror(-999)
 
@@ -101,3 +101,30 @@ def test_gemm_argument_validation_needs_no_device():
     assert lib.trakhip_gemm_tn(p, 2, p, 8, p, 8, 4, 4, 16, 1.0, 0.0, None) == -2          # lda < M
     assert lib.trakhip_spd_inverse(p, 2, 0.0, p, 4, 4, 0, None, None, p, 1 << 30, None) == -2
     assert lib.trakhip_spd_inverse(p, 4, 0.0, p, 4, 4, 0, None, None, p, 16, None) == -6
+
+
+def test_store_entry_points_validate_before_touching_the_device():
+    lib = _lib.load()
+    p = ctypes.c_void_p(4096)
+    red = lambda **kw: lib.trakhip_project_reduce_store(
+        kw.get("ws", p), kw.get("B", 8), kw.get("P", 1000), kw.get("k", 512), kw.get("tiles", 256), 1.0,
+        kw.get("dt", 0), kw.get("out", p), kw.get("ld", 512), None)
+    assert red(k=100) == -1
+    assert red(B=0) == -2 and red(B=33) == -2 and red(ld=508) == -2 and red(P=0) == -2
+    assert red(dt=3) == -3
+    assert red(ws=None) == -5 and red(out=None) == -5
+    assert red(out=ctypes.c_void_p(4100)) == -7 and red(ld=514) == -7
+    assert red(dt=2, out=ctypes.c_void_p(4104)) == -7
+    # a pointer HIP knows nothing about (pageable host memory, here an arbitrary address) is
+    # refused on the host instead of faulting the GPU
+    assert red() == -11
+    fin = lambda **kw: lib.trakhip_scores_finalize(
+        kw.get("acc", p), kw.get("lda", 8), kw.get("N", 4), kw.get("M", 8), kw.get("div", 2.0), None,
+        kw.get("dt", 2), kw.get("out", p), kw.get("ldo", 8), None)
+    assert fin(dt=5) == -3
+    assert fin(lda=7) == -2 and fin(ldo=7) == -2 and fin(div=0.0) == -2
+    assert fin(N=0) == 0 and fin(M=0, lda=0, ldo=0) == 0
+    assert fin(acc=None) == -5 and fin(out=None) == -5
+    assert fin(acc=ctypes.c_void_p(4098)) == -7 and fin(dt=0, out=ctypes.c_void_p(4097)) == -7
+    assert fin() == -11
+    assert "page-locked" in _lib.strerror(-11)

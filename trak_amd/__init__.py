@@ -11,7 +11,9 @@ from .projectors import (
     NoOpProjector,
     ProjectionType,
 )
-from .score_computers import AbstractScoreComputer, BasicScoreComputer
+from .featurize import FeatureWriter
+from .savers import AbstractSaver, MmapSaver, ModelIDException
+from .score_computers import AbstractScoreComputer, BasicScoreComputer, ScoreAccumulator
 from .utils import get_matrix_mult, get_parameter_chunk_sizes, vectorize
 
 __all__ = [
@@ -23,6 +25,11 @@ __all__ = [
     "ProjectionType",
     "AbstractScoreComputer",
     "BasicScoreComputer",
+    "ScoreAccumulator",
+    "FeatureWriter",
+    "AbstractSaver",
+    "MmapSaver",
+    "ModelIDException",
     "get_matrix_mult",
     "get_parameter_chunk_sizes",
     "vectorize",

@@ -48,6 +48,10 @@ def load():
     lib.trakhip_project_gather_partials.restype = i32
     lib.trakhip_project_reduce.argtypes = [vp, u64, u64, u32, u32, f32, vp, vp]
     lib.trakhip_project_reduce.restype = i32
+    lib.trakhip_project_reduce_store.argtypes = [vp, u64, u64, u32, u32, f32, i32, vp, u64, vp]
+    lib.trakhip_project_reduce_store.restype = i32
+    lib.trakhip_scores_finalize.argtypes = [vp, u64, u64, u64, f32, vp, i32, vp, u64, vp]
+    lib.trakhip_scores_finalize.restype = i32
     lib.trakhip_materialize.argtypes = [u32, u32, u64, u64, u64, u32, u32, i32, vp, i32, vp]
     lib.trakhip_materialize.restype = i32
     lib.trakhip_gemm_nt.argtypes = [vp, u64, vp, u64, vp, u64, u64, u64, u64, f32, f32, vp, vp]

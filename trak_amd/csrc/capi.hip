@@ -17,6 +17,8 @@ const char* trakhip_strerror(int code) {
         case TRAKHIP_ERR_LAUNCH: return "HIP kernel launch failed";
         case TRAKHIP_ERR_NOT_SPD: return "matrix is not positive definite";
         case TRAKHIP_ERR_NO_DEVICE: return "no HIP device";
+        case TRAKHIP_ERR_POINTER:
+            return "destination is neither device memory nor page-locked host memory";
         default: return "unknown trakhip error";
     }
 }
@@ -53,6 +55,20 @@ int trakhip_project_reduce(const void* workspace_dev, uint64_t B, uint64_t P, ui
                            uint32_t num_feature_tiles, float scale, float* out_dev, void* stream) {
     return trakhip::project_reduce(workspace_dev, B, P, proj_dim, num_feature_tiles, scale, out_dev,
                                    static_cast<hipStream_t>(stream));
+}
+
+int trakhip_project_reduce_store(const void* workspace_dev, uint64_t B, uint64_t P, uint32_t proj_dim,
+                                 uint32_t num_feature_tiles, float scale, int out_dtype, void* out,
+                                 uint64_t ld_out, void* stream) {
+    return trakhip::project_reduce_store(workspace_dev, B, P, proj_dim, num_feature_tiles, scale, out_dtype, out,
+                                         ld_out, static_cast<hipStream_t>(stream), true);
+}
+
+int trakhip_scores_finalize(const float* acc_dev, uint64_t ld_acc, uint64_t N, uint64_t M, float divisor,
+                            const float* row_factor_dev, int out_dtype, void* out, uint64_t ld_out,
+                            void* stream) {
+    return trakhip::scores_finalize(acc_dev, ld_acc, N, M, divisor, row_factor_dev, out_dtype, out, ld_out,
+                                    static_cast<hipStream_t>(stream));
 }
 
 int trakhip_materialize(uint32_t seed, uint32_t num_feature_tiles, uint64_t P, uint64_t f0, uint64_t nf,

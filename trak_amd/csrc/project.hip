@@ -26,9 +26,12 @@
 #include <stdint.h>
 
 #include "jl_stream.h"
+#include "store_cast.h"
 #include "trakhip_internal.h"
 
 namespace {
+
+using trakhip::store4;
 
 typedef _Float16 half8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
@@ -593,9 +596,11 @@ __global__ __launch_bounds__(kThreads, 2) void jl_project_kernel(
 }
 
 // out[b, c] = scale * sum over tile groups, in group order.
+template <int OUT_DTYPE>
 __global__ __launch_bounds__(256) void jl_reduce_kernel(const float* __restrict__ partial,
-                                                        uint32_t groups, uint64_t n4, float scale,
-                                                        float* __restrict__ out) {
+                                                        uint32_t groups, uint64_t n4, uint32_t k4,
+                                                        float scale, void* __restrict__ out,
+                                                        uint64_t ld_out) {
     const uint64_t i = (uint64_t)blockIdx.x * 256 + threadIdx.x;
     if (i >= n4) return;
     const float4* p = reinterpret_cast<const float4*>(partial) + i;
@@ -636,7 +641,11 @@ __global__ __launch_bounds__(256) void jl_reduce_kernel(const float* __restrict_
     r.y *= scale;
     r.z *= scale;
     r.w *= scale;
-    reinterpret_cast<float4*>(out)[i] = r;
+    // row pitch of the destination in elements; the result is rounded to fp32 first (as a
+    // separate `x *= scale`), then to the store type
+    const uint64_t row = i / k4, c4 = i - row * k4;
+    const uint64_t e = row * ld_out + c4 * 4;
+    store4<OUT_DTYPE>(static_cast<char*>(out) + e * trakhip::out_elem_size(OUT_DTYPE), r);
 }
 
 // S[f0 + i, c0 + j] for i < nf, j < nc, written as binary32, row-major [nf, nc].
@@ -757,17 +766,35 @@ int project_gather_partials(const trakhip_segment* segs, uint32_t n_segs, int dt
     return TRAKHIP_OK;
 }
 
-int project_reduce(const void* ws, uint64_t B, uint64_t P, uint32_t k, uint32_t num_feature_tiles, float scale,
-                   float* out, hipStream_t s) {
+int project_reduce_store(const void* ws, uint64_t B, uint64_t P, uint32_t k, uint32_t num_feature_tiles,
+                         float scale, int out_dtype, void* out, uint64_t ld_out, hipStream_t s,
+                         bool check_destination) {
     if (k == 0 || k % kColsPerWG != 0) return TRAKHIP_ERR_PROJ_DIM;
-    if (B == 0 || B > 32 || P == 0 || P > 0xFFFFFFFFull || num_feature_tiles == 0) return TRAKHIP_ERR_SHAPE;
+    if (B == 0 || B > 32 || P == 0 || P > 0xFFFFFFFFull || num_feature_tiles == 0 || ld_out < k)
+        return TRAKHIP_ERR_SHAPE;
+    if (out_dtype != TRAKHIP_F16 && out_dtype != TRAKHIP_BF16 && out_dtype != TRAKHIP_F32) return TRAKHIP_ERR_DTYPE;
     if (!ws || !out) return TRAKHIP_ERR_NULL;
-    if ((reinterpret_cast<uintptr_t>(ws) % 16) || (reinterpret_cast<uintptr_t>(out) % 16)) return TRAKHIP_ERR_ALIGN;
+    const size_t quad = 4 * out_elem_size(out_dtype);
+    if ((reinterpret_cast<uintptr_t>(ws) % 16) || (reinterpret_cast<uintptr_t>(out) % quad) || (ld_out % 4))
+        return TRAKHIP_ERR_ALIGN;
+    if (check_destination && !kernel_can_write(out)) return TRAKHIP_ERR_POINTER;
     const uint32_t groups = make_plan(P, k, num_feature_tiles).groups;
     const uint64_t n4 = B * k / 4;
-    hipLaunchKernelGGL(jl_reduce_kernel, dim3((uint32_t)((n4 + 255) / 256)), dim3(256), 0, s,
-                       static_cast<const float*>(ws), groups, n4, scale, out);
+    const dim3 grid((uint32_t)((n4 + 255) / 256)), block(256);
+    const float* part = static_cast<const float*>(ws);
+    if (out_dtype == TRAKHIP_F32)
+        hipLaunchKernelGGL(jl_reduce_kernel<TRAKHIP_F32>, grid, block, 0, s, part, groups, n4, k / 4, scale, out, ld_out);
+    else if (out_dtype == TRAKHIP_F16)
+        hipLaunchKernelGGL(jl_reduce_kernel<TRAKHIP_F16>, grid, block, 0, s, part, groups, n4, k / 4, scale, out, ld_out);
+    else
+        hipLaunchKernelGGL(jl_reduce_kernel<TRAKHIP_BF16>, grid, block, 0, s, part, groups, n4, k / 4, scale, out, ld_out);
     return hipGetLastError() == hipSuccess ? TRAKHIP_OK : TRAKHIP_ERR_LAUNCH;
+}
+
+int project_reduce(const void* ws, uint64_t B, uint64_t P, uint32_t k, uint32_t num_feature_tiles, float scale,
+                   float* out, hipStream_t s) {
+    if (out && reinterpret_cast<uintptr_t>(out) % 16) return TRAKHIP_ERR_ALIGN;
+    return project_reduce_store(ws, B, P, k, num_feature_tiles, scale, TRAKHIP_F32, out, k, s, false);
 }
 
 int project(const void* in, int dtype, uint64_t B, uint64_t P, uint64_t ld, float* out, void* ws,

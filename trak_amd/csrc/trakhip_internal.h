@@ -19,6 +19,12 @@ int project_gather_partials(const trakhip_segment* segs, uint32_t n_segs, int dt
                             int proj_type, hipStream_t s);
 int project_reduce(const void* ws, uint64_t B, uint64_t P, uint32_t k, uint32_t num_feature_tiles, float scale,
                    float* out, hipStream_t s);
+int project_reduce_store(const void* ws, uint64_t B, uint64_t P, uint32_t k, uint32_t num_feature_tiles,
+                         float scale, int out_dtype, void* out, uint64_t ld_out, hipStream_t s,
+                         bool check_destination);
+int scores_finalize(const float* acc, uint64_t ld_acc, uint64_t N, uint64_t M, float divisor,
+                    const float* row_factor, int out_dtype, void* out, uint64_t ld_out, hipStream_t s);
+bool kernel_can_write(const void* p);
 int materialize_device(uint32_t seed, uint32_t num_feature_tiles, uint64_t P, uint64_t f0, uint64_t nf,
                        uint32_t c0, uint32_t nc, int proj_type, float* out, hipStream_t s);
 int materialize_host(uint32_t seed, uint32_t num_feature_tiles, uint64_t P, uint64_t f0, uint64_t nf,

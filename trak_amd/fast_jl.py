@@ -124,6 +124,91 @@ def gather_supported(tensors):
     )
 
 
+def _proj_type_code(proj_type):
+    return _lib.NORMAL if str(getattr(proj_type, "value", proj_type)) in ("normal", "1") else _lib.RADEMACHER
+
+
+def _check_destination(out, B, N, device):
+    """`out` receives [B, N] results: a CUDA tensor on `device`, or a page-locked CPU tensor that the
+    kernel writes over PCIe (pageable memory would fault the GPU, so it is refused here)."""
+    if not isinstance(out, torch.Tensor) or out.dim() != 2 or tuple(out.shape) != (B, N):
+        raise RuntimeError(f"out must be a [{B}, {N}] tensor")
+    if out.dtype not in _DTYPES:
+        raise RuntimeError("out must be fp16, bf16 or fp32")
+    if out.is_cuda:
+        if out.device != device:
+            raise RuntimeError("out must live on the input's device")
+    elif not out.is_pinned():
+        raise RuntimeError("a CPU destination must be page-locked (pin_memory)")
+    if out.stride(1) != 1 or (B > 1 and (out.stride(0) < N or out.stride(0) % 4)):
+        raise RuntimeError("out rows must be contiguous with a pitch that is a multiple of 4 elements")
+
+
+def project_into(source, N, seed, num_feature_tiles, proj_type, out, scale=1.0):
+    """out[B, N] = cast(project(source) * scale): the projection with the epilogue of
+    TRAKer.featurize (`grads /= normalize_factor; grads.to(dtype).cpu()`, trak/traker.py:426-428)
+    folded into the cross-tile sum.  `source` is a 2-D CUDA tensor [B, P] or a list of per-parameter
+    gradient tensors [B, ...] (projected in place, as `project_gather`); `out` is a CUDA tensor or a
+    page-locked CPU tensor (fp16 / bf16 / fp32), written on the current stream: synchronize (or
+    wait on an event recorded after this call) before reading a CPU destination."""
+    lib = _lib.load()
+    N, seed, tiles = int(N), int(seed) & 0xFFFFFFFF, int(num_feature_tiles)
+    if N <= 0 or N % 512 != 0:
+        _lib.check(_lib.ERR_PROJ_DIM)
+    pt = _proj_type_code(proj_type)
+    if isinstance(source, torch.Tensor):
+        if not source.is_cuda or source.dim() != 2 or source.dtype not in _DTYPES:
+            raise RuntimeError("input must be a 2D CUDA tensor of fp16, bf16 or fp32")
+        if source.shape[1] > 1 and source.stride(1) != 1:
+            raise RuntimeError("input must be contiguous")
+        B, P = source.shape
+        ld = source.stride(0) if B > 1 else max(P, 1)
+        if ld < P:
+            raise RuntimeError("input must be contiguous")
+        device, dtype, esz = source.device, source.dtype, source.element_size()
+        rows = None
+    else:
+        tensors = list(source)
+        if not gather_supported(tensors):
+            raise RuntimeError("project_into needs CUDA tensors of one supported dtype, device and batch size")
+        flats = [_flat_rows(t) for t in tensors]
+        device, dtype, esz = flats[0].device, flats[0].dtype, flats[0].element_size()
+        B = flats[0].shape[0]
+        rows, first = [], 0
+        for f in flats:
+            numel = f.shape[1]
+            rows.append([f.data_ptr(), first, numel, f.stride(0) if B > 1 else numel])
+            first += numel
+        P = first
+    _check_destination(out, B, N, device)
+    out_ld = out.stride(0) if B > 1 else N
+    with torch.cuda.device(device):
+        nbytes = lib.trakhip_project_workspace(B, P, N, tiles)
+        ws = _workspace(device, nbytes)
+        stream = torch.cuda.current_stream(device).cuda_stream
+        for b0 in range(0, B, 32):
+            nb = min(32, B - b0)
+            if rows is None:
+                code = lib.trakhip_project_partials(
+                    ctypes.c_void_p(source.data_ptr() + b0 * ld * esz), _DTYPES[dtype], nb, P, ld,
+                    ctypes.c_void_p(ws.data_ptr()), ws.numel(), N, seed, tiles, pt, ctypes.c_void_p(stream),
+                )
+            else:
+                table_dev = _segment_table(device, tuple((p + b0 * l * esz, fi, n, l) for p, fi, n, l in rows))
+                code = lib.trakhip_project_gather_partials(
+                    ctypes.c_void_p(table_dev.data_ptr()), len(rows), _DTYPES[dtype], nb, P,
+                    ctypes.c_void_p(ws.data_ptr()), ws.numel(), N, seed, tiles, pt, ctypes.c_void_p(stream),
+                )
+            _lib.check(code)
+            code = lib.trakhip_project_reduce_store(
+                ctypes.c_void_p(ws.data_ptr()), nb, P, N, tiles, float(scale), _DTYPES[out.dtype],
+                ctypes.c_void_p(out.data_ptr() + b0 * out_ld * out.element_size()), out_ld,
+                ctypes.c_void_p(stream),
+            )
+            _lib.check(code)
+    return out
+
+
 def project_gather(tensors, N, seed, num_feature_tiles, proj_type, scale=1.0):
     """Projects the gradient given as a list of per-parameter tensors [B, ...] (in order) without
     materializing the [B, P] matrix: same result, bit for bit, as `project_*` on
@@ -131,41 +216,10 @@ def project_gather(tensors, N, seed, num_feature_tiles, proj_type, scale=1.0):
     tensors = list(tensors)
     if not gather_supported(tensors):
         raise RuntimeError("project_gather needs CUDA tensors of one supported dtype, device and batch size")
-    flats = [_flat_rows(t) for t in tensors]
-    device, dtype = flats[0].device, flats[0].dtype
-    B = flats[0].shape[0]
-    esz = flats[0].element_size()
-    N, seed, tiles = int(N), int(seed) & 0xFFFFFFFF, int(num_feature_tiles)
-    lib = _lib.load()
-    if N <= 0 or N % 512 != 0:
-        _lib.check(_lib.ERR_PROJ_DIM)
-    rows, first = [], 0
-    for f in flats:
-        numel = f.shape[1]
-        ld = f.stride(0) if B > 1 else numel
-        rows.append([f.data_ptr(), first, numel, ld])
-        first += numel
-    P = first
-    pt = _lib.NORMAL if str(getattr(proj_type, "value", proj_type)) in ("normal", "1") else _lib.RADEMACHER
-    with torch.cuda.device(device):
-        out = torch.empty((B, N), dtype=torch.float32, device=device)
-        nbytes = lib.trakhip_project_workspace(B, P, N, tiles)
-        ws = _workspace(device, nbytes)
-        stream = torch.cuda.current_stream(device).cuda_stream
-        for b0 in range(0, B, 32):
-            nb = min(32, B - b0)
-            table_dev = _segment_table(device, tuple((p + b0 * ld * esz, fi, n, ld) for p, fi, n, ld in rows))
-            code = lib.trakhip_project_gather_partials(
-                ctypes.c_void_p(table_dev.data_ptr()), len(rows), _DTYPES[dtype], nb, P,
-                ctypes.c_void_p(ws.data_ptr()), ws.numel(), N, seed, tiles, pt, ctypes.c_void_p(stream),
-            )
-            _lib.check(code)
-            code = lib.trakhip_project_reduce(
-                ctypes.c_void_p(ws.data_ptr()), nb, P, N, tiles, float(scale),
-                ctypes.c_void_p(out.data_ptr() + b0 * N * 4), ctypes.c_void_p(stream),
-            )
-            _lib.check(code)
-    return out
+    t0 = tensors[0]
+    with torch.cuda.device(t0.device):
+        out = torch.empty((t0.shape[0], int(N)), dtype=torch.float32, device=t0.device)
+    return project_into(tensors, N, seed, num_feature_tiles, proj_type, out, scale)
 
 
 def project_rademacher_8(input, N, seed, num_feature_tiles):
@@ -196,7 +250,7 @@ def materialize(seed, num_feature_tiles, P, f0, nf, c0, nc, proj_type, device=No
     """Block S[f0:f0+nf, c0:c0+nc] of the matrix `project_*` uses, as fp32.  device=None runs
     the library's host code and returns a CPU tensor; a CUDA device runs the device kernel."""
     lib = _lib.load()
-    pt = _lib.NORMAL if str(getattr(proj_type, "value", proj_type)) in ("normal", "1") else _lib.RADEMACHER
+    pt = _proj_type_code(proj_type)
     if device is None or torch.device(device).type == "cpu":
         out = torch.empty((nf, nc), dtype=torch.float32)
         code = lib.trakhip_materialize(

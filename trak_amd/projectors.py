@@ -142,6 +142,24 @@ class CudaProjector(AbstractProjector):
         fn = getattr(fast_jl, f"project_{_type_name(self.proj_type)}_{effective_batch_size}")
         return fn(grads, self.proj_dim, self.seed + int(1e4) * model_id, self.num_sms)
 
+    def project_into(self, grads: Union[dict, Tensor], model_id: int, out: Tensor, scale: float = 1.0) -> Tensor:
+        """out[B, proj_dim] = cast(project(grads, model_id) * scale), written by the kernel that sums
+        the feature tiles: `out` is a CUDA tensor or a page-locked CPU tensor of fp16 / bf16 / fp32.
+        Covers `project` plus `grads /= normalize_factor; grads.to(dtype).cpu()` of
+        trak/traker.py:425-428 (scale = 1 / normalize_factor).  Work is only enqueued: synchronize
+        before reading a CPU destination."""
+        if isinstance(grads, dict):
+            tensors = list(grads.values())
+            if fast_jl.gather_supported(tensors) and tensors[0].device == self._device:
+                source = tensors
+            else:
+                source = vectorize(grads, device=self.device)
+        else:
+            source = grads
+        return fast_jl.project_into(
+            source, self.proj_dim, self.seed + int(1e4) * model_id, self.num_sms, _type_name(self.proj_type), out, scale
+        )
+
     def free_memory(self):
         """A no-op method."""
 

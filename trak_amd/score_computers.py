@@ -11,7 +11,7 @@ from abc import ABC, abstractmethod
 import torch
 from torch import Tensor
 
-from .utils import gemm_nt, gemm_tn, spd_inverse
+from .utils import gemm_nt, gemm_tn, scores_finalize, spd_inverse
 
 ch = torch
 
@@ -120,3 +120,89 @@ class BasicScoreComputer(AbstractScoreComputer):
         return gemm_nt(
             features.to(self._dev), target_grads.to(self._dev), alpha=scale, row_scale=out_to_loss.reshape(-1)
         )
+
+
+class ScoreAccumulator:
+    """The checkpoint loop of TRAKer.finalize_scores (trak/traker.py:641-678) with the score sums
+    kept on the GPU.
+
+    The reference adds every checkpoint's [N, M] score matrix into a CPU tensor (one device-to-host
+    copy of the whole matrix per checkpoint) and evaluates
+    `(_scores / n) * (_avg_out_to_losses / n)` with numpy at the end.  Here `add` accumulates in the
+    GEMM epilogue on the device, the out_to_loss sums stay a small host array exactly as in the
+    reference, and `finalize` applies the same expression on the device while the matrix is
+    written, chunk by chunk through page-locked memory, into the scores store: one crossing of
+    PCIe in total.
+
+    Args:
+        score_computer: a BasicScoreComputer of this package.
+        train_set_size, num_targets: N and M.
+        dtype: torch.float16 or torch.float32, the saver's element type (trak/traker.py:127); it
+            fixes the type the out_to_loss sums are kept in, as in the reference.
+    """
+
+    def __init__(self, score_computer, train_set_size, num_targets, dtype=ch.float32):
+        import numpy as np
+
+        self._np = np
+        self.score_computer = score_computer
+        self.shape = (int(train_set_size), int(num_targets))
+        self.dtype = dtype
+        self._acc = ch.zeros(self.shape, dtype=ch.float32, device=score_computer._dev)
+        self._out_to_loss = np.zeros(
+            (self.shape[0], 1), dtype=np.float16 if dtype == ch.float16 else np.float32
+        )
+        self.num_models = 0
+
+    def add(self, features, target_grads, out_to_loss) -> None:
+        """One checkpoint: sums += features @ target_grads^T (trak/traker.py:667) and
+        out_to_loss sums += out_to_loss (trak/traker.py:670)."""
+        self.score_computer.get_scores(features, target_grads, accumulator=self._acc)
+        o = out_to_loss.detach().cpu().numpy() if isinstance(out_to_loss, Tensor) else self._np.asarray(out_to_loss)
+        self._out_to_loss += o.reshape(self.shape[0], 1)
+        self.num_models += 1
+
+    def finalize(self, out, chunk_bytes: int = 256 << 20):
+        """Writes `(sums / n) * (out_to_loss sums / n)` (trak/traker.py:674-676) into `out`, the
+        [N, M] array behind the saver's `<exp>_scores` store (numpy array or memmap of float16 or
+        float32) or a tensor (CUDA, or page-locked CPU).  Returns `out`."""
+        np = self._np
+        if self.num_models == 0:
+            raise ValueError("no checkpoint was added")
+        n = float(self.num_models)
+        # the second factor exactly as numpy computes it in the reference, then widened (exact)
+        row_factor = (self._out_to_loss / n).astype(np.float32).reshape(-1)
+        row_factor = ch.from_numpy(row_factor).to(self._acc.device)
+        N, M = self.shape
+        if isinstance(out, Tensor):
+            scores_finalize(self._acc, n, row_factor, out)
+            if not out.is_cuda:
+                ch.cuda.current_stream(self._acc.device).synchronize()
+            return out
+        if tuple(out.shape) != (N, M) or out.dtype not in (np.float16, np.float32):
+            raise ValueError(f"out must be a [{N}, {M}] array of float16 or float32")
+        tdtype = ch.float16 if out.dtype == np.float16 else ch.float32
+        rows = max(1, min(N, int(chunk_bytes) // max(1, M * out.dtype.itemsize)))
+        stage = [ch.empty((rows, M), dtype=tdtype).pin_memory() for _ in range(2 if rows < N else 1)]
+        pending = [None] * len(stage)
+        stream = ch.cuda.current_stream(self._acc.device)
+
+        def retire(i):
+            if pending[i] is None:
+                return
+            event, r0, r1 = pending[i]
+            event.synchronize()
+            out[r0:r1] = stage[i][: r1 - r0].numpy()
+            pending[i] = None
+
+        for index, r0 in enumerate(range(0, N, rows)):
+            i = index % len(stage)
+            retire(i)
+            r1 = min(N, r0 + rows)
+            scores_finalize(self._acc[r0:r1], n, row_factor[r0:r1], stage[i][: r1 - r0])
+            event = ch.cuda.Event()
+            event.record(stream)
+            pending[i] = (event, r0, r1)
+        for i in range(len(stage)):
+            retire((index + 1 + i) % len(stage))
+        return out

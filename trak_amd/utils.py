@@ -193,6 +193,51 @@ def spd_inverse(a, lambda_reg=0.0, normalize=False):
     return inv, mean_abs
 
 
+_STORE_DTYPES = {torch.float16: _lib.F16, torch.bfloat16: _lib.BF16, torch.float32: _lib.F32}
+
+
+def scores_finalize(acc, divisor, row_factor, out):
+    """out[i, j] = cast((acc[i, j] / divisor) * row_factor[i]): the closing expression of
+    TRAKer.finalize_scores (trak/traker.py:670-678) for fp32 score sums `acc` [N, M] on the GPU.
+    `out` [N, M] (fp16 / bf16 / fp32) is a CUDA tensor on the same device or a page-locked CPU
+    tensor; row_factor (N values, or None) is moved to the device as fp32.  Enqueued on the
+    current stream; synchronize before reading a CPU destination."""
+    if not acc.is_cuda or acc.dtype != torch.float32 or acc.dim() != 2 or (acc.shape[1] > 1 and acc.stride(1) != 1):
+        raise RuntimeError("acc must be an fp32 [N, M] CUDA tensor with unit column stride")
+    N, M = acc.shape
+    if out.dim() != 2 or tuple(out.shape) != (N, M) or out.dtype not in _STORE_DTYPES:
+        raise RuntimeError(f"out must be a [{N}, {M}] tensor of fp16, bf16 or fp32")
+    if M > 1 and out.stride(1) != 1:
+        raise RuntimeError("out must have unit column stride")
+    if out.is_cuda:
+        if out.device != acc.device:
+            raise RuntimeError("out must live on acc's device")
+    elif not out.is_pinned():
+        raise RuntimeError("a CPU destination must be page-locked (pin_memory)")
+    rf = None
+    if row_factor is not None:
+        rf = torch.as_tensor(row_factor).reshape(-1).to(device=acc.device, dtype=torch.float32).contiguous()
+        if rf.numel() != N:
+            raise RuntimeError("row_factor must have N elements")
+    lib = _lib.load()
+    with torch.cuda.device(acc.device):
+        stream = torch.cuda.current_stream(acc.device).cuda_stream
+        code = lib.trakhip_scores_finalize(
+            ctypes.c_void_p(acc.data_ptr()),
+            _ld(acc),
+            N,
+            M,
+            float(divisor),
+            ctypes.c_void_p(rf.data_ptr()) if rf is not None else None,
+            _STORE_DTYPES[out.dtype],
+            ctypes.c_void_p(out.data_ptr()),
+            _ld(out),
+            ctypes.c_void_p(stream),
+        )
+    _lib.check(code)
+    return out
+
+
 def get_matrix_mult(features, target_grads, target_dtype=None, batch_size=8096, use_blockwise=False):
     """features @ target_grads.T (trak/utils.py:248-294).  On the GPU this is one fp32 MFMA GEMM;
     CPU inputs take torch's matmul as in the reference (trak/utils.py:128-132).  The reference's
