@@ -303,6 +303,81 @@ def test_full_size_resnet18_shape(gpu, c_oracle):
         assert np.linalg.norm(got - want) / np.linalg.norm(want) < 1e-3
 
 
+def test_full_size_cpu_runnable_shape(gpu, c_oracle):
+    # gradients [16, 1 048 576] fp32 iid N(0, 1e-3^2), k = 512, seed 42: every column against the
+    # float64 contraction, to the fp32 bar
+    B, P, k, seed, tiles = 16, 1_048_576, 512, 42, 256
+    gen = torch.Generator(device="cpu").manual_seed(42)
+    g = torch.randn(B, P, generator=gen) * 1e-3
+    out = fast_jl.project_rademacher_16(g.to(gpu), k, seed, tiles).cpu().numpy()
+    for c0 in (0, k - 48):
+        want = c_oracle.project(g.numpy(), seed, tiles, c0, 48, R)
+        assert rel_l2_rows(out[:, c0 : c0 + 48], want).max() < 1e-5
+    # JL norm preservation at this shape: |Sg|^2 / k ~ |g|^2 within a few 1/sqrt(k)
+    ratio = (out.astype(np.float64) ** 2).sum(1) / k / (g.double().numpy() ** 2).sum(1)
+    assert np.abs(ratio - 1).max() < 6 * math.sqrt(2.0 / k)
+
+
+def test_full_size_resnet9_shape(gpu, c_oracle):
+    # gradients [32, 4 825 610] fp16 (P not a multiple of anything), N(0, 5e-4^2) with 1 % exact
+    # zeros, k = 2048, seed 0, eight batches through one projector
+    B, P, k, seed = 32, 4_825_610, 2048, 0
+    proj = _projector(P, k, seed, ProjectionType.rademacher, torch.float16, num_sms=256)
+    gen = torch.Generator(device=gpu).manual_seed(20_009)
+    for batch in range(8):
+        g = torch.randn(B, P, generator=gen, device=gpu) * 5e-4
+        g[torch.rand(B, P, generator=gen, device=gpu) < 0.01] = 0.0
+        g = g.half()
+        assert 0.005 < float((g == 0).float().mean()) < 0.02
+        out = proj.project(g, model_id=0)
+        assert out.shape == (B, k) and out.dtype == torch.float32
+        if batch in (0, 7):
+            g32 = to_f32_numpy(g)
+            for c in (0, 1023, 2047):
+                want = c_oracle.project(g32, seed, 256, c, 1, R)[:, 0]
+                got = out[:, c].cpu().numpy().astype(np.float64)
+                assert np.linalg.norm(got - want) / np.linalg.norm(want) < 1e-3
+        if batch == 0:
+            first_in, first_out = g, out.clone()
+    assert torch.equal(proj.project(first_in, model_id=0), first_out)  # no state between batches
+
+
+def test_full_size_bert_normal_chunked_shape(gpu, c_oracle):
+    # gradients [32, 109 482 240] bf16 in 4 parameter chunks, Student-t (nu = 3) * 1e-4, k = 4096,
+    # seed 123, normal matrix, through ChunkedCudaProjector with TRAKer's per-chunk seeds
+    # (trak/traker.py:290-310); two columns against the float64 contraction of every chunk
+    B, P, k, seed, tiles = 32, 109_482_240, 4096, 123, 256
+    sizes = [P // 4] * 4
+    seeds = np.random.default_rng(seed).integers(low=0, high=500, size=4)
+    per_chunk = [_projector(sz, k, int(seeds[i]), ProjectionType.normal, torch.bfloat16, num_sms=tiles)
+                 for i, sz in enumerate(sizes)]
+    proj = ChunkedCudaProjector(per_chunk, max(sizes), sizes, B, "cuda:0", torch.bfloat16)
+    gen = torch.Generator(device=gpu).manual_seed(20_010)
+    grads = {}
+    for i, sz in enumerate(sizes):
+        # Student-t with 3 degrees of freedom: normal / sqrt(chi2_3 / 3)
+        z = torch.randn(B, sz, generator=gen, device=gpu)
+        chi = sum(torch.randn(B, sz, generator=gen, device=gpu) ** 2 for _ in range(3)) / 3
+        grads[f"chunk{i}"] = (z / chi.sqrt() * 1e-4).bfloat16()
+        del z, chi
+    out = proj.project(grads, model_id=0)
+    assert out.shape == (B, k) and out.dtype == torch.bfloat16
+    # the chunk projections in fp32, before the cast the chunked projector applies at the end
+    parts = [per_chunk[i].project(grads[f"chunk{i}"], model_id=0) for i in range(4)]
+    total = sum(p.double() for p in parts)
+    assert torch.equal(total.float().bfloat16(), out) or (total.float() - out.float()).abs().max() <= \
+        out.float().abs().max() * 2 ** -7
+    for c in (5, 4090):
+        want = np.zeros(B)
+        for i in range(4):
+            want += c_oracle.project(to_f32_numpy(grads[f"chunk{i}"]), int(seeds[i]), tiles, c, 1, G)[:, 0]
+        got = total[:, c].cpu().numpy()
+        assert np.linalg.norm(got - want) / np.linalg.norm(want) < 1e-3
+    proj.free_memory()
+    del grads
+    torch.cuda.empty_cache()
+
+
 # ---- the reference's uint32-overflow shapes (tests/test_jl.py:59-73, tests/test_jl_additional.py:11-44) ----
 
 
