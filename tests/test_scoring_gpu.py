@@ -122,3 +122,47 @@ def test_score_computer_matches_float64_oracle(gpu, N, k, M, lam, max_dim):
     fused = sc.get_scaled_scores(feats, Xt.to(gpu), otl.to(gpu))
     assert rel_max(fused.cpu().numpy(), so.finalize_scores_f64(scores_want, otl.numpy(), 1)) < 1e-4
     assert rel_max(get_matrix_mult(feats, Xt.to(gpu)).cpu().numpy(), scores_want) < 1e-4
+
+
+def test_full_size_scoring_shape(gpu):
+    """N = 50 000 training rows, k = 4096, M = 10 000 targets, lambda = 1e-3: the float64 oracle does not
+    finish in seconds on a CPU at this size, so the check uses what does not depend on size: the
+    inverse identity, the trace closed form, symmetry, and row / block samples of every product
+    against float64 (1e-4 relative, the bar stated for the scores)."""
+    N, k, M, lam = 50_000, 4096, 10_000, 1e-3
+    gen = torch.Generator(device=gpu).manual_seed(20_011)
+    X = torch.randn(N, k, generator=gen, device=gpu) / math.sqrt(k)
+    Xt = torch.randn(M, k, generator=gen, device=gpu) / math.sqrt(k)
+    otl = torch.rand(N, generator=gen, device=gpu)
+    sc = BasicScoreComputer(dtype=torch.float32, device="cuda:0", lambda_reg=lam)
+    xtx = sc.get_xtx(X)
+    assert torch.equal(xtx, xtx.T)
+    trace64 = float((X.double() ** 2).sum())
+    # fp32 accumulation over 50 000 positive terms: the bound the GEMM tests use, not better
+    assert abs(float(xtx.double().diagonal().sum()) - trace64) < gemm_tol(N) * trace64
+    cols = torch.arange(1000, 1064, device=gpu)
+    block64 = X[:, cols].double().T @ X.double()[:, 3000:3100]
+    assert rel_max(xtx[cols][:, 3000:3100].cpu().numpy(), block64.cpu().numpy()) < gemm_tol(N)
+
+    inv, mean_abs = spd_inverse(xtx, lambda_reg=lam, normalize=True)
+    a64 = xtx.double() + lam * torch.eye(k, device=gpu, dtype=torch.float64)
+    resid = a64 @ (inv.double() * mean_abs.double()) - torch.eye(k, device=gpu, dtype=torch.float64)
+    assert float(resid.abs().max()) < 1e-4
+    assert abs(float(inv.abs().mean()) - 1.0) < 1e-5                      # the rescaling of score_computers.py:166
+
+    feats = sc.get_x_xtx_inv(X, xtx)
+    rows = torch.tensor([0, 1, 777, 25_000, 49_999], device=gpu)
+    inv64 = torch.linalg.inv(a64)
+    inv64 = inv64 / inv64.abs().mean()
+    feats64 = X[rows].double() @ inv64
+    assert rel_max(feats[rows].cpu().numpy(), feats64.cpu().numpy()) < 1e-4
+
+    acc = torch.zeros(N, M, device=gpu)
+    sc.get_scores(feats, Xt, accumulator=acc)
+    scores64 = feats64 @ Xt.double().T
+    assert rel_max(acc[rows].cpu().numpy(), scores64.cpu().numpy()) < 1e-4
+    tcols = torch.tensor([0, 5000, 9999], device=gpu)
+    col64 = (X.double() @ inv64) @ Xt[tcols].double().T                    # every training row, three targets
+    assert rel_max(acc[:, tcols].cpu().numpy(), col64.cpu().numpy()) < 1e-4
+    fused = sc.get_scaled_scores(feats, Xt, otl)
+    assert rel_max(fused[rows].cpu().numpy(), (scores64 * otl[rows].double()[:, None]).cpu().numpy()) < 1e-4
