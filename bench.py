@@ -345,19 +345,35 @@ def bench_scoring(torch, dev, reps=3):
             best = ms if best is None else min(best, ms)
         return r, best
 
-    from trak_amd.utils import gemm_nt, gemm_tn, spd_inverse
+    from trak_amd.utils import gemm_nt, gemm_nt_split, gemm_tn, spd_inverse, split_rows
 
+    # the fp32 MFMA instruction (v_mfma_f32_32x32x2_f32): priced against the 157.3 TFLOP/s fp32 peak
     xtx, t_xtx = timed(lambda: gemm_tn(X, X))
     (inv, _), t_inv = timed(lambda: spd_inverse(xtx, lambda_reg=lam, normalize=True))
     feats, t_feat = timed(lambda: gemm_nt(X, inv))
     scores, t_sc = timed(lambda: gemm_nt(feats, Xt, row_scale=otl))
     gemm_flop = 2.0 * N * k * k * 2 + 2.0 * N * M * k
     gemm_ms = t_xtx + t_feat + t_sc
+    del scores
+    # the same three products with fp32 operands split exactly into three bf16 terms (six bf16 MFMAs
+    # per k step, fp32 accumulation; what BasicScoreComputer runs by default), splitting included:
+    # fp32-equivalent TFLOP/s = the same 2*M*N*K over the time; 6x that many bf16 flops are executed
+    _, s_xtx = timed(lambda: (lambda xt: gemm_nt_split(xt, xt))(split_rows(X, transposed=True)))
+    _, s_feat = timed(lambda: gemm_nt_split(split_rows(X), split_rows(inv)))
+    _, s_sc = timed(lambda: gemm_nt_split(split_rows(feats), split_rows(Xt), row_scale=otl))
+    split_ms = s_xtx + s_feat + s_sc
     return {
         "shape": {"N": N, "M": M, "k": k, "lambda": lam},
         "xtx_ms": t_xtx, "inverse_ms": t_inv, "x_xtx_inv_ms": t_feat, "scores_ms": t_sc,
         "gemm_tflops": gemm_flop / (gemm_ms * 1e-3) / 1e12,
         "gemm_frac_fp32_mfma_peak": gemm_flop / (gemm_ms * 1e-3) / 1e12 / PEAK_FP32_TFLOPS,
+        "split_bf16x3": {
+            "xtx_ms": s_xtx, "x_xtx_inv_ms": s_feat, "scores_ms": s_sc,
+            "gemm_tflops_fp32_equivalent": gemm_flop / (split_ms * 1e-3) / 1e12,
+            "frac_fp32_mfma_peak": gemm_flop / (split_ms * 1e-3) / 1e12 / PEAK_FP32_TFLOPS,
+            "bf16_mfma_tflops_executed": 6 * gemm_flop / (split_ms * 1e-3) / 1e12,
+            "frac_bf16_mfma_peak": 6 * gemm_flop / (split_ms * 1e-3) / 1e12 / PEAK_FP16_TFLOPS,
+        },
         "inverse_flop": float(k) ** 3,
         "scores_orientation": "[N_train, M_targets]",
     }

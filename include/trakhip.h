@@ -136,6 +136,26 @@ int trakhip_gemm_tn(const float* A_dev, uint64_t lda, const float* B_dev, uint64
                     uint64_t ldc, uint64_t M, uint64_t N, uint64_t K, float alpha, float beta,
                     void* stream);
 
+/* The same products on the bf16 matrix cores (sixteen times the fp32 MFMA rate) without giving up
+ * fp32 accuracy: an operand is first split into three bf16 "planes" whose sum is the fp32 value
+ * exactly (trakhip_split_rows, one pass over the operand), and trakhip_gemm_nt_split multiplies
+ * planes with six bf16 MFMAs per k step, accumulating in fp32; the terms left out are below
+ * 2^-24 of each product, the rounding of one fp32 multiplication.
+ *   trakhip_split_bytes(rows, K)   bytes of the planes of a [rows, K] operand
+ *   trakhip_split_rows             src_dev is [rows, K] with row pitch ld (transposed == 0), or
+ *                                  [K, rows] with row pitch ld (transposed != 0: the operand is
+ *                                  the transpose of what is stored, as X^T in X^T X)
+ *   trakhip_gemm_nt_split          C[M, N] = alpha * A * B^T + beta * C, row i *= row_scale[i];
+ *                                  A_planes from a [M, K] operand, B_planes from a [N, K] one
+ * Stand in, like trakhip_gemm_nt / trakhip_gemm_tn, for trak/score_computers.py:153, :176 and
+ * trak/utils.py:131. */
+size_t trakhip_split_bytes(uint64_t rows, uint64_t K);
+int trakhip_split_rows(const float* src_dev, uint64_t ld, uint64_t rows, uint64_t K, int transposed,
+                       void* planes_dev, size_t planes_bytes, void* stream);
+int trakhip_gemm_nt_split(const void* A_planes_dev, uint64_t M, const void* B_planes_dev, uint64_t N, uint64_t K,
+                          float* C_dev, uint64_t ldc, float alpha, float beta, const float* row_scale_dev,
+                          void* stream);
+
 /* out[i, j] = cast((acc[i, j] / divisor) * row_factor[i]) for the [N, M] fp32 score sums that
  * trakhip_gemm_nt accumulated over checkpoints (beta = 1): the closing expression of
  * TRAKer.finalize_scores, `(_scores / n) * (_avg_out_to_losses / n)` (trak/traker.py:670-678), with

@@ -9,7 +9,7 @@ import torch
 
 from oracle import score_oracle as so
 from trak_amd import BasicScoreComputer, get_matrix_mult
-from trak_amd.utils import gemm_nt, gemm_tn, spd_inverse
+from trak_amd.utils import gemm_nt, gemm_nt_split, gemm_tn, spd_inverse, split_rows
 
 pytestmark = pytest.mark.gpu
 
@@ -93,13 +93,83 @@ def test_spd_inverse_closed_forms_and_failure(gpu):
         spd_inverse(bad.to(gpu))
 
 
+def split_planes_to_numpy(op):
+    """[3, padded rows, padded K] float32 view of a SplitOperand (layout: plane, k-octet, row, 8 bf16)."""
+    Rp, K8 = (op.rows + 255) // 256 * 256, (op.K + 15) // 16 * 2
+    raw = op.planes.cpu().numpy()[: 3 * K8 * Rp * 16].view(np.uint16).reshape(3, K8, Rp, 8)
+    return (raw.astype(np.uint32) << 16).view(np.float32).transpose(0, 2, 1, 3).reshape(3, Rp, K8 * 8)
+
+
+@pytest.mark.parametrize("rows,K,transposed", [(5, 9, False), (300, 70, False), (70, 300, True), (257, 33, True), (256, 16, False)])
+def test_split_is_exact_and_zero_padded(gpu, rows, K, transposed):
+    gen = torch.Generator(device="cpu").manual_seed(rows * K)
+    t = torch.randn((K, rows) if transposed else (rows, K), generator=gen)
+    t *= 10.0 ** torch.randint(-12, 12, t.shape, generator=gen).float()       # every binade in reach
+    t.view(-1)[:3] = torch.tensor([0.0, -0.0, 1.0])
+    wide = torch.zeros(t.shape[0], t.shape[1] + 3)
+    wide[:, 1 : 1 + t.shape[1]] = t
+    for src in (t.to(gpu), wide.to(gpu)[:, 1 : 1 + t.shape[1]]):               # aligned rows, then pitched unaligned rows
+        op = split_rows(src, transposed=transposed)
+        planes = split_planes_to_numpy(op).astype(np.float64)
+        want = (t.T if transposed else t).numpy().astype(np.float64)
+        total = planes[0] + planes[1] + planes[2]
+        assert np.array_equal(total[:rows, :K], want)                          # three bf16 terms, exact sum
+        assert not total[rows:].any() and not total[:, K:].any()               # padding rewritten as zeros
+        nz = want != 0
+        assert (np.abs(planes[1][:rows, :K][nz]) <= 2.0 ** -8 * np.abs(planes[0][:rows, :K][nz])).all()
+        assert (np.abs(planes[2][:rows, :K][nz]) <= 2.0 ** -16 * np.abs(planes[0][:rows, :K][nz])).all()
+
+
+@pytest.mark.parametrize("M,N,K", [(1, 1, 1), (130, 70, 33), (256, 512, 64), (1000, 513, 257), (64, 2048, 4096), (129, 257, 8200)])
+def test_gemm_nt_split(gpu, M, N, K):
+    gen = torch.Generator(device="cpu").manual_seed(M * 7 + N + K)
+    a, b = torch.randn(M, K, generator=gen), torch.randn(N, K, generator=gen)
+    want = a.double().numpy() @ b.double().numpy().T
+    got = gemm_nt_split(split_rows(a.to(gpu)), split_rows(b.to(gpu)))
+    err = rel_max(got.cpu().numpy(), want)
+    assert got.shape == (M, N) and err < gemm_tol(K)
+    # no less accurate than the fp32 MFMA instruction on the same operands (factor 1.5 for noise)
+    assert err <= 1.5 * rel_max(gemm_nt(a.to(gpu), b.to(gpu)).cpu().numpy(), want) + 1e-7
+    # a transposed left operand, alpha, beta and the row scale epilogue
+    at = a.T.contiguous()
+    c0 = torch.randn(M, N, generator=gen)
+    rs = torch.rand(M, generator=gen)
+    got = gemm_nt_split(split_rows(at.to(gpu), transposed=True), split_rows(b.to(gpu)), out=c0.clone().to(gpu),
+                        alpha=0.5, beta=-2.0, row_scale=rs.to(gpu))
+    want2 = (0.5 * want - 2.0 * c0.double().numpy()) * rs.double().numpy()[:, None]
+    assert rel_max(got.cpu().numpy(), want2) < gemm_tol(K)
+    # strided output
+    wide = torch.zeros(M, N + 5, device=gpu)
+    gemm_nt_split(split_rows(a.to(gpu)), split_rows(b.to(gpu)), out=wide[:, 2 : 2 + N])
+    assert rel_max(wide[:, 2 : 2 + N].cpu().numpy(), want) < gemm_tol(K)
+    assert float(wide[:, :2].abs().sum()) == 0 and float(wide[:, 2 + N :].abs().sum()) == 0
+
+
+def test_gemm_nt_split_keeps_small_terms(gpu):
+    # b = 1 + 2^-20 needs 21 significand bits: one bf16 term (8 bits) would return exactly K, the
+    # split product returns K * (1 + 2^-20) to fp32 accuracy (K small enough that the running sum
+    # still resolves the small part, as for any fp32 dot product)
+    K = 16
+    a = torch.ones(32, K)
+    b = torch.full((32, K), 1.0 + 2.0 ** -20)
+    want = K * (1.0 + 2.0 ** -20)
+    got = gemm_nt_split(split_rows(a.to(gpu)), split_rows(b.to(gpu))).cpu().numpy().astype(np.float64)
+    assert np.abs(got - want).max() <= 2.0 ** -23 * K
+    # cross terms of both operands: (1 + 2^-9)(1 - 2^-9) = 1 - 2^-18 needs a1*b2, a2*b1 and a2*b2
+    a = torch.full((32, K), 1.0 + 2.0 ** -9)
+    b = torch.full((32, K), 1.0 - 2.0 ** -9)
+    got = gemm_nt_split(split_rows(a.to(gpu)), split_rows(b.to(gpu))).cpu().numpy().astype(np.float64)
+    assert np.abs(got - K * (1.0 - 2.0 ** -18)).max() <= 2.0 ** -23 * K
+
+
+@pytest.mark.parametrize("gemm", ["split", "fp32"])
 @pytest.mark.parametrize("N,k,M,lam,max_dim", [(700, 512, 90, 1e-3, 20_000), (2500, 1024, 300, 0.0, 1000), (333, 100, 17, 1e-2, 100)])
-def test_score_computer_matches_float64_oracle(gpu, N, k, M, lam, max_dim):
+def test_score_computer_matches_float64_oracle(gpu, N, k, M, lam, max_dim, gemm):
     gen = torch.Generator(device="cpu").manual_seed(N + k)
     X = torch.randn(N, k, generator=gen) / math.sqrt(k)
     Xt = torch.randn(M, k, generator=gen) / math.sqrt(k)
     otl = torch.rand(N, generator=gen)
-    sc = BasicScoreComputer(dtype=torch.float32, device="cuda:0", CUDA_MAX_DIM_SIZE=max_dim, lambda_reg=lam)
+    sc = BasicScoreComputer(dtype=torch.float32, device="cuda:0", CUDA_MAX_DIM_SIZE=max_dim, lambda_reg=lam, gemm=gemm)
     xtx_want = so.xtx_f64(X.numpy())
     feats_want, _, _ = so.x_xtx_inv_f64(X.numpy(), xtx_want, lam)
     scores_want = so.scores_f64(feats_want, Xt.numpy())
@@ -124,7 +194,8 @@ def test_score_computer_matches_float64_oracle(gpu, N, k, M, lam, max_dim):
     assert rel_max(get_matrix_mult(feats, Xt.to(gpu)).cpu().numpy(), scores_want) < 1e-4
 
 
-def test_full_size_scoring_shape(gpu):
+@pytest.mark.parametrize("gemm", ["split", "fp32"])
+def test_full_size_scoring_shape(gpu, gemm):
     """N = 50 000 training rows, k = 4096, M = 10 000 targets, lambda = 1e-3: the float64 oracle does not
     finish in seconds on a CPU at this size, so the check uses what does not depend on size: the
     inverse identity, the trace closed form, symmetry, and row / block samples of every product
@@ -134,9 +205,12 @@ def test_full_size_scoring_shape(gpu):
     X = torch.randn(N, k, generator=gen, device=gpu) / math.sqrt(k)
     Xt = torch.randn(M, k, generator=gen, device=gpu) / math.sqrt(k)
     otl = torch.rand(N, generator=gen, device=gpu)
-    sc = BasicScoreComputer(dtype=torch.float32, device="cuda:0", lambda_reg=lam)
+    sc = BasicScoreComputer(dtype=torch.float32, device="cuda:0", lambda_reg=lam, gemm=gemm)
     xtx = sc.get_xtx(X)
-    assert torch.equal(xtx, xtx.T)
+    # the fp32 instruction sums both triangles in the same order; the split product adds the cross
+    # terms a1*b2 and a2*b1 in the opposite order for (i, j) and (j, i): equal to the last bits only
+    # (the inverse reads the lower triangle)
+    assert torch.equal(xtx, xtx.T) if gemm == "fp32" else float((xtx - xtx.T).abs().max()) <= 2e-6 * float(xtx.abs().max())
     trace64 = float((X.double() ** 2).sum())
     # fp32 accumulation over 50 000 positive terms: the bound the GEMM tests use, not better
     assert abs(float(xtx.double().diagonal().sum()) - trace64) < gemm_tol(N) * trace64

@@ -9,7 +9,7 @@ import sys
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libtrakhip.so")
-SOURCES = ["capi.hip", "project.hip", "gemm.hip", "spd.hip", "store.hip"]
+SOURCES = ["capi.hip", "project.hip", "gemm.hip", "spd.hip", "store.hip", "gemm_split.hip"]
 FLAGS = [
     "--offload-arch=gfx950",
     "-O3",

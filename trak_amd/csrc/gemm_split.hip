@@ -1,0 +1,257 @@
+// fp32 GEMM on the bf16 matrix cores: C[M, N] = alpha * A * B^T + beta * C (row i *= row_scale[i]).
+//
+// The scoring GEMMs of BasicScoreComputer (trak/score_computers.py:153, :176, trak/utils.py:131)
+// are fp32 x fp32.  v_mfma_f32_32x32x2_f32 runs at 157 TFLOP/s; v_mfma_f32_32x32x16_bf16 at 2.5
+// PFLOP/s, sixteen times the rate.  Every fp32 value is the exact sum of three bf16 values
+// (24 significand bits = 3 x 8), x = x1 + x2 + x3 with |x2| <= 2^-8 |x1|, |x3| <= 2^-16 |x1|, so
+//     a * b = a1 b1 + (a1 b2 + a2 b1) + (a1 b3 + a2 b2 + a3 b1) + O(2^-24 |a b|)
+// and six bf16 MFMAs (products exact, fp32 accumulation) give the product sum with the error of an
+// fp32 dot product at 6/16 of the cost of the fp32 instruction.  The three terms left out are each
+// below 2^-24 |a b|, the rounding a single fp32 multiplication makes.
+//
+// Operands are split once, outside the GEMM, into "planes": plane p, k-octet o (8 consecutive k),
+// row r is one 16-byte piece at ((p * K8 + o) * Rp + r) * 16 bytes, rows padded with zeros to a
+// multiple of 256 and octets to an even count.  A 16-byte piece is exactly what one lane feeds to
+// the MFMA (8 consecutive k of one row), consecutive rows are consecutive pieces, so global loads,
+// LDS writes and LDS reads are all linear and conflict free, and the GEMM kernel moves bf16 only.
+//
+// Workgroup = 256 threads = 4 waves (2 x 2), 128 x 256 tile of C, k step 16 (one MFMA deep), two
+// LDS buffers of 36 KB, one barrier per step; a wave owns 64 x 128 of C (128 accumulator VGPRs)
+// and issues 48 MFMAs per step.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "trakhip_internal.h"
+
+namespace {
+
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef uint32_t piece __attribute__((ext_vector_type(4)));  // 16 bytes = 8 bf16 = one lane's MFMA operand
+
+constexpr int kThreads = 256;
+constexpr int BM = 128, BN = 256;
+constexpr int kRowPad = 256;                       // rows of a split operand are padded to this
+constexpr int kAPieces = 3 * 2 * BM;               // 16-byte pieces of an A tile: [plane][half][row]
+constexpr int kBPieces = 3 * 2 * BN;
+constexpr int kBufPieces = kAPieces + kBPieces;    // 2304 pieces = 36 KB
+
+// ---- splitting -----------------------------------------------------------------------------
+
+// binary32 -> nearest bf16 (ties to even) as a binary32 value; finite inputs
+__device__ __forceinline__ float bf16_round(float x) {
+    const uint32_t b = __float_as_uint(x);
+    return __uint_as_float((b + 0x7FFFu + ((b >> 16) & 1u)) & 0xFFFF0000u);
+}
+
+// x = t[0] + t[1] + t[2] exactly (up to underflow of the last term), bf16 bit patterns
+__device__ __forceinline__ void split3(float x, uint32_t (&t)[3]) {
+    const float x1 = bf16_round(x);
+    const float r1 = x - x1;
+    const float x2 = bf16_round(r1);
+    const float r2 = r1 - x2;
+    t[0] = __float_as_uint(x1) >> 16;
+    t[1] = __float_as_uint(x2) >> 16;
+    t[2] = __float_as_uint(bf16_round(r2)) >> 16;
+}
+
+// One thread per (row r, octet o): reads 8 consecutive k of the row, writes its three pieces.
+// TRANS = false: src[r * ld + k];  TRANS = true: src[k * ld + r].  Rows >= rows and k >= K give
+// zeros (the padding is rewritten on every call).  Threads of a workgroup cover 64 rows x 4 octets.
+template <bool TRANS, bool ALIGNED>
+__global__ __launch_bounds__(256) void split_kernel(const float* __restrict__ src, uint64_t ld, uint64_t rows,
+                                                    uint64_t K, uint64_t Rp, uint64_t K8, uint32_t row_blocks,
+                                                    uint4* __restrict__ planes) {
+    const uint64_t r = (uint64_t)(blockIdx.x % row_blocks) * 64 + (threadIdx.x & 63);
+    const uint64_t o = (uint64_t)(blockIdx.x / row_blocks) * 4 + (threadIdx.x >> 6);
+    if (r >= Rp || o >= K8) return;
+    float v[8];
+    if (!TRANS && ALIGNED && r < rows && 8 * o + 8 <= K) {
+        // the four waves of a workgroup read the four octets of a 128-byte line of each row
+        const float4* q = reinterpret_cast<const float4*>(src + r * ld + 8 * o);
+        const float4 lo = q[0], hi = q[1];
+        v[0] = lo.x, v[1] = lo.y, v[2] = lo.z, v[3] = lo.w;
+        v[4] = hi.x, v[5] = hi.y, v[6] = hi.z, v[7] = hi.w;
+    } else {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const uint64_t k = 8 * o + i;
+            v[i] = (r < rows && k < K) ? (TRANS ? src[k * ld + r] : src[r * ld + k]) : 0.0f;
+        }
+    }
+    uint32_t w[3][4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        uint32_t lo[3], hi[3];
+        split3(v[2 * i], lo);
+        split3(v[2 * i + 1], hi);
+#pragma unroll
+        for (int p = 0; p < 3; ++p) w[p][i] = lo[p] | (hi[p] << 16);
+    }
+#pragma unroll
+    for (int p = 0; p < 3; ++p) planes[((uint64_t)p * K8 + o) * Rp + r] = make_uint4(w[p][0], w[p][1], w[p][2], w[p][3]);
+}
+
+// ---- GEMM ----------------------------------------------------------------------------------
+
+__device__ __forceinline__ floatx16 mfma_bf16(const piece& a, const piece& b, floatx16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c,
+                                                   0, 0, 0);
+}
+
+// pieces of step s (octets 2s, 2s + 1) of the tile rows [x0, x0 + ROWS): piece e = (plane, half, row)
+template <int ROWS, int N>
+__device__ __forceinline__ void load_pieces(const piece* __restrict__ planes, uint64_t Rp, uint64_t K8,
+                                            uint64_t x0, uint64_t s, int tid, piece (&r)[N]) {
+#pragma unroll
+    for (int i = 0; i < N; ++i) {
+        const int e = tid + kThreads * i;
+        const int row = e % ROWS, ph = e / ROWS;  // ph = plane * 2 + half
+        r[i] = planes[((uint64_t)(ph >> 1) * K8 + 2 * s + (ph & 1)) * Rp + x0 + row];
+    }
+}
+
+template <int N>
+__device__ __forceinline__ void store_pieces(piece* lds, int tid, const piece (&r)[N]) {
+#pragma unroll
+    for (int i = 0; i < N; ++i) lds[tid + kThreads * i] = r[i];
+}
+
+__global__ __launch_bounds__(kThreads, 2) void gemm_split_kernel(
+    const piece* __restrict__ A, uint64_t Rpa, const piece* __restrict__ B, uint64_t Rpb, uint64_t K8,
+    float* __restrict__ C, uint64_t ldc, uint64_t M, uint64_t N, float alpha, float beta,
+    const float* __restrict__ row_scale, uint32_t tiles_n) {
+    __shared__ piece lds[2][kBufPieces];
+
+    const uint32_t tile_m = blockIdx.x / tiles_n, tile_n = blockIdx.x % tiles_n;
+    const uint64_t m0 = (uint64_t)tile_m * BM, n0 = (uint64_t)tile_n * BN;
+    const int tid = threadIdx.x;
+    const int wave = tid >> 6, lane = tid & 63;
+    const int wm = wave >> 1, wn = wave & 1;
+    const int x = lane & 31, h = lane >> 5;
+
+    floatx16 acc[2][4];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+    const uint64_t steps = K8 / 2;
+    piece ra[kAPieces / kThreads], rb[kBPieces / kThreads];  // 3 + 6 pieces in flight per thread
+    load_pieces<BM>(A, Rpa, K8, m0, 0, tid, ra);
+    load_pieces<BN>(B, Rpb, K8, n0, 0, tid, rb);
+    store_pieces(lds[0], tid, ra);
+    store_pieces(lds[0] + kAPieces, tid, rb);
+    __syncthreads();
+
+    // piece index of this lane's operand for plane p: A rows wm*64 + 32*i + x, B rows wn*128 + 32*j + x
+    const int a_lane = h * BM + wm * 64 + x;
+    const int b_lane = kAPieces + h * BN + wn * 128 + x;
+
+    for (uint64_t s = 0; s < steps; ++s) {
+        const int cur = (int)(s & 1);
+        if (s + 1 < steps) {
+            load_pieces<BM>(A, Rpa, K8, m0, s + 1, tid, ra);
+            load_pieces<BN>(B, Rpb, K8, n0, s + 1, tid, rb);
+        }
+        const piece* l = lds[cur];
+        piece fa[2][3];
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+#pragma unroll
+            for (int p = 0; p < 3; ++p) fa[i][p] = l[a_lane + p * 2 * BM + 32 * i];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            piece fb[3];
+#pragma unroll
+            for (int p = 0; p < 3; ++p) fb[p] = l[b_lane + p * 2 * BN + 32 * j];
+            // the six plane pairs (pa, pb) with pa + pb <= 2, smallest terms first
+            constexpr int kPa[6] = {0, 1, 2, 0, 1, 0};
+            constexpr int kPb[6] = {2, 1, 0, 1, 0, 0};
+#pragma unroll
+            for (int t6 = 0; t6 < 6; ++t6)
+#pragma unroll
+                for (int i = 0; i < 2; ++i) acc[i][j] = mfma_bf16(fa[i][kPa[t6]], fb[kPb[t6]], acc[i][j]);
+        }
+        if (s + 1 < steps) {
+            store_pieces(lds[cur ^ 1], tid, ra);
+            store_pieces(lds[cur ^ 1] + kAPieces, tid, rb);
+        }
+        __syncthreads();
+    }
+
+    // D[m][n] of a 32x32 MFMA: lane holds column n = lane % 32; register r holds row
+    // 8*(r/4) + 4*(lane/32) + r%4.
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const uint64_t row = m0 + wm * 64 + 32 * i + 8 * (r >> 2) + 4 * h + (r & 3);
+            if (row >= M) continue;
+            const float rs = row_scale ? row_scale[row] : 1.0f;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const uint64_t col = n0 + wn * 128 + 32 * j + x;
+                if (col >= N) continue;
+                float* c = C + row * ldc + col;
+                float v = alpha * acc[i][j][r];
+                if (beta != 0.0f) v += beta * *c;
+                *c = v * rs;
+            }
+        }
+    }
+}
+
+uint64_t padded_rows(uint64_t rows) { return (rows + kRowPad - 1) / kRowPad * kRowPad; }
+uint64_t octets(uint64_t K) { return (K + 15) / 16 * 2; }
+
+}  // namespace
+
+namespace trakhip {
+
+size_t split_bytes(uint64_t rows, uint64_t K) {
+    if (rows == 0 || K == 0) return 0;
+    return (size_t)(3 * octets(K) * padded_rows(rows) * 16);
+}
+
+int split_rows(const float* src, uint64_t ld, uint64_t rows, uint64_t K, int transposed, void* planes,
+               size_t planes_bytes, hipStream_t s) {
+    if (rows == 0 || K == 0) return TRAKHIP_ERR_SHAPE;
+    if (ld < (transposed ? rows : K)) return TRAKHIP_ERR_SHAPE;
+    if (!src || !planes) return TRAKHIP_ERR_NULL;
+    if (planes_bytes < split_bytes(rows, K)) return TRAKHIP_ERR_WORKSPACE;
+    if ((reinterpret_cast<uintptr_t>(src) % 4) || (reinterpret_cast<uintptr_t>(planes) % 16)) return TRAKHIP_ERR_ALIGN;
+    const uint64_t Rp = padded_rows(rows), K8 = octets(K);
+    const uint64_t gx = Rp / 64, gy = (K8 + 3) / 4;
+    if (gx * gy > 0x7FFFFFFFull) return TRAKHIP_ERR_SHAPE;
+    const dim3 grid((uint32_t)(gx * gy)), block(256);
+    uint4* out = static_cast<uint4*>(planes);
+    const bool aligned = reinterpret_cast<uintptr_t>(src) % 16 == 0 && ld % 4 == 0;
+    if (transposed)
+        hipLaunchKernelGGL((split_kernel<true, false>), grid, block, 0, s, src, ld, rows, K, Rp, K8, (uint32_t)gx, out);
+    else if (aligned)
+        hipLaunchKernelGGL((split_kernel<false, true>), grid, block, 0, s, src, ld, rows, K, Rp, K8, (uint32_t)gx, out);
+    else
+        hipLaunchKernelGGL((split_kernel<false, false>), grid, block, 0, s, src, ld, rows, K, Rp, K8, (uint32_t)gx, out);
+    return hipGetLastError() == hipSuccess ? TRAKHIP_OK : TRAKHIP_ERR_LAUNCH;
+}
+
+int gemm_nt_split(const void* A_planes, uint64_t M, const void* B_planes, uint64_t N, uint64_t K, float* C,
+                  uint64_t ldc, float alpha, float beta, const float* row_scale, hipStream_t s) {
+    if (M == 0 || N == 0) return TRAKHIP_OK;
+    if (K == 0 || ldc < N) return TRAKHIP_ERR_SHAPE;
+    if (!A_planes || !B_planes || !C) return TRAKHIP_ERR_NULL;
+    if ((reinterpret_cast<uintptr_t>(A_planes) % 16) || (reinterpret_cast<uintptr_t>(B_planes) % 16) ||
+        (reinterpret_cast<uintptr_t>(C) % 4))
+        return TRAKHIP_ERR_ALIGN;
+    const uint64_t tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
+    if (tiles_m * tiles_n > 0x7FFFFFFFull) return TRAKHIP_ERR_SHAPE;
+    hipLaunchKernelGGL(gemm_split_kernel, dim3((uint32_t)(tiles_m * tiles_n)), dim3(kThreads), 0, s,
+                       static_cast<const piece*>(A_planes), padded_rows(M), static_cast<const piece*>(B_planes),
+                       padded_rows(N), octets(K), C, ldc, M, N, alpha, beta, row_scale, (uint32_t)tiles_n);
+    return hipGetLastError() == hipSuccess ? TRAKHIP_OK : TRAKHIP_ERR_LAUNCH;
+}
+
+}  // namespace trakhip

@@ -152,6 +152,68 @@ def gemm_tn(a, b, out=None, alpha=1.0, beta=0.0):
     return out
 
 
+class SplitOperand:
+    """An fp32 matrix [rows, K] stored as three bf16 planes whose sum is the matrix exactly (the
+    operand format of `gemm_nt_split`)."""
+
+    def __init__(self, planes, rows, K):
+        self.planes, self.rows, self.K = planes, int(rows), int(K)
+
+    @property
+    def device(self):
+        return self.planes.device
+
+
+def split_rows(t, transposed=False):
+    """Splits the fp32 CUDA matrix `t` for `gemm_nt_split`.  transposed=False: the operand is `t`
+    itself ([rows, K]); transposed=True: the operand is `t.T` (t is [K, rows]), read in place."""
+    t = _as_f32_rows(t, "t")
+    if not t.is_cuda:
+        raise RuntimeError("split_rows needs a CUDA tensor")
+    rows, K = (t.shape[1], t.shape[0]) if transposed else (t.shape[0], t.shape[1])
+    lib = _lib.load()
+    nbytes = lib.trakhip_split_bytes(rows, K)
+    with torch.cuda.device(t.device):
+        planes = torch.empty(max(nbytes, 16), dtype=torch.uint8, device=t.device)
+        stream = torch.cuda.current_stream(t.device).cuda_stream
+        code = lib.trakhip_split_rows(
+            ctypes.c_void_p(t.data_ptr()), _ld(t), rows, K, int(bool(transposed)),
+            ctypes.c_void_p(planes.data_ptr()), planes.numel(), ctypes.c_void_p(stream),
+        )
+    _lib.check(code)
+    return SplitOperand(planes, rows, K)
+
+
+def gemm_nt_split(a, b, out=None, alpha=1.0, beta=0.0, row_scale=None):
+    """out[M, N] = alpha * A @ B.T + beta * out (rows optionally scaled) for SplitOperands A [M, K]
+    and B [N, K]: six bf16 MFMAs per k step with fp32 accumulation, fp32-level accuracy."""
+    if not isinstance(a, SplitOperand) or not isinstance(b, SplitOperand):
+        raise TypeError("gemm_nt_split takes SplitOperand arguments (see split_rows)")
+    if a.K != b.K or a.device != b.device:
+        raise RuntimeError("operands must share the inner dimension and the device")
+    M, N, K = a.rows, b.rows, a.K
+    if out is None:
+        out = torch.empty((M, N), dtype=torch.float32, device=a.device)
+        beta = 0.0
+    if out.dtype != torch.float32 or tuple(out.shape) != (M, N) or (N > 1 and out.stride(1) != 1) or out.device != a.device:
+        raise RuntimeError("out must be an fp32 [M, N] tensor with unit column stride on the operands' device")
+    rs = None
+    if row_scale is not None:
+        rs = row_scale.to(device=a.device, dtype=torch.float32).contiguous().reshape(-1)
+        if rs.numel() != M:
+            raise RuntimeError("row_scale must have M elements")
+    lib = _lib.load()
+    with torch.cuda.device(a.device):
+        stream = torch.cuda.current_stream(a.device).cuda_stream
+        code = lib.trakhip_gemm_nt_split(
+            ctypes.c_void_p(a.planes.data_ptr()), M, ctypes.c_void_p(b.planes.data_ptr()), N, K,
+            ctypes.c_void_p(out.data_ptr()), _ld(out), float(alpha), float(beta),
+            ctypes.c_void_p(rs.data_ptr()) if rs is not None else None, ctypes.c_void_p(stream),
+        )
+    _lib.check(code)
+    return out
+
+
 def spd_inverse(a, lambda_reg=0.0, normalize=False):
     """(a + lambda*I)^-1 for a symmetric positive definite fp32 matrix on the GPU; with
     normalize=True the result is divided by mean(|inverse|) (trak/score_computers.py:160-166).
@@ -239,7 +301,8 @@ def scores_finalize(acc, divisor, row_factor, out):
 
 
 def get_matrix_mult(features, target_grads, target_dtype=None, batch_size=8096, use_blockwise=False):
-    """features @ target_grads.T (trak/utils.py:248-294).  On the GPU this is one fp32 MFMA GEMM;
+    """features @ target_grads.T (trak/utils.py:248-294).  On the GPU this is one GEMM of fp32 accuracy
+    on the matrix cores (operands split into bf16 terms, see gemm_nt_split);
     CPU inputs take torch's matmul as in the reference (trak/utils.py:128-132).  The reference's
     blockwise host-staged variant exists to fit small GPU memories; `use_blockwise` and
     `batch_size` are accepted for signature compatibility and ignored."""
@@ -247,5 +310,5 @@ def get_matrix_mult(features, target_grads, target_dtype=None, batch_size=8096, 
         target_dtype = features.dtype
     if features.device.type == "cpu":
         return (features @ target_grads.t()).clone().to(target_dtype)
-    out = gemm_nt(features, target_grads.to(features.device))
+    out = gemm_nt_split(split_rows(features), split_rows(target_grads.to(features.device)))
     return out.to(target_dtype)
