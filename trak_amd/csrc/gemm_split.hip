@@ -29,7 +29,7 @@ typedef float floatx16 __attribute__((ext_vector_type(16)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef uint32_t piece __attribute__((ext_vector_type(4)));  // 16 bytes = 8 bf16 = one lane's MFMA operand
 
-constexpr int kThreads = 256;
+constexpr int kWavesN = 2;  // waves along N; 4 (eight waves, 64 x 64 each) measured 4 % slower
 constexpr int BM = 128, BN = 256;
 constexpr int kRowPad = 256;                       // rows of a split operand are padded to this
 constexpr int kAPieces = 3 * 2 * BM;               // 16-byte pieces of an A tile: [plane][half][row]
@@ -99,63 +99,72 @@ __device__ __forceinline__ floatx16 mfma_bf16(const piece& a, const piece& b, fl
                                                    0, 0, 0);
 }
 
-// pieces of step s (octets 2s, 2s + 1) of the tile rows [x0, x0 + ROWS): piece e = (plane, half, row)
-template <int ROWS, int N>
-__device__ __forceinline__ void load_pieces(const piece* __restrict__ planes, uint64_t Rp, uint64_t K8,
-                                            uint64_t x0, uint64_t s, int tid, piece (&r)[N]) {
+// Step s (octets 2s, 2s + 1) of a tile is 2304 pieces, [A: plane][half][128 rows] followed by
+// [B: plane][half][256 rows], moved in 36 chunks of 64 consecutive pieces by the load unit straight
+// into LDS (global_load_lds_dwordx4): the 64 lanes of a wave fetch 64 consecutive rows of one
+// (plane, octet), which land at 64 consecutive 16-byte slots starting at a wave-uniform LDS
+// address; no staging registers, no LDS store instructions.  Wave w of W moves chunks w, w + W, ...
+template <int W>
+__device__ __forceinline__ void dma_step(const piece* __restrict__ A, uint64_t Rpa, const piece* __restrict__ B,
+                                         uint64_t Rpb, uint64_t K8, uint64_t m0, uint64_t n0, uint64_t s,
+                                         int wave, int lane, piece* lds) {
+    constexpr int kChunks = kBufPieces / 64;  // 36
+    constexpr int kAChunks = kAPieces / 64;   // 12
 #pragma unroll
-    for (int i = 0; i < N; ++i) {
-        const int e = tid + kThreads * i;
-        const int row = e % ROWS, ph = e / ROWS;  // ph = plane * 2 + half
-        r[i] = planes[((uint64_t)(ph >> 1) * K8 + 2 * s + (ph & 1)) * Rp + x0 + row];
+    for (int i = 0; i < (kChunks + W - 1) / W; ++i) {
+        const int c = wave + W * i;  // wave-uniform
+        if (c >= kChunks) break;
+        const piece* src;
+        if (c < kAChunks) {
+            const int e = 64 * c + lane, row = e % BM, ph = e / BM;  // ph = plane * 2 + half
+            src = A + ((uint64_t)(ph >> 1) * K8 + 2 * s + (ph & 1)) * Rpa + m0 + row;
+        } else {
+            const int e = 64 * (c - kAChunks) + lane, row = e % BN, ph = e / BN;
+            src = B + ((uint64_t)(ph >> 1) * K8 + 2 * s + (ph & 1)) * Rpb + n0 + row;
+        }
+        __builtin_amdgcn_global_load_lds((const void __attribute__((address_space(1)))*)src,
+                                         (void __attribute__((address_space(3)))*)(lds + 64 * c), 16, 0, 0);
     }
 }
 
-template <int N>
-__device__ __forceinline__ void store_pieces(piece* lds, int tid, const piece (&r)[N]) {
-#pragma unroll
-    for (int i = 0; i < N; ++i) lds[tid + kThreads * i] = r[i];
-}
-
-__global__ __launch_bounds__(kThreads, 2) void gemm_split_kernel(
+// NW = waves side by side along N (2 or 4); two wave rows along M.  A wave owns 64 x (256 / NW) of C.
+template <int NW>
+__global__ __launch_bounds__(128 * NW, NW) void gemm_split_kernel(
     const piece* __restrict__ A, uint64_t Rpa, const piece* __restrict__ B, uint64_t Rpb, uint64_t K8,
     float* __restrict__ C, uint64_t ldc, uint64_t M, uint64_t N, float alpha, float beta,
     const float* __restrict__ row_scale, uint32_t tiles_n) {
+    constexpr int W = 2 * NW;        // waves
+    constexpr int JT = 8 / NW;       // 32-column MFMA tiles per wave
     __shared__ piece lds[2][kBufPieces];
 
     const uint32_t tile_m = blockIdx.x / tiles_n, tile_n = blockIdx.x % tiles_n;
     const uint64_t m0 = (uint64_t)tile_m * BM, n0 = (uint64_t)tile_n * BN;
     const int tid = threadIdx.x;
     const int wave = tid >> 6, lane = tid & 63;
-    const int wm = wave >> 1, wn = wave & 1;
+    const int wm = wave / NW, wn = wave % NW;
     const int x = lane & 31, h = lane >> 5;
 
-    floatx16 acc[2][4];
+    floatx16 acc[2][JT];
 #pragma unroll
     for (int i = 0; i < 2; ++i)
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
+        for (int j = 0; j < JT; ++j)
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
     const uint64_t steps = K8 / 2;
-    piece ra[kAPieces / kThreads], rb[kBPieces / kThreads];  // 3 + 6 pieces in flight per thread
-    load_pieces<BM>(A, Rpa, K8, m0, 0, tid, ra);
-    load_pieces<BN>(B, Rpb, K8, n0, 0, tid, rb);
-    store_pieces(lds[0], tid, ra);
-    store_pieces(lds[0] + kAPieces, tid, rb);
+    dma_step<W>(A, Rpa, B, Rpb, K8, m0, n0, 0, wave, lane, lds[0]);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
 
-    // piece index of this lane's operand for plane p: A rows wm*64 + 32*i + x, B rows wn*128 + 32*j + x
+    // piece index of this lane's operand for plane p: A rows wm*64 + 32*i + x, B rows wn*32*JT + 32*j + x
     const int a_lane = h * BM + wm * 64 + x;
-    const int b_lane = kAPieces + h * BN + wn * 128 + x;
+    const int b_lane = kAPieces + h * BN + wn * (32 * JT) + x;
 
     for (uint64_t s = 0; s < steps; ++s) {
         const int cur = (int)(s & 1);
-        if (s + 1 < steps) {
-            load_pieces<BM>(A, Rpa, K8, m0, s + 1, tid, ra);
-            load_pieces<BN>(B, Rpb, K8, n0, s + 1, tid, rb);
-        }
+        // the other buffer was last read before the barrier that ended the previous step
+        if (s + 1 < steps) dma_step<W>(A, Rpa, B, Rpb, K8, m0, n0, s + 1, wave, lane, lds[cur ^ 1]);
         const piece* l = lds[cur];
         piece fa[2][3];
 #pragma unroll
@@ -163,7 +172,7 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_split_kernel(
 #pragma unroll
             for (int p = 0; p < 3; ++p) fa[i][p] = l[a_lane + p * 2 * BM + 32 * i];
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
+        for (int j = 0; j < JT; ++j) {
             piece fb[3];
 #pragma unroll
             for (int p = 0; p < 3; ++p) fb[p] = l[b_lane + p * 2 * BN + 32 * j];
@@ -175,10 +184,7 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_split_kernel(
 #pragma unroll
                 for (int i = 0; i < 2; ++i) acc[i][j] = mfma_bf16(fa[i][kPa[t6]], fb[kPb[t6]], acc[i][j]);
         }
-        if (s + 1 < steps) {
-            store_pieces(lds[cur ^ 1], tid, ra);
-            store_pieces(lds[cur ^ 1] + kAPieces, tid, rb);
-        }
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wave's pieces of the next step are in LDS
         __syncthreads();
     }
 
@@ -192,8 +198,8 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_split_kernel(
             if (row >= M) continue;
             const float rs = row_scale ? row_scale[row] : 1.0f;
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const uint64_t col = n0 + wn * 128 + 32 * j + x;
+            for (int j = 0; j < JT; ++j) {
+                const uint64_t col = n0 + wn * (32 * JT) + 32 * j + x;
                 if (col >= N) continue;
                 float* c = C + row * ldc + col;
                 float v = alpha * acc[i][j][r];
@@ -248,7 +254,7 @@ int gemm_nt_split(const void* A_planes, uint64_t M, const void* B_planes, uint64
         return TRAKHIP_ERR_ALIGN;
     const uint64_t tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
     if (tiles_m * tiles_n > 0x7FFFFFFFull) return TRAKHIP_ERR_SHAPE;
-    hipLaunchKernelGGL(gemm_split_kernel, dim3((uint32_t)(tiles_m * tiles_n)), dim3(kThreads), 0, s,
+    hipLaunchKernelGGL(gemm_split_kernel<kWavesN>, dim3((uint32_t)(tiles_m * tiles_n)), dim3(128 * kWavesN), 0, s,
                        static_cast<const piece*>(A_planes), padded_rows(M), static_cast<const piece*>(B_planes),
                        padded_rows(N), octets(K), C, ldc, M, N, alpha, beta, row_scale, (uint32_t)tiles_n);
     return hipGetLastError() == hipSuccess ? TRAKHIP_OK : TRAKHIP_ERR_LAUNCH;
