@@ -101,17 +101,16 @@ __device__ __forceinline__ float4 read_frag(const float* lds, int x, int h, int 
     return v;
 }
 
+// One 128 x BN tile of C, tile number `tile` of a row-major tile grid tiles_n wide.
 template <bool AK, bool BK, bool ALIGNED, int WN>
-__global__ __launch_bounds__(kThreads, 2) void gemm_kernel(const float* __restrict__ A, uint64_t lda,
-                                                           const float* __restrict__ B, uint64_t ldb,
-                                                           float* __restrict__ C, uint64_t ldc, uint64_t M,
-                                                           uint64_t N, uint64_t K, float alpha, float beta,
-                                                           const float* __restrict__ row_scale,
-                                                           uint32_t tiles_n, uint32_t flags) {
+__device__ __forceinline__ void gemm_tile(const float* __restrict__ A, uint64_t lda, const float* __restrict__ B,
+                                          uint64_t ldb, float* __restrict__ C, uint64_t ldc, uint64_t M, uint64_t N,
+                                          uint64_t K, float alpha, float beta, const float* __restrict__ row_scale,
+                                          uint32_t tiles_n, uint32_t flags, uint32_t tile) {
     constexpr int BN = 64 * WN;  // two waves side by side, WN 32-column MFMA tiles each
     __shared__ __attribute__((aligned(16))) float lds[2][Tile<BM>::floats + Tile<BN>::floats];
 
-    const uint32_t tile_m = blockIdx.x / tiles_n, tile_n = blockIdx.x % tiles_n;
+    const uint32_t tile_m = tile / tiles_n, tile_n = tile % tiles_n;
     const uint64_t m0 = (uint64_t)tile_m * BM, n0 = (uint64_t)tile_n * BN;
     // tiles strictly above the diagonal are not needed by a caller that reads the lower triangle
     if ((flags & trakhip::kGemmLowerTilesOnly) && n0 > m0 + BM - 1) return;
@@ -197,6 +196,29 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_kernel(const float* __restri
     }
 }
 
+template <bool AK, bool BK, bool ALIGNED, int WN>
+__global__ __launch_bounds__(kThreads, 2) void gemm_kernel(const float* __restrict__ A, uint64_t lda,
+                                                           const float* __restrict__ B, uint64_t ldb,
+                                                           float* __restrict__ C, uint64_t ldc, uint64_t M,
+                                                           uint64_t N, uint64_t K, float alpha, float beta,
+                                                           const float* __restrict__ row_scale,
+                                                           uint32_t tiles_n, uint32_t flags) {
+    gemm_tile<AK, BK, ALIGNED, WN>(A, lda, B, ldb, C, ldc, M, N, K, alpha, beta, row_scale, tiles_n, flags,
+                                   blockIdx.x);
+}
+
+// Several independent products of one shape in one launch: product y = blockIdx.y works on
+// A + batch.a[y], B + batch.b[y], C + batch.c[y] (element offsets).  NN operands, 128 x 128 tiles.
+__global__ __launch_bounds__(kThreads, 2) void gemm_nn_batched_kernel(const float* __restrict__ A, uint64_t lda,
+                                                                      const float* __restrict__ B, uint64_t ldb,
+                                                                      float* __restrict__ C, uint64_t ldc, uint64_t M,
+                                                                      uint64_t N, uint64_t K, float alpha, float beta,
+                                                                      uint32_t tiles_n, trakhip::GemmBatch batch) {
+    const uint32_t y = blockIdx.y;
+    gemm_tile<false, true, true, 2>(A + batch.a[y], lda, B + batch.b[y], ldb, C + batch.c[y], ldc, M, N, K, alpha,
+                                    beta, nullptr, tiles_n, 0u, blockIdx.x);
+}
+
 template <bool AK, bool BK, int WN>
 int launch_tiles(const float* A, uint64_t lda, const float* B, uint64_t ldb, float* C, uint64_t ldc, uint64_t M,
                  uint64_t N, uint64_t K, float alpha, float beta, const float* row_scale, bool aligned,
@@ -247,6 +269,23 @@ int gemm_tn(const float* A, uint64_t lda, const float* B, uint64_t ldb, float* C
 int gemm_nn(const float* A, uint64_t lda, const float* B, uint64_t ldb, float* C, uint64_t ldc, uint64_t M,
             uint64_t N, uint64_t K, float alpha, float beta, hipStream_t s, uint32_t flags) {
     return launch<false, true>(A, lda, B, ldb, C, ldc, M, N, K, alpha, beta, nullptr, flags, s);
+}
+
+int gemm_nn_batched(const float* A, uint64_t lda, const float* B, uint64_t ldb, float* C, uint64_t ldc, uint64_t M,
+                    uint64_t N, uint64_t K, float alpha, float beta, const GemmBatch& batch, hipStream_t s) {
+    if (M == 0 || N == 0 || batch.count == 0) return TRAKHIP_OK;
+    if (!A || !B || !C) return TRAKHIP_ERR_NULL;
+    if (batch.count > kGemmBatchMax || lda < K || ldb < N || ldc < N) return TRAKHIP_ERR_SHAPE;
+    // the batched kernel uses 16-byte loads: every operand start and pitch must allow them
+    if ((reinterpret_cast<uintptr_t>(A) % 16) || (reinterpret_cast<uintptr_t>(B) % 16) || (lda % 4) || (ldb % 4))
+        return TRAKHIP_ERR_ALIGN;
+    for (uint32_t y = 0; y < batch.count; ++y)
+        if ((batch.a[y] % 4) || (batch.b[y] % 4)) return TRAKHIP_ERR_ALIGN;
+    const uint64_t tm = (M + BM - 1) / BM, tn = (N + 127) / 128;
+    if (tm * tn > 0x7FFFFFFFull) return TRAKHIP_ERR_SHAPE;
+    hipLaunchKernelGGL(gemm_nn_batched_kernel, dim3((uint32_t)(tm * tn), batch.count), dim3(kThreads), 0, s, A, lda, B,
+                       ldb, C, ldc, M, N, K, alpha, beta, (uint32_t)tn, batch);
+    return hipGetLastError() == hipSuccess ? TRAKHIP_OK : TRAKHIP_ERR_LAUNCH;
 }
 
 }  // namespace trakhip

@@ -16,6 +16,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <vector>
+
 #include "trakhip_internal.h"
 
 namespace {
@@ -45,15 +47,18 @@ __global__ __launch_bounds__(256) void spd_init_kernel(const float* __restrict__
 // One workgroup of 1024 threads: Cholesky of the 128x128 diagonal block at W (lower triangle
 // used), L block to Lout (upper part zero), its inverse to Linv_out.
 //
-// The block lives in registers, 4 x 4 elements per thread, cyclically distributed so that every
-// thread stays busy as the active part shrinks (four waves per SIMD hide the issue latency of this
-// strictly sequential algorithm).  Step k of the right-looking factorization broadcasts column k
-// of L through LDS and applies the rank-1 update A -= l l^T from registers; the inverse runs the
-// same way on B = I:  X[k, :] = B[k, :] / L[k, k], then B[r, :] -= L[r, k] X[k, :] for r > k.
-// Ownership is chosen so that the threads that publish a column (factorization) or a row
-// (inverse) form half of ONE wave: thread t holds rows t % 32 + 32 i and columns t / 32 + 32 j
-// while factoring, and the transpose of that while inverting.  Updates are not masked: entries of
-// rows or columns <= k are never read again once step k is over, so what lands there is ignored.
+// Both matrices live in registers, 4 x 4 elements per thread each, cyclically distributed so that
+// every thread stays busy as the active part shrinks (four waves per SIMD hide the issue latency of
+// this strictly sequential algorithm).  One loop of 128 steps, one barrier per step, does both
+// jobs: step k broadcasts the unscaled column k of the trailing matrix A (l_k = raw / sqrt(d),
+// d = A[k][k]) and the unscaled row k of B (B starts as I; x_k = B[k, :] / L[k][k] is row k of
+// L^-1) through LDS, then every thread applies
+//     A[r][c] -= raw[r] raw[c] / d                         (right-looking Cholesky)
+//     B[r][c] -= raw[r] Braw[c] / d    for r > k           (forward substitution on all columns)
+// from registers.  Thread t holds A rows t % 32 + 32 i, columns t / 32 + 32 j, and the transpose of
+// that for B, so the threads that publish column k of A and row k of B are the same half of ONE
+// wave.  A updates are not masked: entries of rows or columns <= k are never read again once step
+// k is over.  Rows <= k of B are finished rows of L^-1 and are kept.
 constexpr int kDiagGrid = 32;              // threads per side
 constexpr int kDiagTile = NB / kDiagGrid;  // 4 elements per side per thread
 
@@ -63,32 +68,39 @@ __global__ __launch_bounds__(1024) void spd_diag_kernel(const float* __restrict_
                                                         int32_t* __restrict__ status) {
     constexpr int G = kDiagGrid, T = kDiagTile;
     __shared__ float Ls[NB * kLd];   // the finished factor, column k valid after step k
-    __shared__ float vec[2][NB];     // broadcast buffers (two, so the steps can overlap safely)
+    // column k of A and row k of B, unscaled; entry x = t + 32 i is kept at slot 4 t + i, so the four
+    // values a thread needs are one 16-byte LDS access (two buffers, so the steps can overlap safely)
+    __shared__ __attribute__((aligned(16))) float vec[2][NB];
+    __shared__ __attribute__((aligned(16))) float bvec[2][NB];
     __shared__ float pivot[2];
     const int tid = threadIdx.x;
     const int p = tid % G, q = tid / G;  // p varies inside a half-wave, q selects the half-wave
 
-    // ---- factorization: rows p + G i, columns q + G j ------------------------------------------
-    float a[T][T];
+    float a[T][T], b[T][T];  // A: rows p + G i, columns q + G j;  B: rows q + G i, columns p + G j
 #pragma unroll
     for (int i = 0; i < T; ++i)
 #pragma unroll
         for (int j = 0; j < T; ++j) {
             const int r = p + G * i, c = q + G * j;
             a[i][j] = (c <= r) ? W[(uint64_t)r * ldw + c] : 0.0f;
+            b[i][j] = (q + G * i == p + G * j) ? 1.0f : 0.0f;
         }
 
     for (int k = 0; k < NB; ++k) {
         const int buf = k & 1;
-        const int ks = k / G, kt = k % G;  // column k: threads with q == kt, slot [*][ks]
+        const int ks = k / G, kt = k % G;  // column k of A and row k of B: threads with q == kt, slot ks
         if (q == kt) {                     // one half-wave
-            float col[T];
+            float col[T], row[T];
 #pragma unroll
             for (int i = 0; i < T; ++i) {
                 col[i] = 0.0f;
+                row[i] = 0.0f;
 #pragma unroll
                 for (int j = 0; j < T; ++j)
-                    if (j == ks) col[i] = a[i][j];
+                    if (j == ks) {
+                        col[i] = a[i][j];
+                        row[i] = b[j][i];
+                    }
             }
             if (p == kt) {  // the diagonal element (k, k) is in slot [ks][ks] of this thread
                 float d = 0.0f;
@@ -101,73 +113,48 @@ __global__ __launch_bounds__(1024) void spd_diag_kernel(const float* __restrict_
                 }
                 pivot[buf] = d;
             }
-#pragma unroll
-            for (int i = 0; i < T; ++i) vec[buf][p + G * i] = col[i];  // unscaled column
+            *reinterpret_cast<float4*>(&vec[buf][T * p]) = make_float4(col[0], col[1], col[2], col[3]);
+            *reinterpret_cast<float4*>(&bvec[buf][T * p]) = make_float4(row[0], row[1], row[2], row[3]);
         }
         __syncthreads();
         const float d = pivot[buf];
-        const float inv_d = 1.0f / d;
-        if (q == kt) {  // the finished column of L, off the critical path of the other waves
+        // hardware reciprocal (1 ulp): it only scales the rank-1 updates; the factor itself below
+        // is scaled with the correctly rounded 1 / sqrt(d)
+        const float inv_d = __builtin_amdgcn_rcpf(d);
+        const float4 vp = *reinterpret_cast<const float4*>(&vec[buf][T * p]);
+        const float4 vq = *reinterpret_cast<const float4*>(&vec[buf][T * q]);
+        const float4 bp = *reinterpret_cast<const float4*>(&bvec[buf][T * p]);
+        const float lr[T] = {vp.x, vp.y, vp.z, vp.w};
+        const float xc[T] = {bp.x, bp.y, bp.z, bp.w};
+        const float rq[T] = {vq.x, vq.y, vq.z, vq.w};
+        if (q == kt) {  // finished column k of L and row k of L^-1, off the critical path of the other waves
             const float inv_sd = 1.0f / sqrtf(d);
 #pragma unroll
             for (int i = 0; i < T; ++i) {
                 const int r = p + G * i;
-                Ls[r * kLd + k] = (r >= k) ? vec[buf][r] * inv_sd : 0.0f;  // L[k][k] = d / sqrt(d)
+                Ls[r * kLd + k] = (r >= k) ? lr[i] * inv_sd : 0.0f;  // L[k][k] = d / sqrt(d)
+                const float x = xc[i] * inv_sd;
+#pragma unroll
+                for (int j = 0; j < T; ++j)
+                    if (j == ks) b[j][i] = x;
             }
         }
-        // A[r][c] -= raw[r] * raw[c] / d
-        float lr[T], lc[T];
+        float lc[T], br[T];
 #pragma unroll
-        for (int i = 0; i < T; ++i) lr[i] = vec[buf][p + G * i];
-#pragma unroll
-        for (int j = 0; j < T; ++j) lc[j] = vec[buf][q + G * j] * inv_d;
+        for (int j = 0; j < T; ++j) {
+            const float v = rq[j] * inv_d;
+            lc[j] = v;
+            br[j] = (q + G * j > k) ? v : 0.0f;  // rows <= k of B are finished
+        }
 #pragma unroll
         for (int i = 0; i < T; ++i)
-#pragma unroll
-            for (int j = 0; j < T; ++j) a[i][j] -= lr[i] * lc[j];
-    }
-    __syncthreads();
-
-    // ---- inverse of L: rows q + G i, columns p + G j (transposed ownership) --------------------
-    float b[T][T];
-#pragma unroll
-    for (int i = 0; i < T; ++i)
-#pragma unroll
-        for (int j = 0; j < T; ++j) b[i][j] = (q + G * i == p + G * j) ? 1.0f : 0.0f;
-
-    for (int k = 0; k < NB; ++k) {
-        const int buf = k & 1;
-        const int ks = k / G, kt = k % G;  // row k: threads with q == kt, slot [ks][*]
-        if (q == kt) {
-            const float inv_d = 1.0f / Ls[k * kLd + k];
 #pragma unroll
             for (int j = 0; j < T; ++j) {
-                float v = 0.0f;
-#pragma unroll
-                for (int i = 0; i < T; ++i)
-                    if (i == ks) v = b[i][j];
-                v *= inv_d;
-#pragma unroll
-                for (int i = 0; i < T; ++i)
-                    if (i == ks) b[i][j] = v;
-                vec[buf][p + G * j] = v;
+                a[i][j] -= lr[i] * lc[j];
+                b[i][j] -= br[i] * xc[j];
             }
-        }
-        __syncthreads();
-        // B[r][c] -= L[r][k] * X[k][c] for r > k (rows <= k keep their finished values)
-        float lr[T], xc[T];
-#pragma unroll
-        for (int i = 0; i < T; ++i) {
-            const int r = q + G * i;
-            lr[i] = (r > k) ? Ls[r * kLd + k] : 0.0f;
-        }
-#pragma unroll
-        for (int j = 0; j < T; ++j) xc[j] = vec[buf][p + G * j];
-#pragma unroll
-        for (int i = 0; i < T; ++i)
-#pragma unroll
-            for (int j = 0; j < T; ++j) b[i][j] -= lr[i] * xc[j];
     }
+    __syncthreads();
 
 #pragma unroll
     for (int i = 0; i < T; ++i)
@@ -229,26 +216,59 @@ struct Ctx {
     float* Li;
     uint64_t np;
     hipStream_t s;
-    int err;
 };
 
-// Li[lo:hi, lo:hi] (block units) becomes the inverse of L[lo:hi, lo:hi]; diagonal blocks are
-// already inverted.
-void tri_inverse(Ctx& c, uint64_t lo, uint64_t hi) {
-    if (c.err || hi - lo <= 1) return;
+// Inverse of the block lower-triangular factor by recursive halving:
+//   [A 0; B C]^-1 = [A^-1 0; -C^-1 B A^-1  C^-1],
+// two products per node of the tree (T = B A^-1 into W, which is free once the factorization is
+// done, then -C^-1 T into Li).  Diagonal blocks are already inverted.  Nodes of one depth are
+// independent, so they are collected per depth and every group of equal shape goes out as one
+// batched launch: a dozen launches instead of two per node.
+struct Node {
+    uint64_t lo, mid, hi;  // block units
+};
+
+void collect_nodes(uint64_t lo, uint64_t hi, size_t depth, std::vector<std::vector<Node>>& levels) {
+    if (hi - lo <= 1) return;
     const uint64_t mid = lo + (hi - lo) / 2;
-    tri_inverse(c, lo, mid);
-    tri_inverse(c, mid, hi);
-    const uint64_t r = (hi - mid) * NB, q = (mid - lo) * NB;
+    if (levels.size() <= depth) levels.resize(depth + 1);
+    levels[depth].push_back({lo, mid, hi});
+    collect_nodes(lo, mid, depth + 1, levels);
+    collect_nodes(mid, hi, depth + 1, levels);
+}
+
+int tri_inverse(Ctx& c, uint64_t nblk) {
+    std::vector<std::vector<Node>> levels;
+    collect_nodes(0, nblk, 0, levels);
     const uint64_t np = c.np;
-    const float* B = c.L + mid * NB * np + lo * NB;
-    const float* Ainv = c.Li + lo * NB * np + lo * NB;
-    const float* Cinv = c.Li + mid * NB * np + mid * NB;
-    float* T = c.W + mid * NB * np + lo * NB;  // W is free once the factorization is done
-    float* out = c.Li + mid * NB * np + lo * NB;
-    int e = trakhip::gemm_nn(B, np, Ainv, np, T, np, r, q, q, 1.0f, 0.0f, c.s);
-    if (!e) e = trakhip::gemm_nn(Cinv, np, T, np, out, np, r, q, r, -1.0f, 0.0f, c.s);
-    if (e) c.err = e;
+    for (size_t d = levels.size(); d-- > 0;) {  // children before parents
+        std::vector<Node>& nodes = levels[d];
+        std::vector<char> done(nodes.size(), 0);
+        for (size_t first = 0; first < nodes.size(); ++first) {
+            if (done[first]) continue;
+            const uint64_t r = (nodes[first].hi - nodes[first].mid) * NB, q = (nodes[first].mid - nodes[first].lo) * NB;
+            trakhip::GemmBatch t_of_b, out_of_t;  // T = B * Ainv;  out = -Cinv * T
+            t_of_b.count = out_of_t.count = 0;
+            for (size_t i = first; i < nodes.size() && t_of_b.count < trakhip::kGemmBatchMax; ++i) {
+                const Node& n = nodes[i];
+                if (done[i] || (n.hi - n.mid) * NB != r || (n.mid - n.lo) * NB != q) continue;
+                done[i] = 1;
+                const uint32_t y = t_of_b.count++;
+                out_of_t.count = t_of_b.count;
+                const uint64_t below = n.mid * NB * np + n.lo * NB;  // block (mid, lo)
+                t_of_b.a[y] = below;                                // B      in L
+                t_of_b.b[y] = n.lo * NB * np + n.lo * NB;           // A^-1   in Li
+                t_of_b.c[y] = below;                                // T      in W
+                out_of_t.a[y] = n.mid * NB * np + n.mid * NB;       // C^-1   in Li
+                out_of_t.b[y] = below;                              // T      in W
+                out_of_t.c[y] = below;                              // result in Li
+            }
+            int e = trakhip::gemm_nn_batched(c.L, np, c.Li, np, c.W, np, r, q, q, 1.0f, 0.0f, t_of_b, c.s);
+            if (!e) e = trakhip::gemm_nn_batched(c.Li, np, c.W, np, c.Li, np, r, q, r, -1.0f, 0.0f, out_of_t, c.s);
+            if (e) return e;
+        }
+    }
+    return TRAKHIP_OK;
 }
 
 }  // namespace
@@ -298,13 +318,13 @@ int spd_inverse(const float* A, uint64_t lda, float lambda, float* inv, uint64_t
         if (e) return e;
     }
 
-    Ctx c = {W, L, Li, np, s, 0};
-    tri_inverse(c, 0, nblk);
-    if (c.err) return c.err;
+    Ctx c = {W, L, Li, np, s};
+    int e = tri_inverse(c, nblk);
+    if (e) return e;
 
     // inverse = Li^T * Li (rows of Li at or beyond n do not reach the leading n x n block)
     // Li is lower triangular: Li[k][m] = 0 for k < m, so the sum over k starts at max(m, n)
-    int e = gemm_tn(Li, np, Li, np, inv, ldi, n, n, n, 1.0f, 0.0f, s, kGemmKFromDiagonal);
+    e = gemm_tn(Li, np, Li, np, inv, ldi, n, n, n, 1.0f, 0.0f, s, kGemmKFromDiagonal);
     if (e) return e;
 
     if (normalize || mean_abs) {

@@ -34,6 +34,15 @@ int materialize_host(uint32_t seed, uint32_t num_feature_tiles, uint64_t P, uint
 constexpr uint32_t kGemmLowerTilesOnly = 1u;  // skip output tiles strictly above the diagonal
 constexpr uint32_t kGemmKFromDiagonal = 2u;   // start the k sum at max(tile row origin, tile column origin)
 
+// up to kGemmBatchMax products of one shape in one launch: element offsets of each product's operands
+constexpr uint32_t kGemmBatchMax = 32;
+struct GemmBatch {
+    uint32_t count;
+    uint64_t a[kGemmBatchMax], b[kGemmBatchMax], c[kGemmBatchMax];
+};
+int gemm_nn_batched(const float* A, uint64_t lda, const float* B, uint64_t ldb, float* C, uint64_t ldc, uint64_t M,
+                    uint64_t N, uint64_t K, float alpha, float beta, const GemmBatch& batch, hipStream_t s);
+
 int gemm_nt(const float* A, uint64_t lda, const float* B, uint64_t ldb, float* C, uint64_t ldc, uint64_t M,
             uint64_t N, uint64_t K, float alpha, float beta, const float* row_scale, hipStream_t s,
             uint32_t flags = 0);
