@@ -79,6 +79,19 @@ def test_spd_inverse(gpu, n, lam):
     assert np.abs(prod - np.eye(n)).max() < 1e-3
 
 
+def test_spd_inverse_many_blocks(gpu):
+    # 67 diagonal blocks: more tree nodes of one shape than one batched launch takes, odd block counts
+    n, lam = 8500, 1e-2
+    gen = torch.Generator(device=gpu).manual_seed(8500)
+    X = torch.randn(3 * n, n, generator=gen, device=gpu) / math.sqrt(n)
+    a = (X.double().T @ X.double()).float()
+    inv, mean_abs = spd_inverse(a, lambda_reg=lam, normalize=True)
+    a64 = a.double() + lam * torch.eye(n, device=gpu, dtype=torch.float64)
+    resid = a64 @ (inv.double() * mean_abs.double()) - torch.eye(n, device=gpu, dtype=torch.float64)
+    assert float(resid.abs().max()) < 1e-4
+    assert float((inv - inv.T).abs().max()) <= 1e-5 * float(inv.abs().max())
+
+
 def test_spd_inverse_closed_forms_and_failure(gpu):
     d = torch.arange(1, 201, dtype=torch.float32)
     inv, _ = spd_inverse(torch.diag(d * d).to(gpu), lambda_reg=0.5)
