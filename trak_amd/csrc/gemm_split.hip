@@ -15,9 +15,11 @@
 // the MFMA (8 consecutive k of one row), consecutive rows are consecutive pieces, so global loads,
 // LDS writes and LDS reads are all linear and conflict free, and the GEMM kernel moves bf16 only.
 //
-// Workgroup = 256 threads = 4 waves (2 x 2), 128 x 256 tile of C, k step 16 (one MFMA deep), two
-// LDS buffers of 36 KB, one barrier per step; a wave owns 64 x 128 of C (128 accumulator VGPRs)
-// and issues 48 MFMAs per step.
+// Workgroup = 512 threads = 8 waves (4 x 2), 256 x 256 tile of C, k step 16 (one MFMA deep), two
+// LDS buffers of 48 KB filled by LDS-direct loads, one barrier per step; a wave owns 64 x 128 of C
+// (128 accumulator VGPRs) and issues 48 MFMAs per step.  Measured against this: 128 x 256 tiles with
+// two workgroups per CU (9 % slower), 64 x 64 wave tiles at four waves per SIMD, three LDS buffers,
+// register-staged loads, super-tile orders per XCD (all slower or equal).
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
@@ -29,12 +31,11 @@ typedef float floatx16 __attribute__((ext_vector_type(16)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef uint32_t piece __attribute__((ext_vector_type(4)));  // 16 bytes = 8 bf16 = one lane's MFMA operand
 
-constexpr int kWavesN = 2;  // waves along N; 4 (eight waves, 64 x 64 each) measured 4 % slower
-constexpr int BM = 128, BN = 256;
+constexpr int kWavesN = 2;                         // waves side by side: each owns 64 x 128 of C
+constexpr int BN = 256;
 constexpr int kRowPad = 256;                       // rows of a split operand are padded to this
-constexpr int kAPieces = 3 * 2 * BM;               // 16-byte pieces of an A tile: [plane][half][row]
-constexpr int kBPieces = 3 * 2 * BN;
-constexpr int kBufPieces = kAPieces + kBPieces;    // 2304 pieces = 36 KB
+constexpr int kBPieces = 3 * 2 * BN;               // 16-byte pieces of a B tile: [plane][half][row]
+constexpr int kWavesM = 4;                         // wave rows: the C tile has 64 * kWavesM = 256 rows
 
 // ---- splitting -----------------------------------------------------------------------------
 
@@ -99,17 +100,18 @@ __device__ __forceinline__ floatx16 mfma_bf16(const piece& a, const piece& b, fl
                                                    0, 0, 0);
 }
 
-// Step s (octets 2s, 2s + 1) of a tile is 2304 pieces, [A: plane][half][128 rows] followed by
-// [B: plane][half][256 rows], moved in 36 chunks of 64 consecutive pieces by the load unit straight
+// Step s (octets 2s, 2s + 1) of a tile is 6 * (BM + 256) pieces, [A: plane][half][BM rows] followed
+// by [B: plane][half][256 rows], moved in chunks of 64 consecutive pieces by the load unit straight
 // into LDS (global_load_lds_dwordx4): the 64 lanes of a wave fetch 64 consecutive rows of one
 // (plane, octet), which land at 64 consecutive 16-byte slots starting at a wave-uniform LDS
 // address; no staging registers, no LDS store instructions.  Wave w of W moves chunks w, w + W, ...
-template <int W>
+template <int W, int BM>
 __device__ __forceinline__ void dma_step(const piece* __restrict__ A, uint64_t Rpa, const piece* __restrict__ B,
                                          uint64_t Rpb, uint64_t K8, uint64_t m0, uint64_t n0, uint64_t s,
                                          int wave, int lane, piece* lds) {
-    constexpr int kChunks = kBufPieces / 64;  // 36
-    constexpr int kAChunks = kAPieces / 64;   // 12
+    constexpr int kAPieces = 3 * 2 * BM;
+    constexpr int kChunks = (kAPieces + kBPieces) / 64;
+    constexpr int kAChunks = kAPieces / 64;
 #pragma unroll
     for (int i = 0; i < (kChunks + W - 1) / W; ++i) {
         const int c = wave + W * i;  // wave-uniform
@@ -128,13 +130,16 @@ __device__ __forceinline__ void dma_step(const piece* __restrict__ A, uint64_t R
 }
 
 // NW = waves side by side along N (2 or 4); two wave rows along M.  A wave owns 64 x (256 / NW) of C.
-template <int NW>
-__global__ __launch_bounds__(128 * NW, NW) void gemm_split_kernel(
+template <int MW, int NW>
+__global__ __launch_bounds__(64 * MW * NW, 2) void gemm_split_kernel(
     const piece* __restrict__ A, uint64_t Rpa, const piece* __restrict__ B, uint64_t Rpb, uint64_t K8,
     float* __restrict__ C, uint64_t ldc, uint64_t M, uint64_t N, float alpha, float beta,
     const float* __restrict__ row_scale, uint32_t tiles_n) {
-    constexpr int W = 2 * NW;        // waves
+    constexpr int W = MW * NW;       // waves
     constexpr int JT = 8 / NW;       // 32-column MFMA tiles per wave
+    constexpr int BM = 64 * MW;
+    constexpr int kAPieces = 3 * 2 * BM;             // [plane][half][row]
+    constexpr int kBufPieces = kAPieces + kBPieces;  // 256 x 256 tile: 3072 pieces = 48 KB
     __shared__ piece lds[2][kBufPieces];
 
     const uint32_t tile_m = blockIdx.x / tiles_n, tile_n = blockIdx.x % tiles_n;
@@ -153,7 +158,7 @@ __global__ __launch_bounds__(128 * NW, NW) void gemm_split_kernel(
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
     const uint64_t steps = K8 / 2;
-    dma_step<W>(A, Rpa, B, Rpb, K8, m0, n0, 0, wave, lane, lds[0]);
+    dma_step<W, BM>(A, Rpa, B, Rpb, K8, m0, n0, 0, wave, lane, lds[0]);
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
 
@@ -164,7 +169,7 @@ __global__ __launch_bounds__(128 * NW, NW) void gemm_split_kernel(
     for (uint64_t s = 0; s < steps; ++s) {
         const int cur = (int)(s & 1);
         // the other buffer was last read before the barrier that ended the previous step
-        if (s + 1 < steps) dma_step<W>(A, Rpa, B, Rpb, K8, m0, n0, s + 1, wave, lane, lds[cur ^ 1]);
+        if (s + 1 < steps) dma_step<W, BM>(A, Rpa, B, Rpb, K8, m0, n0, s + 1, wave, lane, lds[cur ^ 1]);
         const piece* l = lds[cur];
         piece fa[2][3];
 #pragma unroll
@@ -252,9 +257,11 @@ int gemm_nt_split(const void* A_planes, uint64_t M, const void* B_planes, uint64
     if ((reinterpret_cast<uintptr_t>(A_planes) % 16) || (reinterpret_cast<uintptr_t>(B_planes) % 16) ||
         (reinterpret_cast<uintptr_t>(C) % 4))
         return TRAKHIP_ERR_ALIGN;
+    constexpr int BM = 64 * kWavesM;
     const uint64_t tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
     if (tiles_m * tiles_n > 0x7FFFFFFFull) return TRAKHIP_ERR_SHAPE;
-    hipLaunchKernelGGL(gemm_split_kernel<kWavesN>, dim3((uint32_t)(tiles_m * tiles_n)), dim3(128 * kWavesN), 0, s,
+    hipLaunchKernelGGL((gemm_split_kernel<kWavesM, kWavesN>), dim3((uint32_t)(tiles_m * tiles_n)),
+                       dim3(64 * kWavesM * kWavesN), 0, s,
                        static_cast<const piece*>(A_planes), padded_rows(M), static_cast<const piece*>(B_planes),
                        padded_rows(N), octets(K), C, ldc, M, N, alpha, beta, row_scale, (uint32_t)tiles_n);
     return hipGetLastError() == hipSuccess ? TRAKHIP_OK : TRAKHIP_ERR_LAUNCH;
