@@ -156,6 +156,14 @@ int trakhip_gemm_nt_split(const void* A_planes_dev, uint64_t M, const void* B_pl
                           float* C_dev, uint64_t ldc, float alpha, float beta, const float* row_scale_dev,
                           void* stream);
 
+/* C[N, N] = alpha * A * A^T + beta * C for one split operand A [N, K]: only the tiles that touch
+ * the lower triangle are computed (half the work of trakhip_gemm_nt_split), then the strict upper
+ * triangle is overwritten with the mirror image of the lower one, so C is exactly symmetric.  With
+ * beta != 0, C must have been produced the same way.  Stands in for the `block.T @ block`
+ * accumulation of trak/score_computers.py:145-155 (A = the split of block^T). */
+int trakhip_gram_split(const void* A_planes_dev, uint64_t N, uint64_t K, float* C_dev, uint64_t ldc, float alpha,
+                       float beta, void* stream);
+
 /* out[i, j] = cast((acc[i, j] / divisor) * row_factor[i]) for the [N, M] fp32 score sums that
  * trakhip_gemm_nt accumulated over checkpoints (beta = 1): the closing expression of
  * TRAKer.finalize_scores, `(_scores / n) * (_avg_out_to_losses / n)` (trak/traker.py:670-678), with

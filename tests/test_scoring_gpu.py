@@ -9,7 +9,7 @@ import torch
 
 from oracle import score_oracle as so
 from trak_amd import BasicScoreComputer, get_matrix_mult
-from trak_amd.utils import gemm_nt, gemm_nt_split, gemm_tn, spd_inverse, split_rows
+from trak_amd.utils import gemm_nt, gemm_nt_split, gemm_tn, gram_split, spd_inverse, split_rows
 
 pytestmark = pytest.mark.gpu
 
@@ -158,6 +158,25 @@ def test_gemm_nt_split(gpu, M, N, K):
     assert float(wide[:, :2].abs().sum()) == 0 and float(wide[:, 2 + N :].abs().sum()) == 0
 
 
+@pytest.mark.parametrize("N,K", [(1, 1), (100, 37), (256, 64), (257, 300), (700, 1030)])
+def test_gram_split_is_symmetric_and_accumulates(gpu, N, K):
+    gen = torch.Generator(device="cpu").manual_seed(N + K)
+    x = torch.randn(K, N, generator=gen)                      # the operand is x^T, as in X^T X
+    want = x.double().numpy().T @ x.double().numpy()
+    op = split_rows(x.to(gpu), transposed=True)
+    got = gram_split(op)
+    assert torch.equal(got, got.T)
+    assert rel_max(got.cpu().numpy(), want) < gemm_tol(K)
+    full = gemm_nt_split(op, op)
+    assert torch.equal(torch.tril(got), torch.tril(full))     # the same tiles, the same arithmetic
+    again = gram_split(op, out=got.clone(), alpha=0.5, beta=1.0)
+    assert torch.equal(again, again.T)
+    assert rel_max(again.cpu().numpy(), 1.5 * want) < gemm_tol(K)
+    wide = torch.full((N, N + 3), 7.0, device=gpu)
+    gram_split(op, out=wide[:, 1 : 1 + N])
+    assert torch.equal(wide[:, 1 : 1 + N], got) and float((wide[:, 0] - 7).abs().sum()) == 0
+
+
 def test_gemm_nt_split_keeps_small_terms(gpu):
     # b = 1 + 2^-20 needs 21 significand bits: one bf16 term (8 bits) would return exactly K, the
     # split product returns K * (1 + 2^-20) to fp32 accuracy (K small enough that the running sum
@@ -220,10 +239,7 @@ def test_full_size_scoring_shape(gpu, gemm):
     otl = torch.rand(N, generator=gen, device=gpu)
     sc = BasicScoreComputer(dtype=torch.float32, device="cuda:0", lambda_reg=lam, gemm=gemm)
     xtx = sc.get_xtx(X)
-    # the fp32 instruction sums both triangles in the same order; the split product adds the cross
-    # terms a1*b2 and a2*b1 in the opposite order for (i, j) and (j, i): equal to the last bits only
-    # (the inverse reads the lower triangle)
-    assert torch.equal(xtx, xtx.T) if gemm == "fp32" else float((xtx - xtx.T).abs().max()) <= 2e-6 * float(xtx.abs().max())
+    assert torch.equal(xtx, xtx.T)
     trace64 = float((X.double() ** 2).sum())
     # fp32 accumulation over 50 000 positive terms: the bound the GEMM tests use, not better
     assert abs(float(xtx.double().diagonal().sum()) - trace64) < gemm_tol(N) * trace64

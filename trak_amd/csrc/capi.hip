@@ -107,6 +107,11 @@ int trakhip_gemm_nt_split(const void* A_planes_dev, uint64_t M, const void* B_pl
                                   static_cast<hipStream_t>(stream));
 }
 
+int trakhip_gram_split(const void* A_planes_dev, uint64_t N, uint64_t K, float* C_dev, uint64_t ldc, float alpha,
+                       float beta, void* stream) {
+    return trakhip::gram_split(A_planes_dev, N, K, C_dev, ldc, alpha, beta, static_cast<hipStream_t>(stream));
+}
+
 size_t trakhip_spd_inverse_workspace(uint64_t n) { return trakhip::spd_inverse_workspace_bytes(n); }
 
 int trakhip_spd_inverse(const float* A_dev, uint64_t lda, float lambda, float* inv_dev, uint64_t ldi,

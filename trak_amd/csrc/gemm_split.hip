@@ -134,7 +134,7 @@ template <int MW, int NW>
 __global__ __launch_bounds__(64 * MW * NW, 2) void gemm_split_kernel(
     const piece* __restrict__ A, uint64_t Rpa, const piece* __restrict__ B, uint64_t Rpb, uint64_t K8,
     float* __restrict__ C, uint64_t ldc, uint64_t M, uint64_t N, float alpha, float beta,
-    const float* __restrict__ row_scale, uint32_t tiles_n) {
+    const float* __restrict__ row_scale, uint32_t tiles_n, uint32_t flags) {
     constexpr int W = MW * NW;       // waves
     constexpr int JT = 8 / NW;       // 32-column MFMA tiles per wave
     constexpr int BM = 64 * MW;
@@ -144,6 +144,8 @@ __global__ __launch_bounds__(64 * MW * NW, 2) void gemm_split_kernel(
 
     const uint32_t tile_m = blockIdx.x / tiles_n, tile_n = blockIdx.x % tiles_n;
     const uint64_t m0 = (uint64_t)tile_m * BM, n0 = (uint64_t)tile_n * BN;
+    // a symmetric product needs only the tiles that touch the lower triangle
+    if ((flags & trakhip::kGemmLowerTilesOnly) && n0 > m0 + BM - 1) return;
     const int tid = threadIdx.x;
     const int wave = tid >> 6, lane = tid & 63;
     const int wm = wave / NW, wn = wave % NW;
@@ -215,6 +217,26 @@ __global__ __launch_bounds__(64 * MW * NW, 2) void gemm_split_kernel(
     }
 }
 
+// C[i][j] = C[j][i] for j > i: completes a symmetric matrix whose lower triangle was computed.
+__global__ __launch_bounds__(256) void mirror_lower_kernel(float* __restrict__ C, uint64_t ldc, uint64_t n) {
+    __shared__ float t[32][33];
+    // 32 x 32 blocks strictly above or on the diagonal, read from their mirror image
+    const uint32_t bi = blockIdx.y, bj = blockIdx.x;
+    if (bj < bi) return;
+    const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;
+#pragma unroll
+    for (int r = ty; r < 32; r += 8) {
+        const uint64_t src_row = (uint64_t)bj * 32 + r, src_col = (uint64_t)bi * 32 + tx;  // block (bj, bi), lower
+        t[r][tx] = (src_row < n && src_col < n) ? C[src_row * ldc + src_col] : 0.0f;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int r = ty; r < 32; r += 8) {
+        const uint64_t row = (uint64_t)bi * 32 + r, col = (uint64_t)bj * 32 + tx;
+        if (row < n && col < n && col > row) C[row * ldc + col] = t[tx][r];
+    }
+}
+
 uint64_t padded_rows(uint64_t rows) { return (rows + kRowPad - 1) / kRowPad * kRowPad; }
 uint64_t octets(uint64_t K) { return (K + 15) / 16 * 2; }
 
@@ -250,7 +272,7 @@ int split_rows(const float* src, uint64_t ld, uint64_t rows, uint64_t K, int tra
 }
 
 int gemm_nt_split(const void* A_planes, uint64_t M, const void* B_planes, uint64_t N, uint64_t K, float* C,
-                  uint64_t ldc, float alpha, float beta, const float* row_scale, hipStream_t s) {
+                  uint64_t ldc, float alpha, float beta, const float* row_scale, hipStream_t s, uint32_t flags) {
     if (M == 0 || N == 0) return TRAKHIP_OK;
     if (K == 0 || ldc < N) return TRAKHIP_ERR_SHAPE;
     if (!A_planes || !B_planes || !C) return TRAKHIP_ERR_NULL;
@@ -263,7 +285,18 @@ int gemm_nt_split(const void* A_planes, uint64_t M, const void* B_planes, uint64
     hipLaunchKernelGGL((gemm_split_kernel<kWavesM, kWavesN>), dim3((uint32_t)(tiles_m * tiles_n)),
                        dim3(64 * kWavesM * kWavesN), 0, s,
                        static_cast<const piece*>(A_planes), padded_rows(M), static_cast<const piece*>(B_planes),
-                       padded_rows(N), octets(K), C, ldc, M, N, alpha, beta, row_scale, (uint32_t)tiles_n);
+                       padded_rows(N), octets(K), C, ldc, M, N, alpha, beta, row_scale, (uint32_t)tiles_n, flags);
+    return hipGetLastError() == hipSuccess ? TRAKHIP_OK : TRAKHIP_ERR_LAUNCH;
+}
+
+int gram_split(const void* A_planes, uint64_t N, uint64_t K, float* C, uint64_t ldc, float alpha, float beta,
+               hipStream_t s) {
+    if (N == 0) return TRAKHIP_OK;
+    const int e = gemm_nt_split(A_planes, N, A_planes, N, K, C, ldc, alpha, beta, nullptr, s, kGemmLowerTilesOnly);
+    if (e) return e;
+    const uint64_t blocks = (N + 31) / 32;
+    if (blocks > 65535) return TRAKHIP_ERR_SHAPE;
+    hipLaunchKernelGGL(mirror_lower_kernel, dim3((uint32_t)blocks, (uint32_t)blocks), dim3(256), 0, s, C, ldc, N);
     return hipGetLastError() == hipSuccess ? TRAKHIP_OK : TRAKHIP_ERR_LAUNCH;
 }
 

@@ -11,7 +11,7 @@ from abc import ABC, abstractmethod
 import torch
 from torch import Tensor
 
-from .utils import gemm_nt, gemm_nt_split, gemm_tn, scores_finalize, spd_inverse, split_rows
+from .utils import gemm_nt, gemm_nt_split, gemm_tn, gram_split, scores_finalize, spd_inverse, split_rows
 
 ch = torch
 
@@ -84,8 +84,8 @@ class BasicScoreComputer(AbstractScoreComputer):
         for block in self._blocks(grads):
             block = block.to(self._dev)
             if self.gemm == "split":
-                bt = split_rows(block, transposed=True)  # the operand is block^T, read in place
-                gemm_nt_split(bt, bt, out=result, alpha=1.0, beta=1.0)
+                # the operand is block^T, read in place; lower-triangle tiles + mirror image
+                gram_split(split_rows(block, transposed=True), out=result, alpha=1.0, beta=1.0)
             else:
                 gemm_tn(block, block, out=result, alpha=1.0, beta=1.0)
         return result.to(self.dtype)

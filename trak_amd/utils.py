@@ -214,6 +214,29 @@ def gemm_nt_split(a, b, out=None, alpha=1.0, beta=0.0, row_scale=None):
     return out
 
 
+def gram_split(a, out=None, alpha=1.0, beta=0.0):
+    """out[N, N] = alpha * A @ A.T + beta * out for a SplitOperand A [N, K]: the lower-triangle tiles
+    are computed and mirrored, so the result is exactly symmetric at about half the cost of
+    `gemm_nt_split(a, a)`.  An `out` that is accumulated into must come from this function."""
+    if not isinstance(a, SplitOperand):
+        raise TypeError("gram_split takes a SplitOperand (see split_rows)")
+    N = a.rows
+    if out is None:
+        out = torch.empty((N, N), dtype=torch.float32, device=a.device)
+        beta = 0.0
+    if out.dtype != torch.float32 or tuple(out.shape) != (N, N) or (N > 1 and out.stride(1) != 1) or out.device != a.device:
+        raise RuntimeError("out must be an fp32 [N, N] tensor with unit column stride on the operand's device")
+    lib = _lib.load()
+    with torch.cuda.device(a.device):
+        stream = torch.cuda.current_stream(a.device).cuda_stream
+        code = lib.trakhip_gram_split(
+            ctypes.c_void_p(a.planes.data_ptr()), N, a.K, ctypes.c_void_p(out.data_ptr()), _ld(out),
+            float(alpha), float(beta), ctypes.c_void_p(stream),
+        )
+    _lib.check(code)
+    return out
+
+
 def spd_inverse(a, lambda_reg=0.0, normalize=False):
     """(a + lambda*I)^-1 for a symmetric positive definite fp32 matrix on the GPU; with
     normalize=True the result is divided by mean(|inverse|) (trak/score_computers.py:160-166).
