@@ -114,9 +114,6 @@ __device__ __forceinline__ void gemm_tile(const float* __restrict__ A, uint64_t 
     const uint64_t m0 = (uint64_t)tile_m * BM, n0 = (uint64_t)tile_n * BN;
     // tiles strictly above the diagonal are not needed by a caller that reads the lower triangle
     if ((flags & trakhip::kGemmLowerTilesOnly) && n0 > m0 + BM - 1) return;
-    // both operands vanish for k < their row/column index (lower-triangular factors stored k-row):
-    // the sum starts at the larger of the tile origins
-    const uint64_t k_first = (flags & trakhip::kGemmKFromDiagonal) ? ((m0 > n0 ? m0 : n0) / BKT) : 0;
 
     const int tid = threadIdx.x;
     const int wave = tid >> 6, lane = tid & 63;
@@ -133,16 +130,14 @@ __device__ __forceinline__ void gemm_tile(const float* __restrict__ A, uint64_t 
 
     const uint64_t nk = (K + BKT - 1) / BKT;
     float4 ra[Tile<BM>::pieces], rb[Tile<BN>::pieces];
-    if (k_first < nk) {
-        load_tile<AK, ALIGNED, BM>(A, lda, m0, M, k_first * BKT, K, tid, ra);
-        load_tile<BK, ALIGNED, BN>(B, ldb, n0, N, k_first * BKT, K, tid, rb);
-        store_tile<AK, BM>(lds[0], tid, ra);
-        store_tile<BK, BN>(lds[0] + Tile<BM>::floats, tid, rb);
-    }
+    load_tile<AK, ALIGNED, BM>(A, lda, m0, M, 0, K, tid, ra);
+    load_tile<BK, ALIGNED, BN>(B, ldb, n0, N, 0, K, tid, rb);
+    store_tile<AK, BM>(lds[0], tid, ra);
+    store_tile<BK, BN>(lds[0] + Tile<BM>::floats, tid, rb);
     __syncthreads();
 
-    for (uint64_t kt = k_first; kt < nk; ++kt) {
-        const int cur = (int)((kt - k_first) & 1);
+    for (uint64_t kt = 0; kt < nk; ++kt) {
+        const int cur = (int)(kt & 1);
         if (kt + 1 < nk) {
             load_tile<AK, ALIGNED, BM>(A, lda, m0, M, (kt + 1) * BKT, K, tid, ra);
             load_tile<BK, ALIGNED, BN>(B, ldb, n0, N, (kt + 1) * BKT, K, tid, rb);

@@ -275,10 +275,17 @@ int tri_inverse(Ctx& c, uint64_t nblk) {
 
 namespace trakhip {
 
+// Workspace: three np x np matrices (W, L, Li), the reduction scratch, and for small n a tail for the
+// split planes of Li^T (for np >= 384 they fit into W and L, which are free by then).
+static size_t planes_tail_bytes(uint64_t n, uint64_t np) {
+    const size_t planes = split_bytes(n, n), free_front = (size_t)(2 * np * np) * sizeof(float);
+    return planes > free_front ? planes : 0;
+}
+
 size_t spd_inverse_workspace_bytes(uint64_t n) {
     if (n == 0) return 0;
     const uint64_t np = (n + NB - 1) / NB * NB;
-    return (size_t)(3 * np * np + kSumBlocks + 4) * sizeof(float);
+    return (size_t)(3 * np * np + kSumBlocks + 4) * sizeof(float) + planes_tail_bytes(n, np);
 }
 
 int spd_inverse(const float* A, uint64_t lda, float lambda, float* inv, uint64_t ldi, uint64_t n, int normalize,
@@ -322,9 +329,12 @@ int spd_inverse(const float* A, uint64_t lda, float lambda, float* inv, uint64_t
     int e = tri_inverse(c, nblk);
     if (e) return e;
 
-    // inverse = Li^T * Li (rows of Li at or beyond n do not reach the leading n x n block)
-    // Li is lower triangular: Li[k][m] = 0 for k < m, so the sum over k starts at max(m, n)
-    e = gemm_tn(Li, np, Li, np, inv, ldi, n, n, n, 1.0f, 0.0f, s, kGemmKFromDiagonal);
+    // inverse = Li^T * Li (rows of Li at or beyond n do not reach the leading n x n block): the
+    // symmetric product of the split operand Li^T, lower-triangle tiles mirrored, so the result is
+    // exactly symmetric.  The planes go where W and L were (or behind the scratch for small n).
+    void* planes = planes_tail_bytes(n, np) ? static_cast<void*>(mean_dev + 4) : static_cast<void*>(W);
+    e = split_rows(Li, np, n, n, 1, planes, split_bytes(n, n), s);
+    if (!e) e = gram_split(planes, n, n, inv, ldi, 1.0f, 0.0f, s);
     if (e) return e;
 
     if (normalize || mean_abs) {

@@ -30,9 +30,8 @@ int materialize_device(uint32_t seed, uint32_t num_feature_tiles, uint64_t P, ui
 int materialize_host(uint32_t seed, uint32_t num_feature_tiles, uint64_t P, uint64_t f0, uint64_t nf,
                      uint32_t c0, uint32_t nc, int proj_type, float* out);
 
-// internal GEMM options (spd.hip)
+// internal GEMM option (symmetric results: spd.hip, gemm_split.hip)
 constexpr uint32_t kGemmLowerTilesOnly = 1u;  // skip output tiles strictly above the diagonal
-constexpr uint32_t kGemmKFromDiagonal = 2u;   // start the k sum at max(tile row origin, tile column origin)
 
 // up to kGemmBatchMax products of one shape in one launch: element offsets of each product's operands
 constexpr uint32_t kGemmBatchMax = 32;
