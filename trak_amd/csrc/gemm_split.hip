@@ -129,7 +129,7 @@ __device__ __forceinline__ void dma_step(const piece* __restrict__ A, uint64_t R
     }
 }
 
-// NW = waves side by side along N (2 or 4); two wave rows along M.  A wave owns 64 x (256 / NW) of C.
+// MW wave rows along M, NW waves side by side along N: the tile is 64 MW x 256, a wave owns 64 x (256 / NW).
 template <int MW, int NW>
 __global__ __launch_bounds__(64 * MW * NW, 2) void gemm_split_kernel(
     const piece* __restrict__ A, uint64_t Rpa, const piece* __restrict__ B, uint64_t Rpb, uint64_t K8,
