@@ -362,6 +362,13 @@ def bench_scoring(torch, dev, reps=3):
     _, s_feat = timed(lambda: gemm_nt_split(split_rows(X), split_rows(inv)))
     _, s_sc = timed(lambda: gemm_nt_split(split_rows(feats), split_rows(Xt), row_scale=otl))
     split_ms = s_xtx + s_feat + s_sc
+    # TRAKer's default stores gradients and features as fp16 (use_half_precision): the same products
+    # from single fp16 planes, one MFMA per k step, exact products
+    Xh, invh, fh, Xth = X.half(), inv.half(), feats.half(), Xt.half()
+    _, h_xtx = timed(lambda: gram_split(split_rows(Xh, transposed=True)))
+    _, h_feat = timed(lambda: gemm_nt_split(split_rows(Xh), split_rows(invh)))
+    _, h_sc = timed(lambda: gemm_nt_split(split_rows(fh), split_rows(Xth), row_scale=otl))
+    del Xh, fh, Xth
     # X^T X is computed on the tiles that touch the lower triangle only (256 x 256 tiles) and mirrored:
     # its flops are counted as computed, not as 2*N*k*k
     t256 = (k + 255) // 256
@@ -378,6 +385,11 @@ def bench_scoring(torch, dev, reps=3):
             "bf16_mfma_tflops_executed": 6 * split_flop / (split_ms * 1e-3) / 1e12,
             "frac_bf16_mfma_peak": 6 * split_flop / (split_ms * 1e-3) / 1e12 / PEAK_FP16_TFLOPS,
             "xtx_note": "symmetric product: lower-triangle tiles computed and mirrored, flops counted as computed",
+        },
+        "fp16_inputs": {
+            "xtx_ms": h_xtx, "x_xtx_inv_ms": h_feat, "scores_ms": h_sc,
+            "gemm_tflops": split_flop / ((h_xtx + h_feat + h_sc) * 1e-3) / 1e12,
+            "frac_fp16_mfma_peak": split_flop / ((h_xtx + h_feat + h_sc) * 1e-3) / 1e12 / PEAK_FP16_TFLOPS,
         },
         "inverse_flop": float(k) ** 3,
         "scores_orientation": "[N_train, M_targets]",

@@ -136,33 +136,34 @@ int trakhip_gemm_tn(const float* A_dev, uint64_t lda, const float* B_dev, uint64
                     uint64_t ldc, uint64_t M, uint64_t N, uint64_t K, float alpha, float beta,
                     void* stream);
 
-/* The same products on the bf16 matrix cores (sixteen times the fp32 MFMA rate) without giving up
- * fp32 accuracy: an operand is first split into three bf16 "planes" whose sum is the fp32 value
- * exactly (trakhip_split_rows, one pass over the operand), and trakhip_gemm_nt_split multiplies
- * planes with six bf16 MFMAs per k step, accumulating in fp32; the terms left out are below
- * 2^-24 of each product, the rounding of one fp32 multiplication.
- *   trakhip_split_bytes(rows, K)   bytes of the planes of a [rows, K] operand
+/* The same products on the 16-bit matrix cores (sixteen times the fp32 MFMA rate) without giving
+ * up fp32 accuracy.  An operand is first brought into "planes" (trakhip_split_rows, one pass):
+ * an fp32 matrix becomes three bf16 planes whose sum is the fp32 value exactly, and the product
+ * uses six bf16 MFMAs per k step with fp32 accumulation (the terms left out are below 2^-24 of each
+ * product, the rounding of one fp32 multiplication); an fp16 or bf16 matrix (what TRAKer stores
+ * with use_half_precision) is one plane and one MFMA, with exact products.
+ *   src_dtype                      TRAKHIP_F32 | TRAKHIP_F16 | TRAKHIP_BF16; both operands of a
+ *                                  product must come from the same type
+ *   trakhip_split_bytes            bytes of the planes of a [rows, K] operand
  *   trakhip_split_rows             src_dev is [rows, K] with row pitch ld (transposed == 0), or
  *                                  [K, rows] with row pitch ld (transposed != 0: the operand is
  *                                  the transpose of what is stored, as X^T in X^T X)
  *   trakhip_gemm_nt_split          C[M, N] = alpha * A * B^T + beta * C, row i *= row_scale[i];
  *                                  A_planes from a [M, K] operand, B_planes from a [N, K] one
- * Stand in, like trakhip_gemm_nt / trakhip_gemm_tn, for trak/score_computers.py:153, :176 and
- * trak/utils.py:131. */
-size_t trakhip_split_bytes(uint64_t rows, uint64_t K);
-int trakhip_split_rows(const float* src_dev, uint64_t ld, uint64_t rows, uint64_t K, int transposed,
+ *   trakhip_gram_split             C[N, N] = alpha * A * A^T + beta * C: only the tiles that touch
+ *                                  the lower triangle are computed, then the strict upper triangle
+ *                                  is overwritten with the mirror image, so C is exactly
+ *                                  symmetric; with beta != 0, C must have been produced this way
+ * Stand in, like trakhip_gemm_nt / trakhip_gemm_tn, for trak/score_computers.py:153 (the Gram
+ * product, A = the planes of block^T), :176 and trak/utils.py:131. */
+size_t trakhip_split_bytes(uint64_t rows, uint64_t K, int src_dtype);
+int trakhip_split_rows(const void* src_dev, int src_dtype, uint64_t ld, uint64_t rows, uint64_t K, int transposed,
                        void* planes_dev, size_t planes_bytes, void* stream);
 int trakhip_gemm_nt_split(const void* A_planes_dev, uint64_t M, const void* B_planes_dev, uint64_t N, uint64_t K,
-                          float* C_dev, uint64_t ldc, float alpha, float beta, const float* row_scale_dev,
-                          void* stream);
-
-/* C[N, N] = alpha * A * A^T + beta * C for one split operand A [N, K]: only the tiles that touch
- * the lower triangle are computed (half the work of trakhip_gemm_nt_split), then the strict upper
- * triangle is overwritten with the mirror image of the lower one, so C is exactly symmetric.  With
- * beta != 0, C must have been produced the same way.  Stands in for the `block.T @ block`
- * accumulation of trak/score_computers.py:145-155 (A = the split of block^T). */
-int trakhip_gram_split(const void* A_planes_dev, uint64_t N, uint64_t K, float* C_dev, uint64_t ldc, float alpha,
-                       float beta, void* stream);
+                          int src_dtype, float* C_dev, uint64_t ldc, float alpha, float beta,
+                          const float* row_scale_dev, void* stream);
+int trakhip_gram_split(const void* A_planes_dev, uint64_t N, uint64_t K, int src_dtype, float* C_dev, uint64_t ldc,
+                       float alpha, float beta, void* stream);
 
 /* out[i, j] = cast((acc[i, j] / divisor) * row_factor[i]) for the [N, M] fp32 score sums that
  * trakhip_gemm_nt accumulated over checkpoints (beta = 1): the closing expression of

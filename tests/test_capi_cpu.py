@@ -133,22 +133,30 @@ def test_store_entry_points_validate_before_touching_the_device():
 def test_split_gemm_entry_points_validate_before_touching_the_device():
     lib = _lib.load()
     p = ctypes.c_void_p(4096)
-    # three planes, octets padded to an even count, rows padded to 256, 16 bytes per (row, octet)
-    assert lib.trakhip_split_bytes(1, 1) == 3 * 2 * 256 * 16
-    assert lib.trakhip_split_bytes(50_000, 4096) == 3 * 512 * 50_176 * 16
-    assert lib.trakhip_split_bytes(257, 17) == 3 * 4 * 512 * 16
-    assert lib.trakhip_split_bytes(0, 5) == 0
+    F16, BF16, F32 = _lib.F16, _lib.BF16, _lib.F32
+    # planes (3 for fp32, 1 for 16-bit types) x octets padded to 8 x rows padded to 256 x 16 bytes
+    assert lib.trakhip_split_bytes(1, 1, F32) == 3 * 8 * 256 * 16
+    assert lib.trakhip_split_bytes(50_000, 4096, F32) == 3 * 512 * 50_176 * 16
+    assert lib.trakhip_split_bytes(50_000, 4096, F16) == 512 * 50_176 * 16
+    assert lib.trakhip_split_bytes(257, 65, BF16) == 16 * 512 * 16
+    assert lib.trakhip_split_bytes(0, 5, F32) == 0 and lib.trakhip_split_bytes(5, 5, 7) == 0
     sp = lambda **kw: lib.trakhip_split_rows(
-        kw.get("src", p), kw.get("ld", 64), kw.get("rows", 10), kw.get("K", 64), kw.get("tr", 0),
+        kw.get("src", p), kw.get("dt", F32), kw.get("ld", 64), kw.get("rows", 10), kw.get("K", 64), kw.get("tr", 0),
         kw.get("out", p), kw.get("bytes", 1 << 30), None)
+    assert sp(dt=9) == -3
     assert sp(rows=0) == -2 and sp(K=0) == -2 and sp(ld=63) == -2 and sp(tr=1, ld=9) == -2
     assert sp(src=None) == -5 and sp(out=None) == -5
     assert sp(bytes=100) == -6
     assert sp(src=ctypes.c_void_p(4098)) == -7 and sp(out=ctypes.c_void_p(4104)) == -7
+    assert sp(dt=F16, src=ctypes.c_void_p(4097)) == -7
     mm = lambda **kw: lib.trakhip_gemm_nt_split(
-        kw.get("a", p), kw.get("M", 8), kw.get("b", p), kw.get("N", 8), kw.get("K", 16), kw.get("c", p),
-        kw.get("ldc", 8), 1.0, 0.0, None, None)
+        kw.get("a", p), kw.get("M", 8), kw.get("b", p), kw.get("N", 8), kw.get("K", 16), kw.get("dt", F32),
+        kw.get("c", p), kw.get("ldc", 8), 1.0, 0.0, None, None)
+    assert mm(dt=-1) == -3
     assert mm(M=0) == 0 and mm(N=0) == 0
     assert mm(K=0) == -2 and mm(ldc=7) == -2
     assert mm(a=None) == -5 and mm(b=None) == -5 and mm(c=None) == -5
     assert mm(a=ctypes.c_void_p(4104)) == -7 and mm(c=ctypes.c_void_p(4098)) == -7
+    gr = lambda **kw: lib.trakhip_gram_split(kw.get("a", p), kw.get("N", 8), kw.get("K", 16), kw.get("dt", F32),
+                                             kw.get("c", p), kw.get("ldc", 8), 1.0, 0.0, None)
+    assert gr(N=0) == 0 and gr(dt=5) == -3 and gr(ldc=7) == -2 and gr(a=None) == -5

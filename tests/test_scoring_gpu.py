@@ -107,10 +107,16 @@ def test_spd_inverse_closed_forms_and_failure(gpu):
 
 
 def split_planes_to_numpy(op):
-    """[3, padded rows, padded K] float32 view of a SplitOperand (layout: plane, k-octet, row, 8 bf16)."""
-    Rp, K8 = (op.rows + 255) // 256 * 256, (op.K + 15) // 16 * 2
-    raw = op.planes.cpu().numpy()[: 3 * K8 * Rp * 16].view(np.uint16).reshape(3, K8, Rp, 8)
-    return (raw.astype(np.uint32) << 16).view(np.float32).transpose(0, 2, 1, 3).reshape(3, Rp, K8 * 8)
+    """[planes, padded rows, padded K] float32 view of a SplitOperand (layout: plane, k-octet, row,
+    8 values of 16 bits: bf16 for an fp32 or bf16 source, fp16 for an fp16 source)."""
+    planes = 3 if op.dtype == torch.float32 else 1
+    Rp, K8 = (op.rows + 255) // 256 * 256, (op.K + 63) // 64 * 8
+    raw = op.planes.cpu().numpy()[: planes * K8 * Rp * 16].view(np.uint16).reshape(planes, K8, Rp, 8)
+    if op.dtype == torch.float16:
+        vals = raw.view(np.float16).astype(np.float32)
+    else:
+        vals = (raw.astype(np.uint32) << 16).view(np.float32)
+    return vals.transpose(0, 2, 1, 3).reshape(planes, Rp, K8 * 8)
 
 
 @pytest.mark.parametrize("rows,K,transposed", [(5, 9, False), (300, 70, False), (70, 300, True), (257, 33, True), (256, 16, False)])
@@ -131,6 +137,45 @@ def test_split_is_exact_and_zero_padded(gpu, rows, K, transposed):
         nz = want != 0
         assert (np.abs(planes[1][:rows, :K][nz]) <= 2.0 ** -8 * np.abs(planes[0][:rows, :K][nz])).all()
         assert (np.abs(planes[2][:rows, :K][nz]) <= 2.0 ** -16 * np.abs(planes[0][:rows, :K][nz])).all()
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("rows,K,transposed", [(5, 9, False), (300, 70, False), (70, 300, True), (257, 33, True), (256, 64, False)])
+def test_sixteen_bit_operands_are_one_exact_plane(gpu, dtype, rows, K, transposed):
+    gen = torch.Generator(device="cpu").manual_seed(rows + K)
+    t = (torch.randn((K, rows) if transposed else (rows, K), generator=gen) * 3).to(dtype)
+    wide = torch.zeros(t.shape[0], t.shape[1] + 3, dtype=dtype)
+    wide[:, 1 : 1 + t.shape[1]] = t
+    for src in (t.to(gpu), wide.to(gpu)[:, 1 : 1 + t.shape[1]]):
+        op = split_rows(src, transposed=transposed)
+        assert op.dtype == dtype
+        planes = split_planes_to_numpy(op)
+        want = (t.T if transposed else t).float().numpy()
+        assert planes.shape[0] == 1 and np.array_equal(planes[0][:rows, :K], want)
+        assert not planes[0][rows:].any() and not planes[0][:, K:].any()
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("M,N,K", [(1, 1, 1), (130, 70, 33), (256, 512, 64), (1000, 513, 257), (300, 700, 4100)])
+def test_gemm_nt_split_sixteen_bit(gpu, dtype, M, N, K):
+    # products of 16-bit values are exact in fp32: the only error is the fp32 accumulation
+    gen = torch.Generator(device="cpu").manual_seed(M + N * 3 + K)
+    a, b = torch.randn(M, K, generator=gen).to(dtype), torch.randn(N, K, generator=gen).to(dtype)
+    want = a.double().numpy() @ b.double().numpy().T
+    sa, sb = split_rows(a.to(gpu)), split_rows(b.to(gpu))
+    got = gemm_nt_split(sa, sb)
+    assert rel_max(got.cpu().numpy(), want) < gemm_tol(K)
+    # the same numbers through the three-plane fp32 path (the extra planes are zero)
+    ref = gemm_nt_split(split_rows(a.float().to(gpu)), split_rows(b.float().to(gpu)))
+    assert rel_max(got.cpu().numpy(), ref.cpu().numpy()) < gemm_tol(K)
+    rs = torch.rand(M, generator=gen)
+    c0 = torch.randn(M, N, generator=gen)
+    got = gemm_nt_split(sa, sb, out=c0.clone().to(gpu), alpha=2.0, beta=0.5, row_scale=rs.to(gpu))
+    assert rel_max(got.cpu().numpy(), (2.0 * want + 0.5 * c0.double().numpy()) * rs.double().numpy()[:, None]) < gemm_tol(K)
+    g = gram_split(split_rows(a.T.contiguous().to(gpu), transposed=True))
+    assert torch.equal(g, g.T) and rel_max(g.cpu().numpy(), a.double().numpy() @ a.double().numpy().T) < gemm_tol(K)
+    with pytest.raises(RuntimeError):
+        gemm_nt_split(sa, split_rows(b.float().to(gpu)))        # operands of different source types
 
 
 @pytest.mark.parametrize("M,N,K", [(1, 1, 1), (130, 70, 33), (256, 512, 64), (1000, 513, 257), (64, 2048, 4096), (129, 257, 8200)])
@@ -269,3 +314,27 @@ def test_full_size_scoring_shape(gpu, gemm):
     assert rel_max(acc[:, tcols].cpu().numpy(), col64.cpu().numpy()) < 1e-4
     fused = sc.get_scaled_scores(feats, Xt, otl)
     assert rel_max(fused[rows].cpu().numpy(), (scores64 * otl[rows].double()[:, None]).cpu().numpy()) < 1e-4
+
+
+def test_score_computer_half_precision_flow(gpu):
+    """TRAKer's default (use_half_precision): fp16 gradients and an fp16 score computer.  Every
+    product runs from single fp16 planes (exact products); results are fp16 tensors as in the
+    reference, compared with float64 computed from the same fp16 inputs at fp16 resolution."""
+    N, k, M, lam = 900, 512, 70, 1e-2
+    gen = torch.Generator(device="cpu").manual_seed(99)
+    X = (torch.randn(N, k, generator=gen) / math.sqrt(k)).half()
+    Xt = (torch.randn(M, k, generator=gen) / math.sqrt(k)).half()
+    sc = BasicScoreComputer(dtype=torch.float16, device="cuda:0", lambda_reg=lam)
+    xtx = sc.get_xtx(X.to(gpu))
+    assert xtx.dtype == torch.float16
+    x64 = X.double().numpy()
+    assert rel_max(xtx.float().cpu().numpy(), x64.T @ x64) < 1e-3            # one fp16 rounding of the result
+    feats = sc.get_x_xtx_inv(X.to(gpu), xtx)
+    assert feats.dtype == torch.float16 and feats.shape == (N, k)
+    inv64 = np.linalg.inv(xtx.double().cpu().numpy() + lam * np.eye(k))
+    inv16 = torch.from_numpy(inv64 / np.abs(inv64).mean()).half().double().numpy()   # the reference casts the inverse
+    assert rel_max(feats.float().cpu().numpy(), x64 @ inv16) < 3e-3
+    acc = torch.zeros(N, M, device=gpu)
+    sc.get_scores(feats, Xt.to(gpu), accumulator=acc)
+    want = feats.double().cpu().numpy() @ Xt.double().numpy().T
+    assert rel_max(acc.cpu().numpy(), want) < gemm_tol(k)                    # exact products, fp32 sums

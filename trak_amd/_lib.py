@@ -58,13 +58,13 @@ def load():
     lib.trakhip_gemm_nt.restype = i32
     lib.trakhip_gemm_tn.argtypes = [vp, u64, vp, u64, vp, u64, u64, u64, u64, f32, f32, vp]
     lib.trakhip_gemm_tn.restype = i32
-    lib.trakhip_split_bytes.argtypes = [u64, u64]
+    lib.trakhip_split_bytes.argtypes = [u64, u64, i32]
     lib.trakhip_split_bytes.restype = sz
-    lib.trakhip_split_rows.argtypes = [vp, u64, u64, u64, i32, vp, sz, vp]
+    lib.trakhip_split_rows.argtypes = [vp, i32, u64, u64, u64, i32, vp, sz, vp]
     lib.trakhip_split_rows.restype = i32
-    lib.trakhip_gemm_nt_split.argtypes = [vp, u64, vp, u64, u64, vp, u64, f32, f32, vp, vp]
+    lib.trakhip_gemm_nt_split.argtypes = [vp, u64, vp, u64, u64, i32, vp, u64, f32, f32, vp, vp]
     lib.trakhip_gemm_nt_split.restype = i32
-    lib.trakhip_gram_split.argtypes = [vp, u64, u64, vp, u64, f32, f32, vp]
+    lib.trakhip_gram_split.argtypes = [vp, u64, u64, i32, vp, u64, f32, f32, vp]
     lib.trakhip_gram_split.restype = i32
     lib.trakhip_spd_inverse_workspace.argtypes = [u64]
     lib.trakhip_spd_inverse_workspace.restype = sz

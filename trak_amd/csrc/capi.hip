@@ -92,24 +92,24 @@ int trakhip_gemm_tn(const float* A_dev, uint64_t lda, const float* B_dev, uint64
                             static_cast<hipStream_t>(stream));
 }
 
-size_t trakhip_split_bytes(uint64_t rows, uint64_t K) { return trakhip::split_bytes(rows, K); }
+size_t trakhip_split_bytes(uint64_t rows, uint64_t K, int dtype) { return trakhip::split_bytes(rows, K, dtype); }
 
-int trakhip_split_rows(const float* src_dev, uint64_t ld, uint64_t rows, uint64_t K, int transposed,
+int trakhip_split_rows(const void* src_dev, int dtype, uint64_t ld, uint64_t rows, uint64_t K, int transposed,
                        void* planes_dev, size_t planes_bytes, void* stream) {
-    return trakhip::split_rows(src_dev, ld, rows, K, transposed, planes_dev, planes_bytes,
+    return trakhip::split_rows(src_dev, dtype, ld, rows, K, transposed, planes_dev, planes_bytes,
                                static_cast<hipStream_t>(stream));
 }
 
 int trakhip_gemm_nt_split(const void* A_planes_dev, uint64_t M, const void* B_planes_dev, uint64_t N, uint64_t K,
-                          float* C_dev, uint64_t ldc, float alpha, float beta, const float* row_scale_dev,
-                          void* stream) {
-    return trakhip::gemm_nt_split(A_planes_dev, M, B_planes_dev, N, K, C_dev, ldc, alpha, beta, row_scale_dev,
+                          int dtype, float* C_dev, uint64_t ldc, float alpha, float beta,
+                          const float* row_scale_dev, void* stream) {
+    return trakhip::gemm_nt_split(A_planes_dev, M, B_planes_dev, N, K, dtype, C_dev, ldc, alpha, beta, row_scale_dev,
                                   static_cast<hipStream_t>(stream));
 }
 
-int trakhip_gram_split(const void* A_planes_dev, uint64_t N, uint64_t K, float* C_dev, uint64_t ldc, float alpha,
-                       float beta, void* stream) {
-    return trakhip::gram_split(A_planes_dev, N, K, C_dev, ldc, alpha, beta, static_cast<hipStream_t>(stream));
+int trakhip_gram_split(const void* A_planes_dev, uint64_t N, uint64_t K, int dtype, float* C_dev, uint64_t ldc,
+                       float alpha, float beta, void* stream) {
+    return trakhip::gram_split(A_planes_dev, N, K, dtype, C_dev, ldc, alpha, beta, static_cast<hipStream_t>(stream));
 }
 
 size_t trakhip_spd_inverse_workspace(uint64_t n) { return trakhip::spd_inverse_workspace_bytes(n); }

@@ -1,25 +1,31 @@
-// fp32 GEMM on the bf16 matrix cores: C[M, N] = alpha * A * B^T + beta * C (row i *= row_scale[i]).
+// fp32-accurate GEMM on the 16-bit matrix cores: C[M, N] = alpha * A * B^T + beta * C (row i *= row_scale[i]).
 //
 // The scoring GEMMs of BasicScoreComputer (trak/score_computers.py:153, :176, trak/utils.py:131)
-// are fp32 x fp32.  v_mfma_f32_32x32x2_f32 runs at 157 TFLOP/s; v_mfma_f32_32x32x16_bf16 at 2.5
-// PFLOP/s, sixteen times the rate.  Every fp32 value is the exact sum of three bf16 values
-// (24 significand bits = 3 x 8), x = x1 + x2 + x3 with |x2| <= 2^-8 |x1|, |x3| <= 2^-16 |x1|, so
+// multiply fp32 matrices (or fp16 ones when TRAKer runs with use_half_precision, its default).
+// v_mfma_f32_32x32x2_f32 runs at 157 TFLOP/s; v_mfma_f32_32x32x16_{bf16,f16} at 2.5 PFLOP/s,
+// sixteen times the rate, with exact products and fp32 accumulation.
+//
+// fp32 operands: every fp32 value is the exact sum of three bf16 values (24 significand bits =
+// 3 x 8), x = x1 + x2 + x3 with |x2| <= 2^-8 |x1|, |x3| <= 2^-16 |x1|, so
 //     a * b = a1 b1 + (a1 b2 + a2 b1) + (a1 b3 + a2 b2 + a3 b1) + O(2^-24 |a b|)
-// and six bf16 MFMAs (products exact, fp32 accumulation) give the product sum with the error of an
-// fp32 dot product at 6/16 of the cost of the fp32 instruction.  The three terms left out are each
-// below 2^-24 |a b|, the rounding a single fp32 multiplication makes.
+// and six bf16 MFMAs give the product sum with the error of an fp32 dot product at 6/16 of the
+// cost of the fp32 instruction.  The three terms left out are each below 2^-24 |a b|, the rounding
+// a single fp32 multiplication makes.
+// fp16 or bf16 operands (both of the same type): one plane, one MFMA, nothing left out.
 //
-// Operands are split once, outside the GEMM, into "planes": plane p, k-octet o (8 consecutive k),
+// Operands are brought once, outside the GEMM, into "planes": plane p, k-octet o (8 consecutive k),
 // row r is one 16-byte piece at ((p * K8 + o) * Rp + r) * 16 bytes, rows padded with zeros to a
-// multiple of 256 and octets to an even count.  A 16-byte piece is exactly what one lane feeds to
+// multiple of 256 and octets to a multiple of 8.  A 16-byte piece is exactly what one lane feeds to
 // the MFMA (8 consecutive k of one row), consecutive rows are consecutive pieces, so global loads,
-// LDS writes and LDS reads are all linear and conflict free, and the GEMM kernel moves bf16 only.
+// LDS writes and LDS reads are all linear and conflict free, and the GEMM kernel moves 16-bit data
+// only.
 //
-// Workgroup = 512 threads = 8 waves (4 x 2), 256 x 256 tile of C, k step 16 (one MFMA deep), two
-// LDS buffers of 48 KB filled by LDS-direct loads, one barrier per step; a wave owns 64 x 128 of C
-// (128 accumulator VGPRs) and issues 48 MFMAs per step.  Measured against this: 128 x 256 tiles with
-// two workgroups per CU (9 % slower), 64 x 64 wave tiles at four waves per SIMD, three LDS buffers,
-// register-staged loads, super-tile orders per XCD (all slower or equal).
+// Workgroup = 512 threads = 8 waves (4 x 2), 256 x 256 tile of C, a wave owns 64 x 128 of C (128
+// accumulator VGPRs).  A step covers 16 S values of k (S = 1 for three planes, 4 for one plane):
+// two LDS buffers of 48 or 64 KB filled by LDS-direct loads, one barrier per step, 48 or 32 MFMAs
+// per wave and step.  Measured against this for three planes: 128 x 256 tiles with two workgroups
+// per CU (9 % slower), 64 x 64 wave tiles at four waves per SIMD, three LDS buffers, register-staged
+// loads, super-tile orders per XCD (all slower or equal).
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
@@ -29,15 +35,16 @@ namespace {
 
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
-typedef uint32_t piece __attribute__((ext_vector_type(4)));  // 16 bytes = 8 bf16 = one lane's MFMA operand
+typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+typedef uint32_t piece __attribute__((ext_vector_type(4)));  // 16 bytes = 8 x 16 bit = one lane's MFMA operand
 
-constexpr int kWavesN = 2;                         // waves side by side: each owns 64 x 128 of C
-constexpr int BN = 256;
-constexpr int kRowPad = 256;                       // rows of a split operand are padded to this
-constexpr int kBPieces = 3 * 2 * BN;               // 16-byte pieces of a B tile: [plane][half][row]
-constexpr int kWavesM = 4;                         // wave rows: the C tile has 64 * kWavesM = 256 rows
+constexpr int kWavesM = 4, kWavesN = 2;            // 4 x 2 waves, each owns 64 x 128 of C
+constexpr int BM = 64 * kWavesM, BN = 128 * kWavesN;
+constexpr int kWaves = kWavesM * kWavesN;
+constexpr int kRowPad = 256;                       // rows of an operand are padded to this
+constexpr int kOctetPad = 8;                       // octets (64 values of k) are padded to this
 
-// ---- splitting -----------------------------------------------------------------------------
+// ---- bringing operands into planes ---------------------------------------------------------
 
 // binary32 -> nearest bf16 (ties to even) as a binary32 value; finite inputs
 __device__ __forceinline__ float bf16_round(float x) {
@@ -56,7 +63,7 @@ __device__ __forceinline__ void split3(float x, uint32_t (&t)[3]) {
     t[2] = __float_as_uint(bf16_round(r2)) >> 16;
 }
 
-// One thread per (row r, octet o): reads 8 consecutive k of the row, writes its three pieces.
+// One thread per (row r, octet o): reads 8 consecutive k of the row, writes its pieces.
 // TRANS = false: src[r * ld + k];  TRANS = true: src[k * ld + r].  Rows >= rows and k >= K give
 // zeros (the padding is rewritten on every call).  Threads of a workgroup cover 64 rows x 4 octets.
 template <bool TRANS, bool ALIGNED>
@@ -93,53 +100,82 @@ __global__ __launch_bounds__(256) void split_kernel(const float* __restrict__ sr
     for (int p = 0; p < 3; ++p) planes[((uint64_t)p * K8 + o) * Rp + r] = make_uint4(w[p][0], w[p][1], w[p][2], w[p][3]);
 }
 
-// ---- GEMM ----------------------------------------------------------------------------------
-
-__device__ __forceinline__ floatx16 mfma_bf16(const piece& a, const piece& b, floatx16 c) {
-    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c,
-                                                   0, 0, 0);
+// The same for a 16-bit source (fp16 or bf16 bit patterns): one plane, the values themselves.
+template <bool TRANS, bool ALIGNED>
+__global__ __launch_bounds__(256) void relayout16_kernel(const uint16_t* __restrict__ src, uint64_t ld, uint64_t rows,
+                                                         uint64_t K, uint64_t Rp, uint64_t K8, uint32_t row_blocks,
+                                                         uint4* __restrict__ planes) {
+    const uint64_t r = (uint64_t)(blockIdx.x % row_blocks) * 64 + (threadIdx.x & 63);
+    const uint64_t o = (uint64_t)(blockIdx.x / row_blocks) * 4 + (threadIdx.x >> 6);
+    if (r >= Rp || o >= K8) return;
+    uint4 w;
+    if (!TRANS && ALIGNED && r < rows && 8 * o + 8 <= K) {
+        w = *reinterpret_cast<const uint4*>(src + r * ld + 8 * o);
+    } else {
+        uint32_t v[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const uint64_t k = 8 * o + i;
+            v[i] = (r < rows && k < K) ? (uint32_t)(TRANS ? src[k * ld + r] : src[r * ld + k]) : 0u;
+        }
+        w = make_uint4(v[0] | (v[1] << 16), v[2] | (v[3] << 16), v[4] | (v[5] << 16), v[6] | (v[7] << 16));
+    }
+    planes[o * Rp + r] = w;
 }
 
-// Step s (octets 2s, 2s + 1) of a tile is 6 * (BM + 256) pieces, [A: plane][half][BM rows] followed
-// by [B: plane][half][256 rows], moved in chunks of 64 consecutive pieces by the load unit straight
-// into LDS (global_load_lds_dwordx4): the 64 lanes of a wave fetch 64 consecutive rows of one
-// (plane, octet), which land at 64 consecutive 16-byte slots starting at a wave-uniform LDS
-// address; no staging registers, no LDS store instructions.  Wave w of W moves chunks w, w + W, ...
-template <int W, int BM>
+// ---- GEMM ----------------------------------------------------------------------------------
+
+template <bool F16>
+__device__ __forceinline__ floatx16 mfma16(const piece& a, const piece& b, floatx16 c) {
+    if constexpr (F16)
+        return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8, a), __builtin_bit_cast(half8, b), c,
+                                                      0, 0, 0);
+    else
+        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b),
+                                                       c, 0, 0, 0);
+}
+
+// A step of a tile is S sub-steps (two octets = one MFMA depth each); sub-step u holds
+// [A: plane][half][256 rows] followed by [B: plane][half][256 rows].  The pieces are moved in chunks
+// of 64 consecutive ones by the load unit straight into LDS (global_load_lds_dwordx4): the 64
+// lanes of a wave fetch 64 consecutive rows of one (plane, octet), which land at 64 consecutive
+// 16-byte slots starting at a wave-uniform LDS address; no staging registers, no LDS store
+// instructions.  Wave w moves chunks w, w + 8, ...
+template <int P, int S>
 __device__ __forceinline__ void dma_step(const piece* __restrict__ A, uint64_t Rpa, const piece* __restrict__ B,
                                          uint64_t Rpb, uint64_t K8, uint64_t m0, uint64_t n0, uint64_t s,
                                          int wave, int lane, piece* lds) {
-    constexpr int kAPieces = 3 * 2 * BM;
-    constexpr int kChunks = (kAPieces + kBPieces) / 64;
-    constexpr int kAChunks = kAPieces / 64;
+    constexpr int kAChunks = P * 2 * BM / 64, kBChunks = P * 2 * BN / 64;
+    constexpr int kSubChunks = kAChunks + kBChunks, kChunks = S * kSubChunks;
+    static_assert(kChunks % kWaves == 0, "every wave moves the same number of chunks");
 #pragma unroll
-    for (int i = 0; i < (kChunks + W - 1) / W; ++i) {
-        const int c = wave + W * i;  // wave-uniform
-        if (c >= kChunks) break;
+    for (int i = 0; i < kChunks / kWaves; ++i) {
+        const int c = wave + kWaves * i;  // wave-uniform
+        const int u = c / kSubChunks, cc = c % kSubChunks;
         const piece* src;
-        if (c < kAChunks) {
-            const int e = 64 * c + lane, row = e % BM, ph = e / BM;  // ph = plane * 2 + half
-            src = A + ((uint64_t)(ph >> 1) * K8 + 2 * s + (ph & 1)) * Rpa + m0 + row;
+        if (cc < kAChunks) {
+            const int e = 64 * cc + lane, row = e % BM, ph = e / BM;  // ph = plane * 2 + half
+            src = A + ((uint64_t)(ph >> 1) * K8 + 2 * (s * S + u) + (ph & 1)) * Rpa + m0 + row;
         } else {
-            const int e = 64 * (c - kAChunks) + lane, row = e % BN, ph = e / BN;
-            src = B + ((uint64_t)(ph >> 1) * K8 + 2 * s + (ph & 1)) * Rpb + n0 + row;
+            const int e = 64 * (cc - kAChunks) + lane, row = e % BN, ph = e / BN;
+            src = B + ((uint64_t)(ph >> 1) * K8 + 2 * (s * S + u) + (ph & 1)) * Rpb + n0 + row;
         }
         __builtin_amdgcn_global_load_lds((const void __attribute__((address_space(1)))*)src,
                                          (void __attribute__((address_space(3)))*)(lds + 64 * c), 16, 0, 0);
     }
 }
 
-// MW wave rows along M, NW waves side by side along N: the tile is 64 MW x 256, a wave owns 64 x (256 / NW).
-template <int MW, int NW>
-__global__ __launch_bounds__(64 * MW * NW, 2) void gemm_split_kernel(
+// P planes per operand (3: split fp32, 1: a 16-bit type), F16 selects the fp16 MFMA, S sub-steps
+// per barrier.
+template <int P, bool F16, int S>
+__global__ __launch_bounds__(64 * kWaves, 2) void gemm_split_kernel(
     const piece* __restrict__ A, uint64_t Rpa, const piece* __restrict__ B, uint64_t Rpb, uint64_t K8,
     float* __restrict__ C, uint64_t ldc, uint64_t M, uint64_t N, float alpha, float beta,
     const float* __restrict__ row_scale, uint32_t tiles_n, uint32_t flags) {
-    constexpr int W = MW * NW;       // waves
-    constexpr int JT = 8 / NW;       // 32-column MFMA tiles per wave
-    constexpr int BM = 64 * MW;
-    constexpr int kAPieces = 3 * 2 * BM;             // [plane][half][row]
-    constexpr int kBufPieces = kAPieces + kBPieces;  // 256 x 256 tile: 3072 pieces = 48 KB
+    constexpr int JT = BN / kWavesN / 32;            // 32-column MFMA tiles per wave
+    constexpr int kAPieces = P * 2 * BM;             // [plane][half][row]
+    constexpr int kSubPieces = P * 2 * (BM + BN);    // three planes: 3072 pieces = 48 KB
+    constexpr int kBufPieces = S * kSubPieces;
     __shared__ piece lds[2][kBufPieces];
 
     const uint32_t tile_m = blockIdx.x / tiles_n, tile_n = blockIdx.x % tiles_n;
@@ -148,7 +184,7 @@ __global__ __launch_bounds__(64 * MW * NW, 2) void gemm_split_kernel(
     if ((flags & trakhip::kGemmLowerTilesOnly) && n0 > m0 + BM - 1) return;
     const int tid = threadIdx.x;
     const int wave = tid >> 6, lane = tid & 63;
-    const int wm = wave / NW, wn = wave % NW;
+    const int wm = wave / kWavesN, wn = wave % kWavesN;
     const int x = lane & 31, h = lane >> 5;
 
     floatx16 acc[2][JT];
@@ -159,37 +195,46 @@ __global__ __launch_bounds__(64 * MW * NW, 2) void gemm_split_kernel(
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
-    const uint64_t steps = K8 / 2;
-    dma_step<W, BM>(A, Rpa, B, Rpb, K8, m0, n0, 0, wave, lane, lds[0]);
+    const uint64_t steps = K8 / (2 * S);
+    dma_step<P, S>(A, Rpa, B, Rpb, K8, m0, n0, 0, wave, lane, lds[0]);
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
 
-    // piece index of this lane's operand for plane p: A rows wm*64 + 32*i + x, B rows wn*32*JT + 32*j + x
+    // piece index of this lane's operand for plane p: A rows wm*64 + 32*i + x, B rows wn*128 + 32*j + x
     const int a_lane = h * BM + wm * 64 + x;
     const int b_lane = kAPieces + h * BN + wn * (32 * JT) + x;
 
     for (uint64_t s = 0; s < steps; ++s) {
         const int cur = (int)(s & 1);
         // the other buffer was last read before the barrier that ended the previous step
-        if (s + 1 < steps) dma_step<W, BM>(A, Rpa, B, Rpb, K8, m0, n0, s + 1, wave, lane, lds[cur ^ 1]);
-        const piece* l = lds[cur];
-        piece fa[2][3];
+        if (s + 1 < steps) dma_step<P, S>(A, Rpa, B, Rpb, K8, m0, n0, s + 1, wave, lane, lds[cur ^ 1]);
 #pragma unroll
-        for (int i = 0; i < 2; ++i)
+        for (int u = 0; u < S; ++u) {
+            const piece* l = lds[cur] + u * kSubPieces;
+            piece fa[2][P];
 #pragma unroll
-            for (int p = 0; p < 3; ++p) fa[i][p] = l[a_lane + p * 2 * BM + 32 * i];
+            for (int i = 0; i < 2; ++i)
 #pragma unroll
-        for (int j = 0; j < JT; ++j) {
-            piece fb[3];
+                for (int p = 0; p < P; ++p) fa[i][p] = l[a_lane + p * 2 * BM + 32 * i];
 #pragma unroll
-            for (int p = 0; p < 3; ++p) fb[p] = l[b_lane + p * 2 * BN + 32 * j];
-            // the six plane pairs (pa, pb) with pa + pb <= 2, smallest terms first
-            constexpr int kPa[6] = {0, 1, 2, 0, 1, 0};
-            constexpr int kPb[6] = {2, 1, 0, 1, 0, 0};
+            for (int j = 0; j < JT; ++j) {
+                piece fb[P];
 #pragma unroll
-            for (int t6 = 0; t6 < 6; ++t6)
+                for (int p = 0; p < P; ++p) fb[p] = l[b_lane + p * 2 * BN + 32 * j];
+                if constexpr (P == 3) {
+                    // the six plane pairs (pa, pb) with pa + pb <= 2, smallest terms first
+                    constexpr int kPa[6] = {0, 1, 2, 0, 1, 0};
+                    constexpr int kPb[6] = {2, 1, 0, 1, 0, 0};
 #pragma unroll
-                for (int i = 0; i < 2; ++i) acc[i][j] = mfma_bf16(fa[i][kPa[t6]], fb[kPb[t6]], acc[i][j]);
+                    for (int t6 = 0; t6 < 6; ++t6)
+#pragma unroll
+                        for (int i = 0; i < 2; ++i)
+                            acc[i][j] = mfma16<F16>(fa[i][kPa[t6]], fb[kPb[t6]], acc[i][j]);
+                } else {
+#pragma unroll
+                    for (int i = 0; i < 2; ++i) acc[i][j] = mfma16<F16>(fa[i][0], fb[0], acc[i][j]);
+                }
+            }
         }
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wave's pieces of the next step are in LDS
         __syncthreads();
@@ -238,61 +283,86 @@ __global__ __launch_bounds__(256) void mirror_lower_kernel(float* __restrict__ C
 }
 
 uint64_t padded_rows(uint64_t rows) { return (rows + kRowPad - 1) / kRowPad * kRowPad; }
-uint64_t octets(uint64_t K) { return (K + 15) / 16 * 2; }
+uint64_t octets(uint64_t K) { return (K + 8 * kOctetPad - 1) / (8 * kOctetPad) * kOctetPad; }
+int planes_of(int dtype) { return dtype == TRAKHIP_F32 ? 3 : 1; }
+bool known_dtype(int dtype) { return dtype == TRAKHIP_F16 || dtype == TRAKHIP_BF16 || dtype == TRAKHIP_F32; }
 
 }  // namespace
 
 namespace trakhip {
 
-size_t split_bytes(uint64_t rows, uint64_t K) {
-    if (rows == 0 || K == 0) return 0;
-    return (size_t)(3 * octets(K) * padded_rows(rows) * 16);
+size_t split_bytes(uint64_t rows, uint64_t K, int dtype) {
+    if (rows == 0 || K == 0 || !known_dtype(dtype)) return 0;
+    return (size_t)(planes_of(dtype) * octets(K) * padded_rows(rows) * 16);
 }
 
-int split_rows(const float* src, uint64_t ld, uint64_t rows, uint64_t K, int transposed, void* planes,
+int split_rows(const void* src, int dtype, uint64_t ld, uint64_t rows, uint64_t K, int transposed, void* planes,
                size_t planes_bytes, hipStream_t s) {
+    if (!known_dtype(dtype)) return TRAKHIP_ERR_DTYPE;
     if (rows == 0 || K == 0) return TRAKHIP_ERR_SHAPE;
     if (ld < (transposed ? rows : K)) return TRAKHIP_ERR_SHAPE;
     if (!src || !planes) return TRAKHIP_ERR_NULL;
-    if (planes_bytes < split_bytes(rows, K)) return TRAKHIP_ERR_WORKSPACE;
-    if ((reinterpret_cast<uintptr_t>(src) % 4) || (reinterpret_cast<uintptr_t>(planes) % 16)) return TRAKHIP_ERR_ALIGN;
+    if (planes_bytes < split_bytes(rows, K, dtype)) return TRAKHIP_ERR_WORKSPACE;
+    const size_t esz = dtype == TRAKHIP_F32 ? 4 : 2;
+    if ((reinterpret_cast<uintptr_t>(src) % esz) || (reinterpret_cast<uintptr_t>(planes) % 16)) return TRAKHIP_ERR_ALIGN;
     const uint64_t Rp = padded_rows(rows), K8 = octets(K);
     const uint64_t gx = Rp / 64, gy = (K8 + 3) / 4;
     if (gx * gy > 0x7FFFFFFFull) return TRAKHIP_ERR_SHAPE;
     const dim3 grid((uint32_t)(gx * gy)), block(256);
     uint4* out = static_cast<uint4*>(planes);
-    const bool aligned = reinterpret_cast<uintptr_t>(src) % 16 == 0 && ld % 4 == 0;
-    if (transposed)
-        hipLaunchKernelGGL((split_kernel<true, false>), grid, block, 0, s, src, ld, rows, K, Rp, K8, (uint32_t)gx, out);
-    else if (aligned)
-        hipLaunchKernelGGL((split_kernel<false, true>), grid, block, 0, s, src, ld, rows, K, Rp, K8, (uint32_t)gx, out);
-    else
-        hipLaunchKernelGGL((split_kernel<false, false>), grid, block, 0, s, src, ld, rows, K, Rp, K8, (uint32_t)gx, out);
+    // 16-byte loads of 8 (fp32: 4) consecutive values need the row starts aligned
+    const bool aligned = reinterpret_cast<uintptr_t>(src) % 16 == 0 && (ld * esz) % 16 == 0;
+    if (dtype == TRAKHIP_F32) {
+        const float* f = static_cast<const float*>(src);
+        if (transposed)
+            hipLaunchKernelGGL((split_kernel<true, false>), grid, block, 0, s, f, ld, rows, K, Rp, K8, (uint32_t)gx, out);
+        else if (aligned)
+            hipLaunchKernelGGL((split_kernel<false, true>), grid, block, 0, s, f, ld, rows, K, Rp, K8, (uint32_t)gx, out);
+        else
+            hipLaunchKernelGGL((split_kernel<false, false>), grid, block, 0, s, f, ld, rows, K, Rp, K8, (uint32_t)gx, out);
+    } else {
+        const uint16_t* h = static_cast<const uint16_t*>(src);
+        if (transposed)
+            hipLaunchKernelGGL((relayout16_kernel<true, false>), grid, block, 0, s, h, ld, rows, K, Rp, K8, (uint32_t)gx, out);
+        else if (aligned)
+            hipLaunchKernelGGL((relayout16_kernel<false, true>), grid, block, 0, s, h, ld, rows, K, Rp, K8, (uint32_t)gx, out);
+        else
+            hipLaunchKernelGGL((relayout16_kernel<false, false>), grid, block, 0, s, h, ld, rows, K, Rp, K8, (uint32_t)gx, out);
+    }
     return hipGetLastError() == hipSuccess ? TRAKHIP_OK : TRAKHIP_ERR_LAUNCH;
 }
 
-int gemm_nt_split(const void* A_planes, uint64_t M, const void* B_planes, uint64_t N, uint64_t K, float* C,
+int gemm_nt_split(const void* A_planes, uint64_t M, const void* B_planes, uint64_t N, uint64_t K, int dtype, float* C,
                   uint64_t ldc, float alpha, float beta, const float* row_scale, hipStream_t s, uint32_t flags) {
+    if (!known_dtype(dtype)) return TRAKHIP_ERR_DTYPE;
     if (M == 0 || N == 0) return TRAKHIP_OK;
     if (K == 0 || ldc < N) return TRAKHIP_ERR_SHAPE;
     if (!A_planes || !B_planes || !C) return TRAKHIP_ERR_NULL;
     if ((reinterpret_cast<uintptr_t>(A_planes) % 16) || (reinterpret_cast<uintptr_t>(B_planes) % 16) ||
         (reinterpret_cast<uintptr_t>(C) % 4))
         return TRAKHIP_ERR_ALIGN;
-    constexpr int BM = 64 * kWavesM;
     const uint64_t tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
     if (tiles_m * tiles_n > 0x7FFFFFFFull) return TRAKHIP_ERR_SHAPE;
-    hipLaunchKernelGGL((gemm_split_kernel<kWavesM, kWavesN>), dim3((uint32_t)(tiles_m * tiles_n)),
-                       dim3(64 * kWavesM * kWavesN), 0, s,
-                       static_cast<const piece*>(A_planes), padded_rows(M), static_cast<const piece*>(B_planes),
-                       padded_rows(N), octets(K), C, ldc, M, N, alpha, beta, row_scale, (uint32_t)tiles_n, flags);
+    const dim3 grid((uint32_t)(tiles_m * tiles_n)), block(64 * kWaves);
+    const piece* a = static_cast<const piece*>(A_planes);
+    const piece* b = static_cast<const piece*>(B_planes);
+    const uint64_t Rpa = padded_rows(M), Rpb = padded_rows(N), K8 = octets(K);
+    if (dtype == TRAKHIP_F32)
+        hipLaunchKernelGGL((gemm_split_kernel<3, false, 1>), grid, block, 0, s, a, Rpa, b, Rpb, K8, C, ldc, M, N, alpha,
+                           beta, row_scale, (uint32_t)tiles_n, flags);
+    else if (dtype == TRAKHIP_F16)
+        hipLaunchKernelGGL((gemm_split_kernel<1, true, 4>), grid, block, 0, s, a, Rpa, b, Rpb, K8, C, ldc, M, N, alpha,
+                           beta, row_scale, (uint32_t)tiles_n, flags);
+    else
+        hipLaunchKernelGGL((gemm_split_kernel<1, false, 4>), grid, block, 0, s, a, Rpa, b, Rpb, K8, C, ldc, M, N, alpha,
+                           beta, row_scale, (uint32_t)tiles_n, flags);
     return hipGetLastError() == hipSuccess ? TRAKHIP_OK : TRAKHIP_ERR_LAUNCH;
 }
 
-int gram_split(const void* A_planes, uint64_t N, uint64_t K, float* C, uint64_t ldc, float alpha, float beta,
+int gram_split(const void* A_planes, uint64_t N, uint64_t K, int dtype, float* C, uint64_t ldc, float alpha, float beta,
                hipStream_t s) {
     if (N == 0) return TRAKHIP_OK;
-    const int e = gemm_nt_split(A_planes, N, A_planes, N, K, C, ldc, alpha, beta, nullptr, s, kGemmLowerTilesOnly);
+    const int e = gemm_nt_split(A_planes, N, A_planes, N, K, dtype, C, ldc, alpha, beta, nullptr, s, kGemmLowerTilesOnly);
     if (e) return e;
     const uint64_t blocks = (N + 31) / 32;
     if (blocks > 65535) return TRAKHIP_ERR_SHAPE;

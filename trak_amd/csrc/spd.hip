@@ -278,7 +278,7 @@ namespace trakhip {
 // Workspace: three np x np matrices (W, L, Li), the reduction scratch, and for small n a tail for the
 // split planes of Li^T (for np >= 384 they fit into W and L, which are free by then).
 static size_t planes_tail_bytes(uint64_t n, uint64_t np) {
-    const size_t planes = split_bytes(n, n), free_front = (size_t)(2 * np * np) * sizeof(float);
+    const size_t planes = split_bytes(n, n, TRAKHIP_F32), free_front = (size_t)(2 * np * np) * sizeof(float);
     return planes > free_front ? planes : 0;
 }
 
@@ -333,8 +333,8 @@ int spd_inverse(const float* A, uint64_t lda, float lambda, float* inv, uint64_t
     // symmetric product of the split operand Li^T, lower-triangle tiles mirrored, so the result is
     // exactly symmetric.  The planes go where W and L were (or behind the scratch for small n).
     void* planes = planes_tail_bytes(n, np) ? static_cast<void*>(mean_dev + 4) : static_cast<void*>(W);
-    e = split_rows(Li, np, n, n, 1, planes, split_bytes(n, n), s);
-    if (!e) e = gram_split(planes, n, n, inv, ldi, 1.0f, 0.0f, s);
+    e = split_rows(Li, TRAKHIP_F32, np, n, n, 1, planes, split_bytes(n, n, TRAKHIP_F32), s);
+    if (!e) e = gram_split(planes, n, n, TRAKHIP_F32, inv, ldi, 1.0f, 0.0f, s);
     if (e) return e;
 
     if (normalize || mean_abs) {

@@ -49,12 +49,13 @@ int gemm_tn(const float* A, uint64_t lda, const float* B, uint64_t ldb, float* C
             uint64_t N, uint64_t K, float alpha, float beta, hipStream_t s, uint32_t flags = 0);
 int gemm_nn(const float* A, uint64_t lda, const float* B, uint64_t ldb, float* C, uint64_t ldc, uint64_t M,
             uint64_t N, uint64_t K, float alpha, float beta, hipStream_t s, uint32_t flags = 0);
-size_t split_bytes(uint64_t rows, uint64_t K);
-int split_rows(const float* src, uint64_t ld, uint64_t rows, uint64_t K, int transposed, void* planes,
+// dtype = element type of the source matrices (TRAKHIP_F32: three bf16 planes; F16 / BF16: one plane)
+size_t split_bytes(uint64_t rows, uint64_t K, int dtype);
+int split_rows(const void* src, int dtype, uint64_t ld, uint64_t rows, uint64_t K, int transposed, void* planes,
                size_t planes_bytes, hipStream_t s);
-int gemm_nt_split(const void* A_planes, uint64_t M, const void* B_planes, uint64_t N, uint64_t K, float* C,
+int gemm_nt_split(const void* A_planes, uint64_t M, const void* B_planes, uint64_t N, uint64_t K, int dtype, float* C,
                   uint64_t ldc, float alpha, float beta, const float* row_scale, hipStream_t s, uint32_t flags = 0);
-int gram_split(const void* A_planes, uint64_t N, uint64_t K, float* C, uint64_t ldc, float alpha, float beta,
+int gram_split(const void* A_planes, uint64_t N, uint64_t K, int dtype, float* C, uint64_t ldc, float alpha, float beta,
                hipStream_t s);
 size_t spd_inverse_workspace_bytes(uint64_t n);
 int spd_inverse(const float* A, uint64_t lda, float lambda, float* inv, uint64_t ldi, uint64_t n,

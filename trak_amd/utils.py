@@ -153,11 +153,11 @@ def gemm_tn(a, b, out=None, alpha=1.0, beta=0.0):
 
 
 class SplitOperand:
-    """An fp32 matrix [rows, K] stored as three bf16 planes whose sum is the matrix exactly (the
-    operand format of `gemm_nt_split`)."""
+    """A matrix [rows, K] in the operand format of `gemm_nt_split`: three bf16 planes whose sum is
+    the matrix exactly (fp32 source) or the matrix itself as one plane (fp16 / bf16 source)."""
 
-    def __init__(self, planes, rows, K):
-        self.planes, self.rows, self.K = planes, int(rows), int(K)
+    def __init__(self, planes, rows, K, dtype):
+        self.planes, self.rows, self.K, self.dtype = planes, int(rows), int(K), dtype
 
     @property
     def device(self):
@@ -165,32 +165,48 @@ class SplitOperand:
 
 
 def split_rows(t, transposed=False):
-    """Splits the fp32 CUDA matrix `t` for `gemm_nt_split`.  transposed=False: the operand is `t`
-    itself ([rows, K]); transposed=True: the operand is `t.T` (t is [K, rows]), read in place."""
-    t = _as_f32_rows(t, "t")
+    """Brings the CUDA matrix `t` (fp32, fp16 or bf16; anything else is converted to fp32) into the
+    operand format of `gemm_nt_split`.  transposed=False: the operand is `t` itself ([rows, K]);
+    transposed=True: the operand is `t.T` (t is [K, rows]), read in place."""
+    if t.dim() != 2:
+        raise RuntimeError("t must be 2D")
+    if t.dtype not in _STORE_DTYPES:
+        t = t.float()
+    if t.stride(1) != 1 or (t.shape[0] > 1 and t.stride(0) < t.shape[1]):
+        t = t.contiguous()
     if not t.is_cuda:
         raise RuntimeError("split_rows needs a CUDA tensor")
     rows, K = (t.shape[1], t.shape[0]) if transposed else (t.shape[0], t.shape[1])
     lib = _lib.load()
-    nbytes = lib.trakhip_split_bytes(rows, K)
+    code_dtype = _STORE_DTYPES[t.dtype]
+    nbytes = lib.trakhip_split_bytes(rows, K, code_dtype)
     with torch.cuda.device(t.device):
         planes = torch.empty(max(nbytes, 16), dtype=torch.uint8, device=t.device)
         stream = torch.cuda.current_stream(t.device).cuda_stream
         code = lib.trakhip_split_rows(
-            ctypes.c_void_p(t.data_ptr()), _ld(t), rows, K, int(bool(transposed)),
+            ctypes.c_void_p(t.data_ptr()), code_dtype, _ld(t), rows, K, int(bool(transposed)),
             ctypes.c_void_p(planes.data_ptr()), planes.numel(), ctypes.c_void_p(stream),
         )
     _lib.check(code)
-    return SplitOperand(planes, rows, K)
+    return SplitOperand(planes, rows, K, t.dtype)
+
+
+def split_pair(a, b, a_transposed=False):
+    """Both operands of one product in a common format: 16-bit operands of one type stay as they
+    are (one plane each), any other combination is multiplied from fp32 splits."""
+    if a.dtype != b.dtype or a.dtype not in (torch.float16, torch.bfloat16):
+        a, b = a.float(), b.float()
+    return split_rows(a, transposed=a_transposed), split_rows(b)
 
 
 def gemm_nt_split(a, b, out=None, alpha=1.0, beta=0.0, row_scale=None):
     """out[M, N] = alpha * A @ B.T + beta * out (rows optionally scaled) for SplitOperands A [M, K]
-    and B [N, K]: six bf16 MFMAs per k step with fp32 accumulation, fp32-level accuracy."""
+    and B [N, K] made from matrices of one dtype: exact products on the 16-bit matrix cores, fp32
+    accumulation, fp32-level accuracy."""
     if not isinstance(a, SplitOperand) or not isinstance(b, SplitOperand):
         raise TypeError("gemm_nt_split takes SplitOperand arguments (see split_rows)")
-    if a.K != b.K or a.device != b.device:
-        raise RuntimeError("operands must share the inner dimension and the device")
+    if a.K != b.K or a.device != b.device or a.dtype != b.dtype:
+        raise RuntimeError("operands must share the inner dimension, the device and the source dtype")
     M, N, K = a.rows, b.rows, a.K
     if out is None:
         out = torch.empty((M, N), dtype=torch.float32, device=a.device)
@@ -207,7 +223,7 @@ def gemm_nt_split(a, b, out=None, alpha=1.0, beta=0.0, row_scale=None):
         stream = torch.cuda.current_stream(a.device).cuda_stream
         code = lib.trakhip_gemm_nt_split(
             ctypes.c_void_p(a.planes.data_ptr()), M, ctypes.c_void_p(b.planes.data_ptr()), N, K,
-            ctypes.c_void_p(out.data_ptr()), _ld(out), float(alpha), float(beta),
+            _STORE_DTYPES[a.dtype], ctypes.c_void_p(out.data_ptr()), _ld(out), float(alpha), float(beta),
             ctypes.c_void_p(rs.data_ptr()) if rs is not None else None, ctypes.c_void_p(stream),
         )
     _lib.check(code)
@@ -230,8 +246,8 @@ def gram_split(a, out=None, alpha=1.0, beta=0.0):
     with torch.cuda.device(a.device):
         stream = torch.cuda.current_stream(a.device).cuda_stream
         code = lib.trakhip_gram_split(
-            ctypes.c_void_p(a.planes.data_ptr()), N, a.K, ctypes.c_void_p(out.data_ptr()), _ld(out),
-            float(alpha), float(beta), ctypes.c_void_p(stream),
+            ctypes.c_void_p(a.planes.data_ptr()), N, a.K, _STORE_DTYPES[a.dtype], ctypes.c_void_p(out.data_ptr()),
+            _ld(out), float(alpha), float(beta), ctypes.c_void_p(stream),
         )
     _lib.check(code)
     return out
@@ -333,5 +349,5 @@ def get_matrix_mult(features, target_grads, target_dtype=None, batch_size=8096, 
         target_dtype = features.dtype
     if features.device.type == "cpu":
         return (features @ target_grads.t()).clone().to(target_dtype)
-    out = gemm_nt_split(split_rows(features), split_rows(target_grads.to(features.device)))
+    out = gemm_nt_split(*split_pair(features, target_grads.to(features.device)))
     return out.to(target_dtype)
