@@ -74,7 +74,7 @@ def test_one_hot_rows_read_the_matrix_back_exactly(gpu, c_oracle, proj_type, dty
 @pytest.mark.parametrize(
     "B,P,k,tiles",
     [(32, 20_000, 512, 256), (16, 10_002, 1024, 256), (9, 10_001, 512, 108), (1, 25, 512, 256), (45, 1049, 512, 256),
-     (8, 70_001, 512, 7)],
+     (8, 70_001, 512, 7), (32, 9_000, 1536, 256), (12, 5_003, 2048, 64), (32, 6_001, 2560, 256)],
 )
 def test_projection_matches_float64_contraction(gpu, c_oracle, proj_type, dtype, B, P, k, tiles):
     gen = torch.Generator(device="cpu").manual_seed(1000 + B + P)
@@ -82,7 +82,9 @@ def test_projection_matches_float64_contraction(gpu, c_oracle, proj_type, dtype,
     seed = 123 + B
     out = fn(proj_type)(g, k, seed, tiles)
     assert out.shape == (B, k) and out.dtype == torch.float32 and out.device == g.device  # fast_jl.cu:48-49,78
-    cols = [0, 31, 32, 511] if k == 512 else [0, 500, 1023]
+    # 512-, 1024- and 1536-column boundaries: four-wave workgroups (k an odd multiple of 512) cover 512
+    # columns, eight-wave ones 1024
+    cols = [c for c in (0, 31, 32, 511, 512, 1023, 1024, 1535, 2047, 2559) if c < k]
     g32 = to_f32_numpy(g)
     for c in cols:
         want = c_oracle.project(g32, seed, tiles, c, 1, proj_type)
