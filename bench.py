@@ -267,7 +267,7 @@ def bench_store_paths(torch, dev):
     def reference_batch(i):
         x = proj.project(g, 0)
         x /= nf
-        store[i * B:(i + 1) * B] = x.to(torch.float16).cpu().clone().detach()
+        store[i * B:(i + 1) * B] = x.to(torch.float16).cpu().clone().detach().numpy()
 
     writer = FeatureWriter(proj, k, nf, dtype=torch.float16, max_batch_size=B, depth=2)
 
