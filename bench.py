@@ -380,6 +380,7 @@ def bench_scoring(torch, dev, reps=3):
         "gemm_frac_fp32_mfma_peak": gemm_flop / (gemm_ms * 1e-3) / 1e12 / PEAK_FP32_TFLOPS,
         "split_bf16x3": {
             "xtx_ms": s_xtx, "x_xtx_inv_ms": s_feat, "scores_ms": s_sc,
+            "gemm_tflops_algorithmic": gemm_flop / (split_ms * 1e-3) / 1e12,  # 4*N*k*k + 2*N*M*k over the time
             "gemm_tflops_fp32_equivalent": split_flop / (split_ms * 1e-3) / 1e12,
             "frac_fp32_mfma_peak": split_flop / (split_ms * 1e-3) / 1e12 / PEAK_FP32_TFLOPS,
             "bf16_mfma_tflops_executed": 6 * split_flop / (split_ms * 1e-3) / 1e12,
@@ -416,9 +417,9 @@ def cpu_baseline(torch):
         "value": flop / dt / 1e12, "unit": "TFLOP/s", "cores": cores, "kind": "port",
         "sample": f"BasicProjector restatement, full config [16,1048576] fp32 -> 512 rademacher, {dt:.2f} s",
     }
-    N, M, kk = 20_000, 4_000, 2048
-    X = torch.randn(N, kk, generator=gen) / 32
-    Xt = torch.randn(M, kk, generator=gen) / 32
+    N, M, kk = 50_000, 10_000, 4096  # the scoring configuration in full
+    X = torch.randn(N, kk, generator=gen) / 64
+    Xt = torch.randn(M, kk, generator=gen) / 64
     sc = BasicScoreComputerCPU(lambda_reg=1e-3)
     t0 = time.perf_counter()
     xtx = sc.get_xtx(X)
@@ -428,6 +429,11 @@ def cpu_baseline(torch):
     dts = time.perf_counter() - t0
     res["scoring_tflops"] = (4.0 * N * kk * kk + 2.0 * N * M * kk) / dts / 1e12
     res["scoring_sample"] = f"BasicScoreComputer restatement N={N}, M={M}, k={kk} fp32, {dts:.2f} s (inverse included)"
+    try:
+        with open("/proc/cpuinfo") as f:
+            res["cpu_model"] = next(l.split(":", 1)[1].strip() for l in f if l.startswith("model name"))
+    except (OSError, StopIteration):
+        res["cpu_model"] = "unknown"
     return res
 
 
