@@ -272,3 +272,42 @@ def test_featurize_finalize_score_through_the_saver(gpu, tmp_path):
     got = np.load(tmp_path / "scores" / "t.mmap", mmap_mode="r")
     assert got.shape == (N, M)
     assert np.abs(np.asarray(got, dtype=np.float64) - want).max() <= 1e-4 * np.abs(want).max()
+
+
+def test_projection_and_scoring_replay_from_a_hip_graph(gpu):
+    """The library only launches kernels on the caller's stream (no allocation, no memset, no sync), so a
+    caller can capture it: a captured projection + epilogue + score product is replayed three times
+    with new inputs, with eager work and synchronizations in between, and must equal the eager
+    result bit for bit every time."""
+    B, P, k, M = 32, 30_000, 1024, 96
+    gen = torch.Generator(device=gpu).manual_seed(5)
+    g_static = torch.zeros(B, P, dtype=torch.float16, device=gpu)
+    targets = torch.randn(M, k, generator=gen, device=gpu)
+    feats = torch.empty(B, k, dtype=torch.float32, device=gpu)
+    scores = torch.empty(B, M, device=gpu)
+    from trak_amd.utils import split_rows
+
+    def work():
+        fast_jl.project_into(g_static, k, 3, 64, "rademacher", feats, 0.125)
+        gemm_nt(feats, targets, out=scores)
+
+    work()  # warm-up: sizes the cached workspace outside the capture
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            work()
+    torch.cuda.current_stream().wait_stream(side)
+    for rep in range(3):
+        g_new = (torch.randn(B, P, generator=gen, device=gpu) * 0.01).half()
+        g_static.copy_(g_new)
+        graph.replay()
+        torch.cuda.synchronize()
+        got_feats, got_scores = feats.clone(), scores.clone()
+        work()                                   # eager, same buffers
+        torch.cuda.synchronize()
+        assert torch.equal(got_feats, feats) and torch.equal(got_scores, scores), rep
+        assert float(got_scores.abs().sum()) > 0
+        _ = split_rows(targets)                  # unrelated eager work between replays
