@@ -39,6 +39,25 @@ def test_gemm_nt(gpu, M, N, K):
     assert rel_max(got.cpu().numpy(), want2) < gemm_tol(K)
 
 
+@pytest.mark.parametrize("M,N,K", [(130, 70, 40), (300, 515, 128), (129, 1, 8), (2100, 2050, 128), (4000, 3000, 120)])
+def test_gemm_nt_short_contraction(gpu, M, N, K):
+    """K <= 128 in multiples of 8 with aligned rows takes the kernel that holds both operand tiles
+    whole (up to 512 tiles); ragged edges, accumulation into C, and the hand-over to the general
+    kernel above that tile count."""
+    gen = torch.Generator(device="cpu").manual_seed(M + 3 * N + K)
+    a, b = torch.randn(M, K, generator=gen), torch.randn(N, K, generator=gen)
+    c0 = torch.randn(M, N, generator=gen)
+    want = a.double().numpy() @ b.double().numpy().T
+    got = gemm_nt(a.to(gpu), b.to(gpu))
+    assert rel_max(got.cpu().numpy(), want) < gemm_tol(K)
+    got = gemm_nt(a.to(gpu), b.to(gpu), out=c0.clone().to(gpu), alpha=-1.0, beta=1.0)
+    assert rel_max(got.cpu().numpy(), c0.double().numpy() - want) < gemm_tol(K)
+    # a padded destination keeps its padding
+    wide = torch.full((M, N + 5), 7.0, device=gpu)
+    gemm_nt(a.to(gpu), b.to(gpu), out=wide[:, :N])
+    assert rel_max(wide[:, :N].cpu().numpy(), want) < gemm_tol(K) and bool((wide[:, N:] == 7.0).all())
+
+
 @pytest.mark.parametrize("M,N,K", [(128, 128, 16), (96, 200, 1000), (33, 17, 5), (512, 512, 2050)])
 def test_gemm_tn(gpu, M, N, K):
     gen = torch.Generator(device="cpu").manual_seed(M + N + K)

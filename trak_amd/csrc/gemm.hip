@@ -214,6 +214,121 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_nn_batched_kernel(const floa
                                     beta, nullptr, tiles_n, 0u, blockIdx.x);
 }
 
+// NT product with a short contraction (K <= 128, the panel width of the blocked factorization):
+// C[M, N] = alpha * A[M, K] * B[N, K]^T + beta * C, 128 x 128 tiles.  The general kernel walks k in
+// steps of 16 with one global-memory round trip per step, which is all latency when there are
+// only eight steps; here both operand tiles are loaded whole (one round trip, 135 KB of LDS, one
+// barrier) and the MFMAs run back to back.  Needs 16-byte aligned rows and K a multiple of 8.
+constexpr int kShortK = 128;
+constexpr int kShortStride = kShortK + 4;  // floats; 528-byte rows keep 16-byte reads conflict free
+
+__global__ __launch_bounds__(kThreads, 1) void gemm_nt_short_k_kernel(const float* __restrict__ A, uint64_t lda,
+                                                                      const float* __restrict__ B, uint64_t ldb,
+                                                                      float* __restrict__ C, uint64_t ldc, uint64_t M,
+                                                                      uint64_t N, uint32_t K, float alpha, float beta,
+                                                                      uint32_t tiles_n, uint32_t flags) {
+    __shared__ __attribute__((aligned(16))) float lds[2 * BM * kShortStride];
+    // With kGemmLowerTilesOnly the grid holds the lower-triangle tiles alone, numbered row by row
+    // (a workgroup that only returns would still wait for a CU with this much LDS free).
+    uint32_t tile_m, tile_n;
+    if (flags & trakhip::kGemmLowerTilesOnly) {
+        tile_m = (uint32_t)((sqrtf(8.0f * (float)blockIdx.x + 1.0f) - 1.0f) * 0.5f);
+        while (tile_m * (tile_m + 1) / 2 > blockIdx.x) --tile_m;
+        while ((tile_m + 1) * (tile_m + 2) / 2 <= blockIdx.x) ++tile_m;
+        tile_n = blockIdx.x - tile_m * (tile_m + 1) / 2;
+    } else {
+        tile_m = blockIdx.x / tiles_n;
+        tile_n = blockIdx.x % tiles_n;
+    }
+    const uint64_t m0 = (uint64_t)tile_m * BM, n0 = (uint64_t)tile_n * BM;
+    const int tid = threadIdx.x;
+    const int wave = tid >> 6, lane = tid & 63;
+    const int wm = wave >> 1, wn = wave & 1;
+    const int x = lane & 31, h = lane >> 5;
+
+    // 128 rows x 32 float4 per operand = 16 pieces per thread and operand, all in flight at once
+    constexpr int kPiecesPerThread = BM * (kShortK / 4) / kThreads;
+    float4 ra[kPiecesPerThread], rb[kPiecesPerThread];
+#pragma unroll
+    for (int i = 0; i < kPiecesPerThread; ++i) {
+        const int id = tid + kThreads * i;
+        const uint32_t row = id >> 5, k4 = 4 * (id & 31);
+        ra[i] = (m0 + row < M && k4 < K) ? *reinterpret_cast<const float4*>(A + (m0 + row) * lda + k4)
+                                         : make_float4(0.f, 0.f, 0.f, 0.f);
+        rb[i] = (n0 + row < N && k4 < K) ? *reinterpret_cast<const float4*>(B + (n0 + row) * ldb + k4)
+                                         : make_float4(0.f, 0.f, 0.f, 0.f);
+    }
+    float* as = lds;
+    float* bs = lds + BM * kShortStride;
+#pragma unroll
+    for (int i = 0; i < kPiecesPerThread; ++i) {
+        const int id = tid + kThreads * i;
+        const uint32_t row = id >> 5, k4 = 4 * (id & 31);
+        *reinterpret_cast<float4*>(as + row * kShortStride + k4) = ra[i];
+        *reinterpret_cast<float4*>(bs + row * kShortStride + k4) = rb[i];
+    }
+    __syncthreads();
+
+    floatx16 acc[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+    // the old values of C are fetched here, so that their latency passes under the MFMAs
+    floatx16 prev[2][2];
+    if (beta != 0.0f) {
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+#pragma unroll
+            for (int j = 0; j < 2; ++j)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const uint64_t row = m0 + wm * 64 + 32 * i + 8 * (r >> 2) + 4 * h + (r & 3);
+                    const uint64_t col = n0 + wn * 64 + 32 * j + x;
+                    prev[i][j][r] = (row < M && col < N) ? C[row * ldc + col] : 0.f;
+                }
+    }
+    // lane half h takes k = 8 s + 4 h + t for the t-th MFMA of sub-step s, as in the general kernel
+    for (uint32_t s = 0; s < K / 8; ++s) {
+        float4 fa[2], fb[2];
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+            fa[i] = *reinterpret_cast<const float4*>(as + (wm * 64 + 32 * i + x) * kShortStride + 8 * s + 4 * h);
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+            fb[j] = *reinterpret_cast<const float4*>(bs + (wn * 64 + 32 * j + x) * kShortStride + 8 * s + 4 * h);
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+#pragma unroll
+            for (int i = 0; i < 2; ++i)
+#pragma unroll
+                for (int j = 0; j < 2; ++j) {
+                    const float av = t == 0 ? fa[i].x : (t == 1 ? fa[i].y : (t == 2 ? fa[i].z : fa[i].w));
+                    const float bv = t == 0 ? fb[j].x : (t == 1 ? fb[j].y : (t == 2 ? fb[j].z : fb[j].w));
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(av, bv, acc[i][j], 0, 0, 0);
+                }
+    }
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const uint64_t row = m0 + wm * 64 + 32 * i + 8 * (r >> 2) + 4 * h + (r & 3);
+            if (row >= M) continue;
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                const uint64_t col = n0 + wn * 64 + 32 * j + x;
+                if (col >= N) continue;
+                float* c = C + row * ldc + col;
+                float v = alpha * acc[i][j][r];
+                if (beta != 0.0f) v += beta * prev[i][j][r];
+                *c = v;
+            }
+        }
+    }
+}
+
 template <bool AK, bool BK, int WN>
 int launch_tiles(const float* A, uint64_t lda, const float* B, uint64_t ldb, float* C, uint64_t ldc, uint64_t M,
                  uint64_t N, uint64_t K, float alpha, float beta, const float* row_scale, bool aligned,
@@ -253,6 +368,23 @@ namespace trakhip {
 
 int gemm_nt(const float* A, uint64_t lda, const float* B, uint64_t ldb, float* C, uint64_t ldc, uint64_t M,
             uint64_t N, uint64_t K, float alpha, float beta, const float* row_scale, hipStream_t s, uint32_t flags) {
+    const bool aligned = A && B && (reinterpret_cast<uintptr_t>(A) % 16 == 0) &&
+                         (reinterpret_cast<uintptr_t>(B) % 16 == 0) && (lda % 4 == 0) && (ldb % 4 == 0);
+    if (M && N && C && aligned && !row_scale && K >= 8 && K <= kShortK && K % 8 == 0 && lda >= K && ldb >= K &&
+        ldc >= N) {
+        const uint64_t tm = (M + BM - 1) / BM, tn = (N + BM - 1) / BM;
+        // one workgroup per CU (its LDS) and no overlap between them: only while one round covers the launch
+        // Lower tiles only: a square tile grid is launched as its triangle; otherwise the flag is dropped
+        // (computing the upper tiles too is allowed, skipping them is an optimisation).
+        const bool triangle = (flags & kGemmLowerTilesOnly) && tm == tn;
+        const uint64_t working = triangle ? tm * (tm + 1) / 2 : tm * tn;
+        // one workgroup per CU (its LDS) and no overlap inside it: worth it for up to two rounds
+        if (working <= 512 && (triangle || !(flags & kGemmLowerTilesOnly))) {
+            hipLaunchKernelGGL(gemm_nt_short_k_kernel, dim3((uint32_t)working), dim3(kThreads), 0, s, A, lda, B, ldb, C,
+                               ldc, M, N, (uint32_t)K, alpha, beta, (uint32_t)tn, triangle ? kGemmLowerTilesOnly : 0u);
+            return hipGetLastError() == hipSuccess ? TRAKHIP_OK : TRAKHIP_ERR_LAUNCH;
+        }
+    }
     return launch<false, false>(A, lda, B, ldb, C, ldc, M, N, K, alpha, beta, row_scale, flags, s);
 }
 
