@@ -170,22 +170,35 @@ __device__ __forceinline__ void gemm_tile(const float* __restrict__ A, uint64_t 
     }
 
     // D[m][n] of a 32x32 MFMA: lane holds column n = lane % 32; register r holds row
-    // 8*(r/4) + 4*(lane/32) + r%4.
+    // 8*(r/4) + 4*(lane/32) + r%4.  When C is accumulated into, its old values are fetched for 32 rows
+    // at a time before any of them is overwritten (loads and stores through one pointer would
+    // otherwise alternate, one memory round trip per element).
+    const uint64_t col0 = n0 + wn * (32 * WN) + x;
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
+        const uint64_t row0 = m0 + wm * 64 + 32 * i + 4 * h;
+        floatx16 prev[WN];
+        if (beta != 0.0f) {
+#pragma unroll
+            for (int j = 0; j < WN; ++j)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const uint64_t row = row0 + 8 * (r >> 2) + (r & 3), col = col0 + 32 * j;
+                    prev[j][r] = (row < M && col < N) ? C[row * ldc + col] : 0.0f;
+                }
+        }
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
-            const uint64_t row = m0 + wm * 64 + 32 * i + 8 * (r >> 2) + 4 * h + (r & 3);
+            const uint64_t row = row0 + 8 * (r >> 2) + (r & 3);
             if (row >= M) continue;
             const float rs = row_scale ? row_scale[row] : 1.0f;
 #pragma unroll
             for (int j = 0; j < WN; ++j) {
-                const uint64_t col = n0 + wn * (32 * WN) + 32 * j + x;
+                const uint64_t col = col0 + 32 * j;
                 if (col >= N) continue;
-                float* c = C + row * ldc + col;
                 float v = alpha * acc[i][j][r];
-                if (beta != 0.0f) v += beta * *c;
-                *c = v * rs;
+                if (beta != 0.0f) v += beta * prev[j][r];
+                C[row * ldc + col] = v * rs;
             }
         }
     }

@@ -167,7 +167,7 @@ __device__ __forceinline__ void dma_step(const piece* __restrict__ A, uint64_t R
 
 // P planes per operand (3: split fp32, 1: a 16-bit type), F16 selects the fp16 MFMA, S sub-steps
 // per barrier.
-template <int P, bool F16, int S>
+template <int P, bool F16, int S, bool ACCUM>
 __global__ __launch_bounds__(64 * kWaves, 2) void gemm_split_kernel(
     const piece* __restrict__ A, uint64_t Rpa, const piece* __restrict__ B, uint64_t Rpb, uint64_t K8,
     float* __restrict__ C, uint64_t ldc, uint64_t M, uint64_t N, float alpha, float beta,
@@ -241,24 +241,49 @@ __global__ __launch_bounds__(64 * kWaves, 2) void gemm_split_kernel(
     }
 
     // D[m][n] of a 32x32 MFMA: lane holds column n = lane % 32; register r holds row
-    // 8*(r/4) + 4*(lane/32) + r%4.
+    // 8*(r/4) + 4*(lane/32) + r%4.  When C is accumulated into, its old values are fetched for 32 rows
+    // at a time before any of them is overwritten (loads and stores through one pointer would
+    // otherwise alternate, one memory round trip per element).
+    const uint64_t col0 = n0 + wn * (32 * JT) + x;
+    if constexpr (!ACCUM) {
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const uint64_t row = m0 + wm * 64 + 32 * i + 8 * (r >> 2) + 4 * h + (r & 3);
+                if (row >= M) continue;
+                const float rs = row_scale ? row_scale[row] : 1.0f;
+#pragma unroll
+                for (int j = 0; j < JT; ++j) {
+                    const uint64_t col = col0 + 32 * j;
+                    if (col < N) C[row * ldc + col] = alpha * acc[i][j][r] * rs;
+                }
+            }
+        }
+    } else {
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
+        const uint64_t row0 = m0 + wm * 64 + 32 * i + 4 * h;
+        floatx16 prev[JT];
+#pragma unroll
+        for (int j = 0; j < JT; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const uint64_t row = row0 + 8 * (r >> 2) + (r & 3), col = col0 + 32 * j;
+                prev[j][r] = (row < M && col < N) ? C[row * ldc + col] : 0.0f;
+            }
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
-            const uint64_t row = m0 + wm * 64 + 32 * i + 8 * (r >> 2) + 4 * h + (r & 3);
+            const uint64_t row = row0 + 8 * (r >> 2) + (r & 3);
             if (row >= M) continue;
             const float rs = row_scale ? row_scale[row] : 1.0f;
 #pragma unroll
             for (int j = 0; j < JT; ++j) {
-                const uint64_t col = n0 + wn * (32 * JT) + 32 * j + x;
-                if (col >= N) continue;
-                float* c = C + row * ldc + col;
-                float v = alpha * acc[i][j][r];
-                if (beta != 0.0f) v += beta * *c;
-                *c = v * rs;
+                const uint64_t col = col0 + 32 * j;
+                if (col < N) C[row * ldc + col] = (alpha * acc[i][j][r] + beta * prev[j][r]) * rs;
             }
         }
+    }
     }
 }
 
@@ -347,15 +372,18 @@ int gemm_nt_split(const void* A_planes, uint64_t M, const void* B_planes, uint64
     const piece* a = static_cast<const piece*>(A_planes);
     const piece* b = static_cast<const piece*>(B_planes);
     const uint64_t Rpa = padded_rows(M), Rpb = padded_rows(N), K8 = octets(K);
+    // ACCUM (beta != 0) fetches the old C in the epilogue; kept out of the plain kernel
+    void (*kernel)(const piece*, uint64_t, const piece*, uint64_t, uint64_t, float*, uint64_t, uint64_t, uint64_t, float,
+                   float, const float*, uint32_t, uint32_t);
+    const bool accum = beta != 0.0f;
     if (dtype == TRAKHIP_F32)
-        hipLaunchKernelGGL((gemm_split_kernel<3, false, 1>), grid, block, 0, s, a, Rpa, b, Rpb, K8, C, ldc, M, N, alpha,
-                           beta, row_scale, (uint32_t)tiles_n, flags);
+        kernel = accum ? gemm_split_kernel<3, false, 1, true> : gemm_split_kernel<3, false, 1, false>;
     else if (dtype == TRAKHIP_F16)
-        hipLaunchKernelGGL((gemm_split_kernel<1, true, 4>), grid, block, 0, s, a, Rpa, b, Rpb, K8, C, ldc, M, N, alpha,
-                           beta, row_scale, (uint32_t)tiles_n, flags);
+        kernel = accum ? gemm_split_kernel<1, true, 4, true> : gemm_split_kernel<1, true, 4, false>;
     else
-        hipLaunchKernelGGL((gemm_split_kernel<1, false, 4>), grid, block, 0, s, a, Rpa, b, Rpb, K8, C, ldc, M, N, alpha,
-                           beta, row_scale, (uint32_t)tiles_n, flags);
+        kernel = accum ? gemm_split_kernel<1, false, 4, true> : gemm_split_kernel<1, false, 4, false>;
+    hipLaunchKernelGGL(kernel, grid, block, 0, s, a, Rpa, b, Rpb, K8, C, ldc, M, N, alpha, beta, row_scale,
+                       (uint32_t)tiles_n, flags);
     return hipGetLastError() == hipSuccess ? TRAKHIP_OK : TRAKHIP_ERR_LAUNCH;
 }
 
