@@ -345,7 +345,7 @@ def bench_scoring(torch, dev, reps=3):
             best = ms if best is None else min(best, ms)
         return r, best
 
-    from trak_amd.utils import gemm_nt, gemm_nt_split, gemm_tn, gram_split, spd_inverse, split_rows
+    from trak_amd.utils import gemm_nt, gemm_nt16, gemm_nt_split, gemm_tn, gram_split, spd_inverse, split_rows
 
     # the fp32 MFMA instruction (v_mfma_f32_32x32x2_f32): priced against the 157.3 TFLOP/s fp32 peak
     xtx, t_xtx = timed(lambda: gemm_tn(X, X))
@@ -363,11 +363,12 @@ def bench_scoring(torch, dev, reps=3):
     _, s_sc = timed(lambda: gemm_nt_split(split_rows(feats), split_rows(Xt), row_scale=otl))
     split_ms = s_xtx + s_feat + s_sc
     # TRAKer's default stores gradients and features as fp16 (use_half_precision): the same products
-    # from single fp16 planes, one MFMA per k step, exact products
+    # with one MFMA per k step and exact products; X^T X from one fp16 plane (the transposed operand
+    # needs the re-layout), the two row-major products read in place (what BasicScoreComputer runs)
     Xh, invh, fh, Xth = X.half(), inv.half(), feats.half(), Xt.half()
     _, h_xtx = timed(lambda: gram_split(split_rows(Xh, transposed=True)))
-    _, h_feat = timed(lambda: gemm_nt_split(split_rows(Xh), split_rows(invh)))
-    _, h_sc = timed(lambda: gemm_nt_split(split_rows(fh), split_rows(Xth), row_scale=otl))
+    _, h_feat = timed(lambda: gemm_nt16(Xh, invh))
+    _, h_sc = timed(lambda: gemm_nt16(fh, Xth, row_scale=otl))
     del Xh, fh, Xth
     # X^T X is computed on the tiles that touch the lower triangle only (256 x 256 tiles) and mirrored:
     # its flops are counted as computed, not as 2*N*k*k

@@ -165,6 +165,19 @@ int trakhip_gemm_nt_split(const void* A_planes_dev, uint64_t M, const void* B_pl
 int trakhip_gram_split(const void* A_planes_dev, uint64_t N, uint64_t K, int src_dtype, float* C_dev, uint64_t ldc,
                        float alpha, float beta, void* stream);
 
+/* C[M, N] (fp32) = alpha * A[M, K] * B[N, K]^T + beta * C, row i *= row_scale[i], for fp16 or bf16
+ * operands read where they are: no planes, no extra pass.  For the two products of a TRAKer that
+ * stores half precision whose operands are row-major along the contraction: `block @ xtx_inv`
+ * (trak/score_computers.py:176) and `features @ target_grads.t()` (trak/utils.py:131).
+ *   dtype      TRAKHIP_F16 | TRAKHIP_BF16, both operands
+ *   K          a multiple of 64 (TRAKHIP_ERR_SHAPE otherwise; proj_dim is a multiple of 512)
+ *   A_dev, B_dev  16-byte aligned, lda and ldb multiples of 8 elements (TRAKHIP_ERR_ALIGN otherwise)
+ * A caller whose operands do not qualify uses trakhip_split_rows + trakhip_gemm_nt_split; the results
+ * are the same bits (same MFMAs in the same order). */
+int trakhip_gemm_nt16(const void* A_dev, uint64_t lda, const void* B_dev, uint64_t ldb, int dtype, float* C_dev,
+                      uint64_t ldc, uint64_t M, uint64_t N, uint64_t K, float alpha, float beta,
+                      const float* row_scale_dev, void* stream);
+
 /* out[i, j] = cast((acc[i, j] / divisor) * row_factor[i]) for the [N, M] fp32 score sums that
  * trakhip_gemm_nt accumulated over checkpoints (beta = 1): the closing expression of
  * TRAKer.finalize_scores, `(_scores / n) * (_avg_out_to_losses / n)` (trak/traker.py:670-678), with

@@ -130,6 +130,22 @@ def test_store_entry_points_validate_before_touching_the_device():
     assert "page-locked" in _lib.strerror(-11)
 
 
+def test_gemm_nt16_validates_before_touching_the_device():
+    lib = _lib.load()
+    p = ctypes.c_void_p(4096)
+    F16, BF16, F32 = _lib.F16, _lib.BF16, _lib.F32
+    mm = lambda **kw: lib.trakhip_gemm_nt16(
+        kw.get("a", p), kw.get("lda", 64), kw.get("b", p), kw.get("ldb", 64), kw.get("dt", F16), kw.get("c", p),
+        kw.get("ldc", 8), kw.get("M", 8), kw.get("N", 8), kw.get("K", 64), 1.0, 0.0, None, None)
+    assert mm(dt=F32) == -3 and mm(dt=5) == -3
+    assert mm(M=0) == 0 and mm(N=0, dt=BF16) == 0
+    assert mm(K=0) == -2 and mm(K=32) == -2 and mm(K=100, lda=104, ldb=104) == -2     # K % 64
+    assert mm(lda=56) == -2 and mm(ldb=63) == -2 and mm(ldc=7) == -2
+    assert mm(a=None) == -5 and mm(b=None) == -5 and mm(c=None) == -5
+    assert mm(a=ctypes.c_void_p(4104)) == -7 and mm(b=ctypes.c_void_p(4098)) == -7     # 16-byte rows
+    assert mm(lda=68) == -7 and mm(ldb=100) == -7 and mm(c=ctypes.c_void_p(4098)) == -7
+
+
 def test_split_gemm_entry_points_validate_before_touching_the_device():
     lib = _lib.load()
     p = ctypes.c_void_p(4096)

@@ -9,7 +9,7 @@ import torch
 
 from oracle import score_oracle as so
 from trak_amd import BasicScoreComputer, get_matrix_mult
-from trak_amd.utils import gemm_nt, gemm_nt_split, gemm_tn, gram_split, spd_inverse, split_rows
+from trak_amd.utils import gemm_nt, gemm_nt16, gemm_nt_split, gemm_tn, gram_split, matmul_nt, spd_inverse, split_rows
 
 pytestmark = pytest.mark.gpu
 
@@ -195,6 +195,53 @@ def test_gemm_nt_split_sixteen_bit(gpu, dtype, M, N, K):
     assert torch.equal(g, g.T) and rel_max(g.cpu().numpy(), a.double().numpy() @ a.double().numpy().T) < gemm_tol(K)
     with pytest.raises(RuntimeError):
         gemm_nt_split(sa, split_rows(b.float().to(gpu)))        # operands of different source types
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("M,N,K", [(1, 1, 64), (130, 70, 128), (256, 512, 64), (1000, 513, 256), (300, 700, 4096), (257, 255, 1088)])
+def test_gemm_nt16_reads_operands_in_place(gpu, dtype, M, N, K):
+    """The in-place 16-bit product issues the same MFMAs in the same order as the one-plane product,
+    so the two agree bit for bit; ragged tiles, accumulation, row scale, operands that are column
+    slices of wider buffers."""
+    gen = torch.Generator(device="cpu").manual_seed(M + N * 3 + K)
+    a, b = torch.randn(M, K, generator=gen).to(dtype), torch.randn(N, K, generator=gen).to(dtype)
+    want = a.double().numpy() @ b.double().numpy().T
+    ag, bg = a.to(gpu), b.to(gpu)
+    got = gemm_nt16(ag, bg)
+    assert got.dtype == torch.float32 and rel_max(got.cpu().numpy(), want) < gemm_tol(K)
+    assert torch.equal(got, gemm_nt_split(split_rows(ag), split_rows(bg)))
+    assert torch.equal(got, matmul_nt(ag, bg))
+    rs = torch.rand(M, generator=gen)
+    c0 = torch.randn(M, N, generator=gen)
+    got = gemm_nt16(ag, bg, out=c0.clone().to(gpu), alpha=2.0, beta=0.5, row_scale=rs.to(gpu))
+    assert rel_max(got.cpu().numpy(), (2.0 * want + 0.5 * c0.double().numpy()) * rs.double().numpy()[:, None]) < gemm_tol(K)
+    # slices of wider buffers: pitch K + 24, first column 8 (rows stay 16-byte aligned)
+    wa = torch.zeros(M, K + 24, dtype=dtype, device=gpu)
+    wb = torch.zeros(N, K + 24, dtype=dtype, device=gpu)
+    wa[:, 8:8 + K], wb[:, 8:8 + K] = ag, bg
+    wide = torch.full((M, N + 3), -1.0, device=gpu)
+    gemm_nt16(wa[:, 8:8 + K], wb[:, 8:8 + K], out=wide[:, :N])
+    assert torch.equal(wide[:, :N], gemm_nt16(ag, bg)) and bool((wide[:, N:] == -1.0).all())
+
+
+def test_gemm_nt16_refuses_what_it_cannot_read_in_place(gpu):
+    a = torch.randn(64, 128, device=gpu).half()
+    b = torch.randn(32, 128, device=gpu).half()
+    with pytest.raises(RuntimeError):
+        gemm_nt16(a[:, :100], b[:, :100])                    # K not a multiple of 64
+    with pytest.raises(RuntimeError):
+        gemm_nt16(a[:, 4:68], b[:, 4:68])                    # rows start 8 bytes off
+    with pytest.raises(RuntimeError):
+        gemm_nt16(a, b.bfloat16())                           # operands of different types
+    with pytest.raises(RuntimeError):
+        gemm_nt16(a.float(), b.float())
+    # matmul_nt takes all of them (through planes)
+    want = a[:, :100].double() @ b[:, :100].double().T
+    assert rel_max(matmul_nt(a[:, :100], b[:, :100]).cpu().numpy(), want.cpu().numpy()) < gemm_tol(100)
+    want = a[:, 4:68].double() @ b[:, 4:68].double().T
+    assert rel_max(matmul_nt(a[:, 4:68], b[:, 4:68]).cpu().numpy(), want.cpu().numpy()) < gemm_tol(64)
+    want = a.double() @ b.bfloat16().double().T
+    assert rel_max(matmul_nt(a, b.bfloat16()).cpu().numpy(), want.cpu().numpy()) < gemm_tol(128)
 
 
 @pytest.mark.parametrize("M,N,K", [(1, 1, 1), (130, 70, 33), (256, 512, 64), (1000, 513, 257), (64, 2048, 4096), (129, 257, 8200)])

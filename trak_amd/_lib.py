@@ -66,6 +66,8 @@ def load():
     lib.trakhip_gemm_nt_split.restype = i32
     lib.trakhip_gram_split.argtypes = [vp, u64, u64, i32, vp, u64, f32, f32, vp]
     lib.trakhip_gram_split.restype = i32
+    lib.trakhip_gemm_nt16.argtypes = [vp, u64, vp, u64, i32, vp, u64, u64, u64, u64, f32, f32, vp, vp]
+    lib.trakhip_gemm_nt16.restype = i32
     lib.trakhip_spd_inverse_workspace.argtypes = [u64]
     lib.trakhip_spd_inverse_workspace.restype = sz
     lib.trakhip_spd_inverse.argtypes = [vp, u64, f32, vp, u64, u64, i32, vp, vp, vp, sz, vp]

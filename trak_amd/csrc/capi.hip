@@ -112,6 +112,13 @@ int trakhip_gram_split(const void* A_planes_dev, uint64_t N, uint64_t K, int dty
     return trakhip::gram_split(A_planes_dev, N, K, dtype, C_dev, ldc, alpha, beta, static_cast<hipStream_t>(stream));
 }
 
+int trakhip_gemm_nt16(const void* A_dev, uint64_t lda, const void* B_dev, uint64_t ldb, int dtype, float* C_dev,
+                      uint64_t ldc, uint64_t M, uint64_t N, uint64_t K, float alpha, float beta,
+                      const float* row_scale_dev, void* stream) {
+    return trakhip::gemm_nt16(A_dev, lda, B_dev, ldb, dtype, C_dev, ldc, M, N, K, alpha, beta, row_scale_dev,
+                              static_cast<hipStream_t>(stream));
+}
+
 size_t trakhip_spd_inverse_workspace(uint64_t n) { return trakhip::spd_inverse_workspace_bytes(n); }
 
 int trakhip_spd_inverse(const float* A_dev, uint64_t lda, float lambda, float* inv_dev, uint64_t ldi,

@@ -135,6 +135,56 @@ __device__ __forceinline__ floatx16 mfma16(const piece& a, const piece& b, float
                                                        c, 0, 0, 0);
 }
 
+// Epilogue of a wave's 64 x (32 JT) part of C.  D[m][n] of a 32x32 MFMA: lane holds column
+// n = lane % 32; register r holds row 8*(r/4) + 4*(lane/32) + r%4.  When C is accumulated into (ACCUM),
+// its old values are fetched for 32 rows at a time before any of them is overwritten (loads and stores
+// through one pointer would otherwise alternate, one memory round trip per element).
+template <bool ACCUM, int JT>
+__device__ __forceinline__ void store_c(const floatx16 (&acc)[2][JT], float* __restrict__ C, uint64_t ldc, uint64_t M,
+                                        uint64_t N, uint64_t row_base, uint64_t col0, int h, float alpha, float beta,
+                                        const float* __restrict__ row_scale) {
+    if constexpr (!ACCUM) {
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const uint64_t row = row_base + 32 * i + 8 * (r >> 2) + 4 * h + (r & 3);
+                if (row >= M) continue;
+                const float rs = row_scale ? row_scale[row] : 1.0f;
+#pragma unroll
+                for (int j = 0; j < JT; ++j) {
+                    const uint64_t col = col0 + 32 * j;
+                    if (col < N) C[row * ldc + col] = alpha * acc[i][j][r] * rs;
+                }
+            }
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            const uint64_t row0 = row_base + 32 * i + 4 * h;
+            floatx16 prev[JT];
+#pragma unroll
+            for (int j = 0; j < JT; ++j)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const uint64_t row = row0 + 8 * (r >> 2) + (r & 3), col = col0 + 32 * j;
+                    prev[j][r] = (row < M && col < N) ? C[row * ldc + col] : 0.0f;
+                }
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const uint64_t row = row0 + 8 * (r >> 2) + (r & 3);
+                if (row >= M) continue;
+                const float rs = row_scale ? row_scale[row] : 1.0f;
+#pragma unroll
+                for (int j = 0; j < JT; ++j) {
+                    const uint64_t col = col0 + 32 * j;
+                    if (col < N) C[row * ldc + col] = (alpha * acc[i][j][r] + beta * prev[j][r]) * rs;
+                }
+            }
+        }
+    }
+}
+
 // A step of a tile is S sub-steps (two octets = one MFMA depth each); sub-step u holds
 // [A: plane][half][256 rows] followed by [B: plane][half][256 rows].  The pieces are moved in chunks
 // of 64 consecutive ones by the load unit straight into LDS (global_load_lds_dwordx4): the 64
@@ -240,51 +290,94 @@ __global__ __launch_bounds__(64 * kWaves, 2) void gemm_split_kernel(
         __syncthreads();
     }
 
-    // D[m][n] of a 32x32 MFMA: lane holds column n = lane % 32; register r holds row
-    // 8*(r/4) + 4*(lane/32) + r%4.  When C is accumulated into, its old values are fetched for 32 rows
-    // at a time before any of them is overwritten (loads and stores through one pointer would
-    // otherwise alternate, one memory round trip per element).
-    const uint64_t col0 = n0 + wn * (32 * JT) + x;
-    if constexpr (!ACCUM) {
+    store_c<ACCUM, JT>(acc, C, ldc, M, N, m0 + wm * 64, n0 + wn * (32 * JT) + x, h, alpha, beta, row_scale);
+}
+
+// ---- 16-bit operands read in place -----------------------------------------------------------
+//
+// Row-major fp16 / bf16 operands A[M, K], B[N, K] with K a multiple of 64 and 16-byte aligned rows need
+// no planes.  A step is 64 values of k = one 128-byte line of every row: chunk c of a step is the
+// lines of rows 8c .. 8c+7 of [256 rows of A | 256 rows of B], lane l of the moving wave fetches
+// the 16-byte piece (row 8c + l/8, octet (l % 8) ^ (l / 8)) into slot l of the chunk, i.e. LDS
+// holds each row's eight octets permuted by XOR with (row % 8).  A wave's load instruction reads eight
+// full lines, and the eight lanes of a ds_read_b128 group (eight consecutive rows, one octet) hit eight
+// different 16-byte columns: linear global reads, conflict-free LDS reads, and the same MFMA loop as
+// the one-plane kernel.  Rows past M or N are fetched from the last row (their results are not stored).
+template <bool F16, bool ACCUM>
+__global__ __launch_bounds__(64 * kWaves, 2) void gemm_nt16_kernel(
+    const piece* __restrict__ A, uint64_t lda8, const piece* __restrict__ B, uint64_t ldb8, uint64_t steps,
+    float* __restrict__ C, uint64_t ldc, uint64_t M, uint64_t N, float alpha, float beta,
+    const float* __restrict__ row_scale, uint32_t tiles_n) {
+    constexpr int JT = BN / kWavesN / 32;
+    constexpr int kBufPieces = 8 * (BM + BN);  // 64 KB
+    constexpr int kMoves = (BM + BN) / 8 / kWaves, kMovesA = BM / 8 / kWaves;  // chunks per wave and step
+    __shared__ piece lds[2][kBufPieces];
+
+    const uint32_t tile_m = blockIdx.x / tiles_n, tile_n = blockIdx.x % tiles_n;
+    const uint64_t m0 = (uint64_t)tile_m * BM, n0 = (uint64_t)tile_n * BN;
+    const int tid = threadIdx.x;
+    const int wave = tid >> 6, lane = tid & 63;
+    const int wm = wave / kWavesN, wn = wave % kWavesN;
+    const int x = lane & 31, h = lane >> 5;
+
+    // this lane's piece of step 0 in each chunk that its wave moves (chunks wave, wave + 8, ...)
+    const piece* src[kMoves];
+    {
+        const int sub = lane >> 3, oct = (lane & 7) ^ sub;
 #pragma unroll
-        for (int i = 0; i < 2; ++i) {
-#pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const uint64_t row = m0 + wm * 64 + 32 * i + 8 * (r >> 2) + 4 * h + (r & 3);
-                if (row >= M) continue;
-                const float rs = row_scale ? row_scale[row] : 1.0f;
-#pragma unroll
-                for (int j = 0; j < JT; ++j) {
-                    const uint64_t col = col0 + 32 * j;
-                    if (col < N) C[row * ldc + col] = alpha * acc[i][j][r] * rs;
-                }
+        for (int i = 0; i < kMoves; ++i) {
+            const int row = 8 * (wave + kWaves * (i % kMovesA)) + sub;
+            if (i < kMovesA) {
+                const uint64_t g = m0 + row < M ? m0 + row : M - 1;
+                src[i] = A + g * lda8 + oct;
+            } else {
+                const uint64_t g = n0 + row < N ? n0 + row : N - 1;
+                src[i] = B + g * ldb8 + oct;
             }
         }
-    } else {
+    }
+    auto dma = [&](uint64_t s, piece* buf) {
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
-        const uint64_t row0 = m0 + wm * 64 + 32 * i + 4 * h;
-        floatx16 prev[JT];
+        for (int i = 0; i < kMoves; ++i) {
+            const int c = (i < kMovesA ? 0 : BM / 8) + wave + kWaves * (i % kMovesA);  // wave-uniform
+            __builtin_amdgcn_global_load_lds((const void __attribute__((address_space(1)))*)(src[i] + 8 * s),
+                                             (void __attribute__((address_space(3)))*)(buf + 64 * c), 16, 0, 0);
+        }
+    };
+
+    floatx16 acc[2][JT];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
 #pragma unroll
         for (int j = 0; j < JT; ++j)
 #pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const uint64_t row = row0 + 8 * (r >> 2) + (r & 3), col = col0 + 32 * j;
-                prev[j][r] = (row < M && col < N) ? C[row * ldc + col] : 0.0f;
-            }
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+    dma(0, lds[0]);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+
+    const int a_row = (wm * 64 + x) * 8, b_row = (BM + wn * (32 * JT) + x) * 8;  // first piece of the lane's rows
+    for (uint64_t s = 0; s < steps; ++s) {
+        const int cur = (int)(s & 1);
+        if (s + 1 < steps) dma(s + 1, lds[cur ^ 1]);
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-            const uint64_t row = row0 + 8 * (r >> 2) + (r & 3);
-            if (row >= M) continue;
-            const float rs = row_scale ? row_scale[row] : 1.0f;
+        for (int u = 0; u < 4; ++u) {
+            const piece* l = lds[cur] + ((2 * u + h) ^ (x & 7));
+            piece fa[2];
+#pragma unroll
+            for (int i = 0; i < 2; ++i) fa[i] = l[a_row + 256 * i];
 #pragma unroll
             for (int j = 0; j < JT; ++j) {
-                const uint64_t col = col0 + 32 * j;
-                if (col < N) C[row * ldc + col] = (alpha * acc[i][j][r] + beta * prev[j][r]) * rs;
+                const piece fb = l[b_row + 256 * j];
+#pragma unroll
+                for (int i = 0; i < 2; ++i) acc[i][j] = mfma16<F16>(fa[i], fb, acc[i][j]);
             }
         }
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
     }
-    }
+    store_c<ACCUM, JT>(acc, C, ldc, M, N, m0 + wm * 64, n0 + wn * (32 * JT) + x, h, alpha, beta, row_scale);
 }
 
 // C[i][j] = C[j][i] for j > i: completes a symmetric matrix whose lower triangle was computed.
@@ -384,6 +477,30 @@ int gemm_nt_split(const void* A_planes, uint64_t M, const void* B_planes, uint64
         kernel = accum ? gemm_split_kernel<1, false, 4, true> : gemm_split_kernel<1, false, 4, false>;
     hipLaunchKernelGGL(kernel, grid, block, 0, s, a, Rpa, b, Rpb, K8, C, ldc, M, N, alpha, beta, row_scale,
                        (uint32_t)tiles_n, flags);
+    return hipGetLastError() == hipSuccess ? TRAKHIP_OK : TRAKHIP_ERR_LAUNCH;
+}
+
+int gemm_nt16(const void* A, uint64_t lda, const void* B, uint64_t ldb, int dtype, float* C, uint64_t ldc, uint64_t M,
+              uint64_t N, uint64_t K, float alpha, float beta, const float* row_scale, hipStream_t s) {
+    if (dtype != TRAKHIP_F16 && dtype != TRAKHIP_BF16) return TRAKHIP_ERR_DTYPE;
+    if (M == 0 || N == 0) return TRAKHIP_OK;
+    if (K == 0 || K % 64 || lda < K || ldb < K || ldc < N) return TRAKHIP_ERR_SHAPE;
+    if (!A || !B || !C) return TRAKHIP_ERR_NULL;
+    if ((reinterpret_cast<uintptr_t>(A) % 16) || (reinterpret_cast<uintptr_t>(B) % 16) || (lda % 8) || (ldb % 8) ||
+        (reinterpret_cast<uintptr_t>(C) % 4))
+        return TRAKHIP_ERR_ALIGN;
+    const uint64_t tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
+    if (tiles_m * tiles_n > 0x7FFFFFFFull) return TRAKHIP_ERR_SHAPE;
+    void (*kernel)(const piece*, uint64_t, const piece*, uint64_t, uint64_t, float*, uint64_t, uint64_t, uint64_t, float,
+                   float, const float*, uint32_t);
+    const bool accum = beta != 0.0f;
+    if (dtype == TRAKHIP_F16)
+        kernel = accum ? gemm_nt16_kernel<true, true> : gemm_nt16_kernel<true, false>;
+    else
+        kernel = accum ? gemm_nt16_kernel<false, true> : gemm_nt16_kernel<false, false>;
+    hipLaunchKernelGGL(kernel, dim3((uint32_t)(tiles_m * tiles_n)), dim3(64 * kWaves), 0, s,
+                       static_cast<const piece*>(A), lda / 8, static_cast<const piece*>(B), ldb / 8, K / 64, C, ldc, M, N,
+                       alpha, beta, row_scale, (uint32_t)tiles_n);
     return hipGetLastError() == hipSuccess ? TRAKHIP_OK : TRAKHIP_ERR_LAUNCH;
 }
 

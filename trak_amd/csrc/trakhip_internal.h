@@ -57,6 +57,8 @@ int gemm_nt_split(const void* A_planes, uint64_t M, const void* B_planes, uint64
                   uint64_t ldc, float alpha, float beta, const float* row_scale, hipStream_t s, uint32_t flags = 0);
 int gram_split(const void* A_planes, uint64_t N, uint64_t K, int dtype, float* C, uint64_t ldc, float alpha, float beta,
                hipStream_t s);
+int gemm_nt16(const void* A, uint64_t lda, const void* B, uint64_t ldb, int dtype, float* C, uint64_t ldc, uint64_t M,
+              uint64_t N, uint64_t K, float alpha, float beta, const float* row_scale, hipStream_t s);
 size_t spd_inverse_workspace_bytes(uint64_t n);
 int spd_inverse(const float* A, uint64_t lda, float lambda, float* inv, uint64_t ldi, uint64_t n,
                 int normalize, float* mean_abs, int32_t* status, void* ws, size_t ws_bytes, hipStream_t s);

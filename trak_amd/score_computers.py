@@ -11,7 +11,18 @@ from abc import ABC, abstractmethod
 import torch
 from torch import Tensor
 
-from .utils import gemm_nt, gemm_nt_split, gemm_tn, gram_split, scores_finalize, spd_inverse, split_pair, split_rows
+from .utils import (
+    _nt16_ok,
+    gemm_nt,
+    gemm_nt16,
+    gemm_nt_split,
+    gemm_tn,
+    gram_split,
+    matmul_nt,
+    scores_finalize,
+    spd_inverse,
+    split_rows,
+)
 
 ch = torch
 
@@ -99,14 +110,19 @@ class BasicScoreComputer(AbstractScoreComputer):
         result = ch.empty(grads.shape[0], xtx_inv.shape[1], dtype=ch.float32, device=self._dev)
         # 16-bit gradients meet the inverse cast to their type (as in the reference) as single planes
         half = grads.dtype == xtx_inv.dtype and grads.dtype in (ch.float16, ch.bfloat16)
-        inv_split = split_rows(xtx_inv if half else xtx_inv.float()) if self.gemm == "split" else None
+        inv_split = None  # planes of the inverse, made when the first block needs them
         start = 0
         for block in self._blocks(grads):
             end = start + block.shape[0]
             # the inverse is symmetric, so block @ inv == block @ inv^T
-            if inv_split is not None:
+            if self.gemm == "split":
                 block = block.to(self._dev)
-                gemm_nt_split(split_rows(block if half else block.float()), inv_split, out=result[start:end])
+                if half and _nt16_ok(block, xtx_inv):
+                    gemm_nt16(block, xtx_inv, out=result[start:end])
+                else:
+                    if inv_split is None:
+                        inv_split = split_rows(xtx_inv if half else xtx_inv.float())
+                    gemm_nt_split(split_rows(block if half else block.float()), inv_split, out=result[start:end])
             else:
                 gemm_nt(block.to(self._dev), xtx_inv, out=result[start:end])
             start = end
@@ -143,7 +159,7 @@ class BasicScoreComputer(AbstractScoreComputer):
 
     def _matmul_nt(self, a, b, out=None, alpha=1.0, beta=0.0, row_scale=None):
         if self.gemm == "split":
-            return gemm_nt_split(*split_pair(a, b), out=out, alpha=alpha, beta=beta, row_scale=row_scale)
+            return matmul_nt(a, b, out=out, alpha=alpha, beta=beta, row_scale=row_scale)
         return gemm_nt(a, b, out=out, alpha=alpha, beta=beta, row_scale=row_scale)
 
 

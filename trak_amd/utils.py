@@ -230,6 +230,58 @@ def gemm_nt_split(a, b, out=None, alpha=1.0, beta=0.0, row_scale=None):
     return out
 
 
+def _nt16_ok(a, b):
+    """Whether `gemm_nt16` can read these operands where they are."""
+    if a.dtype != b.dtype or a.dtype not in (torch.float16, torch.bfloat16):
+        return False
+    if a.dim() != 2 or b.dim() != 2 or not a.is_cuda or a.device != b.device:
+        return False
+    if a.shape[1] != b.shape[1] or a.shape[1] == 0 or a.shape[1] % 64:
+        return False
+    for t in (a, b):
+        if t.stride(1) != 1 or t.data_ptr() % 16 or (t.shape[0] > 1 and (t.stride(0) % 8 or t.stride(0) < t.shape[1])):
+            return False
+    return True
+
+
+def gemm_nt16(a, b, out=None, alpha=1.0, beta=0.0, row_scale=None):
+    """out[M, N] (fp32) = alpha * a @ b.T + beta * out (rows optionally scaled) for fp16 or bf16 CUDA
+    matrices a [M, K], b [N, K] read in place: K a multiple of 64, rows 16-byte aligned (see
+    `matmul_nt` for the general case).  Exact products, fp32 accumulation."""
+    if not _nt16_ok(a, b):
+        raise RuntimeError("gemm_nt16 needs two fp16 or two bf16 CUDA matrices with K % 64 == 0 and 16-byte aligned rows")
+    M, N, K = a.shape[0], b.shape[0], a.shape[1]
+    if out is None:
+        out = torch.empty((M, N), dtype=torch.float32, device=a.device)
+        beta = 0.0
+    if out.dtype != torch.float32 or tuple(out.shape) != (M, N) or (N > 1 and out.stride(1) != 1) or out.device != a.device:
+        raise RuntimeError("out must be an fp32 [M, N] tensor with unit column stride on the operands' device")
+    rs = None
+    if row_scale is not None:
+        rs = row_scale.to(device=a.device, dtype=torch.float32).contiguous().reshape(-1)
+        if rs.numel() != M:
+            raise RuntimeError("row_scale must have M elements")
+    lib = _lib.load()
+    with torch.cuda.device(a.device):
+        stream = torch.cuda.current_stream(a.device).cuda_stream
+        code = lib.trakhip_gemm_nt16(
+            ctypes.c_void_p(a.data_ptr()), _ld(a), ctypes.c_void_p(b.data_ptr()), _ld(b), _STORE_DTYPES[a.dtype],
+            ctypes.c_void_p(out.data_ptr()), _ld(out), M, N, K, float(alpha), float(beta),
+            ctypes.c_void_p(rs.data_ptr()) if rs is not None else None, ctypes.c_void_p(stream),
+        )
+    _lib.check(code)
+    return out
+
+
+def matmul_nt(a, b, out=None, alpha=1.0, beta=0.0, row_scale=None):
+    """alpha * a @ b.T + beta * out with fp32 accuracy on the 16-bit matrix cores, whatever the operand
+    types: two fp16 or two bf16 matrices that qualify are multiplied where they are (`gemm_nt16`),
+    other 16-bit pairs as single planes, anything else from fp32 splits (`gemm_nt_split`)."""
+    if _nt16_ok(a, b):
+        return gemm_nt16(a, b, out=out, alpha=alpha, beta=beta, row_scale=row_scale)
+    return gemm_nt_split(*split_pair(a, b), out=out, alpha=alpha, beta=beta, row_scale=row_scale)
+
+
 def gram_split(a, out=None, alpha=1.0, beta=0.0):
     """out[N, N] = alpha * A @ A.T + beta * out for a SplitOperand A [N, K]: the lower-triangle tiles
     are computed and mirrored, so the result is exactly symmetric at about half the cost of
@@ -349,5 +401,5 @@ def get_matrix_mult(features, target_grads, target_dtype=None, batch_size=8096, 
         target_dtype = features.dtype
     if features.device.type == "cpu":
         return (features @ target_grads.t()).clone().to(target_dtype)
-    out = gemm_nt_split(*split_pair(features, target_grads.to(features.device)))
+    out = matmul_nt(features, target_grads.to(features.device))
     return out.to(target_dtype)
