@@ -298,10 +298,12 @@ __global__ __launch_bounds__(64 * kWaves, 2) void gemm_split_kernel(
 // Row-major fp16 / bf16 operands A[M, K], B[N, K] with K a multiple of 64 and 16-byte aligned rows need
 // no planes.  A step is 64 values of k = one 128-byte line of every row: chunk c of a step is the
 // lines of rows 8c .. 8c+7 of [256 rows of A | 256 rows of B], lane l of the moving wave fetches
-// the 16-byte piece (row 8c + l/8, octet (l % 8) ^ (l / 8)) into slot l of the chunk, i.e. LDS
-// holds each row's eight octets permuted by XOR with (row % 8).  A wave's load instruction reads eight
-// full lines, and the eight lanes of a ds_read_b128 group (eight consecutive rows, one octet) hit eight
-// different 16-byte columns: linear global reads, conflict-free LDS reads, and the same MFMA loop as
+// the 16-byte piece of row r = 8c + l/8 that belongs in slot l % 8, i.e. LDS holds each row's eight
+// octets permuted: octet o sits in slot o ^ ((r / 2) % 8).  A wave's load instruction reads eight full
+// lines; LDS serves a ds_read_b128 sixteen lanes at a time from 64 banks (256 bytes), and the sixteen
+// lanes of a group (sixteen consecutive rows, one octet) land on sixteen different 16-byte columns
+// of those 256 bytes - rows of equal parity share a 128-byte half and differ in r / 2.  Linear global
+// reads, conflict-free LDS reads (XOR with r % 8 instead leaves a two-way conflict), and the same MFMA loop as
 // the one-plane kernel.  Rows past M or N are fetched from the last row (their results are not stored).
 template <bool F16, bool ACCUM>
 __global__ __launch_bounds__(64 * kWaves, 2) void gemm_nt16_kernel(
@@ -323,7 +325,8 @@ __global__ __launch_bounds__(64 * kWaves, 2) void gemm_nt16_kernel(
     // this lane's piece of step 0 in each chunk that its wave moves (chunks wave, wave + 8, ...)
     const piece* src[kMoves];
     {
-        const int sub = lane >> 3, oct = (lane & 7) ^ sub;
+        // rows 8c + sub of chunk c = wave + 8 i': (row >> 1) % 8 = 4 (wave % 2) + sub / 2
+        const int sub = lane >> 3, oct = (lane & 7) ^ ((4 * (wave & 1) + (sub >> 1)) & 7);
 #pragma unroll
         for (int i = 0; i < kMoves; ++i) {
             const int row = 8 * (wave + kWaves * (i % kMovesA)) + sub;
@@ -363,7 +366,7 @@ __global__ __launch_bounds__(64 * kWaves, 2) void gemm_nt16_kernel(
         if (s + 1 < steps) dma(s + 1, lds[cur ^ 1]);
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
-            const piece* l = lds[cur] + ((2 * u + h) ^ (x & 7));
+            const piece* l = lds[cur] + ((2 * u + h) ^ ((x >> 1) & 7));
             piece fa[2];
 #pragma unroll
             for (int i = 0; i < 2; ++i) fa[i] = l[a_row + 256 * i];
