@@ -1,5 +1,4 @@
 """Host-side mirror of the reference's projector helpers (no GPU needed)."""
-import numpy as np
 import pytest
 import torch
 
