@@ -23,7 +23,6 @@
 namespace {
 
 constexpr int NB = 128;
-constexpr int kLd = NB + 1;
 constexpr int kSumBlocks = 1024;
 
 __global__ __launch_bounds__(256) void spd_init_kernel(const float* __restrict__ A, uint64_t lda, float lambda,
@@ -44,126 +43,232 @@ __global__ __launch_bounds__(256) void spd_init_kernel(const float* __restrict__
     Li[idx] = 0.0f;
 }
 
-// One workgroup of 1024 threads: Cholesky of the 128x128 diagonal block at W (lower triangle
-// used), L block to Lout (upper part zero), its inverse to Linv_out.
+// One workgroup of four waves: Cholesky of the 128x128 diagonal block at W (lower triangle used),
+// L block to Lout (upper part zero), its inverse to Linv_out.
 //
-// Both matrices live in registers, 4 x 4 elements per thread each, cyclically distributed so that
-// every thread stays busy as the active part shrinks (four waves per SIMD hide the issue latency of
-// this strictly sequential algorithm).  One loop of 128 steps, one barrier per step, does both
-// jobs: step k broadcasts the unscaled column k of the trailing matrix A (l_k = raw / sqrt(d),
-// d = A[k][k]) and the unscaled row k of B (B starts as I; x_k = B[k, :] / L[k][k] is row k of
-// L^-1) through LDS, then every thread applies
-//     A[r][c] -= raw[r] raw[c] / d                         (right-looking Cholesky)
-//     B[r][c] -= raw[r] Braw[c] / d    for r > k           (forward substitution on all columns)
-// from registers.  Thread t holds A rows t % 32 + 32 i, columns t / 32 + 32 j, and the transpose of
-// that for B, so the threads that publish column k of A and row k of B are the same half of ONE
-// wave.  A updates are not masked: entries of rows or columns <= k are never read again once step
-// k is over.  Rows <= k of B are finished rows of L^-1 and are kept.
-constexpr int kDiagGrid = 32;              // threads per side
-constexpr int kDiagTile = NB / kDiagGrid;  // 4 elements per side per thread
+// The block is handled as 4 x 4 sub-blocks of 32 in LDS (row pitch 129 floats: conflict free by rows
+// and by columns).  For sub-block column p:
+//   - ONE WAVE factors the 32 x 32 diagonal sub-block and inverts the factor, registers only, values of
+//     other lanes through v_readlane: no barriers and no LDS round trips inside this strictly
+//     sequential part (see factor_sub_block);
+//   - the sub-blocks below become L = A X^T and the trailing sub-blocks get A -= L L^T, both on
+//     v_mfma_f32_32x32x2_f32, one 32 x 32 tile per wave at a time.
+// The off-diagonal sub-blocks of the inverse follow by halving, [A 0; B C]^-1 = [A^-1 0; -C^-1 B A^-1 C^-1],
+// two levels (32 -> 64 -> 128), again on the MFMA.  About 1200 vector instructions per sub-block on one
+// wave and a dozen workgroup barriers, against 128 barriers (and an LDS round trip
+// each) for a column-at-a-time loop over the whole block.
+constexpr int kSub = 32;
+constexpr int kPitch = NB + 1;
+constexpr int kTPitch = 2 * kSub + 1;
 
-__global__ __launch_bounds__(1024) void spd_diag_kernel(const float* __restrict__ W, uint64_t ldw,
-                                                        float* __restrict__ Lout, float* __restrict__ Linv_out,
-                                                        uint64_t ldl, int32_t block_index,
-                                                        int32_t* __restrict__ status) {
-    constexpr int G = kDiagGrid, T = kDiagTile;
-    __shared__ float Ls[NB * kLd];   // the finished factor, column k valid after step k
-    // column k of A and row k of B, unscaled; entry x = t + 32 i is kept at slot 4 t + i, so the four
-    // values a thread needs are one 16-byte LDS access (two buffers, so the steps can overlap safely)
-    __shared__ __attribute__((aligned(16))) float vec[2][NB];
-    __shared__ __attribute__((aligned(16))) float bvec[2][NB];
-    __shared__ float pivot[2];
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+
+__device__ __forceinline__ float lane_value(float v, int lane) {
+    return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), lane));
+}
+
+// Row 8*(r/4) + 4*(lane/32) + r%4 of a 32x32 MFMA result is in register r; its column is lane % 32.
+__device__ __forceinline__ int mfma_row(int r, int h) { return 8 * (r >> 2) + 4 * h + (r & 3); }
+
+// Factor and invert the 32 x 32 sub-block at (base, base) of As with one wave.  Lane x of the lower
+// half-wave holds row x of A in v[0..31]; lane 32 + c of the upper half holds column c of X, which
+// starts as the identity (v[j] = X[j][c]).  Step k scales v[k] by s = 1 / sqrt(A[k][k]) in every lane
+// (lower half: column k of L; upper half: the finished row k of X = L^-1), then for j > k every lane
+// does v[j] -= v[k] L[j][k] with L[j][k] read from lane j: the trailing update of A in the lower half,
+// forward elimination of the identity in the upper half - one lane read and one multiply-add per (k, j).
+__device__ __forceinline__ void factor_sub_block(float* As, float* Xs, int base, int lane, int32_t first_index,
+                                                 int32_t* status) {
+    const int x = lane & 31;
+    const bool lower = lane < kSub;
+    float v[kSub];
+    int32_t bad = 0;  // 1 + index of the first pivot that is not positive
+    // every lane reads its row (the upper half-wave the same one again): 32 loads in flight, no
+    // branch per element around them
+    float row[kSub];
+#pragma unroll
+    for (int j = 0; j < kSub; ++j) row[j] = As[(base + x) * kPitch + base + j];
+#pragma unroll
+    for (int j = 0; j < kSub; ++j) {
+        asm volatile("" : "+v"(row[j]));
+        v[j] = lower ? row[j] : (j == x ? 1.0f : 0.0f);
+    }
+#pragma unroll
+    for (int k = 0; k < kSub; ++k) {
+        float d = lane_value(v[k], k);
+        // a pivot that is not positive is recorded and replaced, without a branch: the 32 steps stay one
+        // straight line of code
+        const bool ok = d > 0.0f;
+        bad = (ok || bad != 0) ? bad : 1 + first_index + k;
+        d = ok ? d : 1.0f;
+        float s = __builtin_amdgcn_rsqf(d);
+        s = s * __builtin_fmaf(-0.5f * d * s, s, 1.5f);  // one Newton step on the 1 ulp hardware value
+        const float t = v[k] * s;
+        v[k] = t;
+        // All lane reads first, then the multiply-adds: a scalar register written by a vector
+        // instruction cannot be read by the next one.  The empty volatile statement and the fences pin
+        // each step between its neighbours (otherwise lane reads of later steps drift up here and
+        // their scalar results spill).
+        __builtin_amdgcn_sched_barrier(0);
+        float lj[kSub];
+#pragma unroll
+        for (int j = k + 1; j < kSub; ++j) lj[j] = lane_value(t, j);
+#pragma unroll
+        for (int j = k + 1; j < kSub; ++j) v[j] = __builtin_fmaf(-t, lj[j], v[j]);
+        if (k + 1 < kSub) asm volatile("" : "+v"(v[k + 1]));
+        __builtin_amdgcn_sched_barrier(0);
+    }
+    if (bad != 0 && lane == 0 && status && *status == 0) *status = bad;
+    // lower half: row x of L (zero above the diagonal); upper half: X[j][x], zero above the diagonal by
+    // construction.  One store per j for the whole wave.
+    float* dst = lower ? As + (base + x) * kPitch + base : Xs + base * kPitch + base + x;
+    const int step = lower ? 1 : kPitch;
+#pragma unroll
+    for (int j = 0; j < kSub; ++j) dst[j * step] = (lower && j > x) ? 0.0f : v[j];
+}
+
+// acc += sign * A[32 x K] * op(B): A rows at `a` (pitch pa, k contiguous); B^T rows at `b` (B_T: pitch
+// pb, k contiguous) or B rows at `b` (k down the rows, pitch pb).  LDS operands.
+template <bool B_T>
+__device__ __forceinline__ floatx16 tile_product(const float* a, int pa, const float* b, int pb, int K, float sign,
+                                                 floatx16 acc, int lane) {
+    const int x = lane & 31, h = lane >> 5;
+    for (int k2 = 0; k2 < K; k2 += 2) {  // the half-wave h takes k2 + h
+        const int k = k2 + h;
+        const float av = sign * a[x * pa + k];
+        const float bv = B_T ? b[x * pb + k] : b[k * pb + x];
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(av, bv, acc, 0, 0, 0);
+    }
+    return acc;
+}
+
+__device__ __forceinline__ floatx16 tile_load(const float* c, int pc, int lane) {
+    const int x = lane & 31, h = lane >> 5;
+    floatx16 acc;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[r] = c[mfma_row(r, h) * pc + x];
+    return acc;
+}
+
+__device__ __forceinline__ void tile_store(float* c, int pc, const floatx16& acc, int lane) {
+    const int x = lane & 31, h = lane >> 5;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) c[mfma_row(r, h) * pc + x] = acc[r];
+}
+
+__device__ __forceinline__ floatx16 tile_zero() {
+    floatx16 acc;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[r] = 0.0f;
+    return acc;
+}
+
+__global__ __launch_bounds__(256) void spd_diag_kernel(const float* __restrict__ W, uint64_t ldw,
+                                                       float* __restrict__ Lout, float* __restrict__ Linv_out,
+                                                       uint64_t ldl, int32_t block_index,
+                                                       int32_t* __restrict__ status) {
+    __shared__ float As[NB * kPitch];           // the block, overwritten by its factor
+    __shared__ float Xs[NB * kPitch];           // the inverse of the factor
+    __shared__ float Ts[2 * kSub * kTPitch];    // B A^-1 of the halving steps
     const int tid = threadIdx.x;
-    const int p = tid % G, q = tid / G;  // p varies inside a half-wave, q selects the half-wave
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;  // wave index in a scalar register
 
-    float a[T][T], b[T][T];  // A: rows p + G i, columns q + G j;  B: rows q + G i, columns p + G j
+    // thread -> (row tid / 32 + 8 i, four columns from 4 (tid % 32)); all sixteen loads in flight at once
+    // (the block starts at a multiple of 128 floats of a 16-byte aligned matrix with ldw % 128 == 0)
+    {
+        const int r0 = tid >> 5, c = 4 * (tid & 31);
+        float4 v[16];
 #pragma unroll
-    for (int i = 0; i < T; ++i)
+        for (int i = 0; i < 16; ++i) v[i] = *reinterpret_cast<const float4*>(W + (uint64_t)(r0 + 8 * i) * ldw + c);
 #pragma unroll
-        for (int j = 0; j < T; ++j) {
-            const int r = p + G * i, c = q + G * j;
-            a[i][j] = (c <= r) ? W[(uint64_t)r * ldw + c] : 0.0f;
-            b[i][j] = (q + G * i == p + G * j) ? 1.0f : 0.0f;
+        for (int i = 0; i < 16; ++i) {
+            const int r = r0 + 8 * i;
+            float* a = As + r * kPitch + c;
+            float* x = Xs + r * kPitch + c;
+            a[0] = (c + 0 <= r) ? v[i].x : 0.0f;
+            a[1] = (c + 1 <= r) ? v[i].y : 0.0f;
+            a[2] = (c + 2 <= r) ? v[i].z : 0.0f;
+            a[3] = (c + 3 <= r) ? v[i].w : 0.0f;
+            x[0] = x[1] = x[2] = x[3] = 0.0f;
         }
-
-    for (int k = 0; k < NB; ++k) {
-        const int buf = k & 1;
-        const int ks = k / G, kt = k % G;  // column k of A and row k of B: threads with q == kt, slot ks
-        if (q == kt) {                     // one half-wave
-            float col[T], row[T];
-#pragma unroll
-            for (int i = 0; i < T; ++i) {
-                col[i] = 0.0f;
-                row[i] = 0.0f;
-#pragma unroll
-                for (int j = 0; j < T; ++j)
-                    if (j == ks) {
-                        col[i] = a[i][j];
-                        row[i] = b[j][i];
-                    }
-            }
-            if (p == kt) {  // the diagonal element (k, k) is in slot [ks][ks] of this thread
-                float d = 0.0f;
-#pragma unroll
-                for (int i = 0; i < T; ++i)
-                    if (i == ks) d = col[i];
-                if (!(d > 0.0f)) {
-                    if (status && *status == 0) *status = 1 + block_index * NB + k;
-                    d = 1.0f;
-                }
-                pivot[buf] = d;
-            }
-            *reinterpret_cast<float4*>(&vec[buf][T * p]) = make_float4(col[0], col[1], col[2], col[3]);
-            *reinterpret_cast<float4*>(&bvec[buf][T * p]) = make_float4(row[0], row[1], row[2], row[3]);
-        }
-        __syncthreads();
-        const float d = pivot[buf];
-        // hardware reciprocal (1 ulp): it only scales the rank-1 updates; the factor itself below
-        // is scaled with the correctly rounded 1 / sqrt(d)
-        const float inv_d = __builtin_amdgcn_rcpf(d);
-        const float4 vp = *reinterpret_cast<const float4*>(&vec[buf][T * p]);
-        const float4 vq = *reinterpret_cast<const float4*>(&vec[buf][T * q]);
-        const float4 bp = *reinterpret_cast<const float4*>(&bvec[buf][T * p]);
-        const float lr[T] = {vp.x, vp.y, vp.z, vp.w};
-        const float xc[T] = {bp.x, bp.y, bp.z, bp.w};
-        const float rq[T] = {vq.x, vq.y, vq.z, vq.w};
-        if (q == kt) {  // finished column k of L and row k of L^-1, off the critical path of the other waves
-            const float inv_sd = 1.0f / sqrtf(d);
-#pragma unroll
-            for (int i = 0; i < T; ++i) {
-                const int r = p + G * i;
-                Ls[r * kLd + k] = (r >= k) ? lr[i] * inv_sd : 0.0f;  // L[k][k] = d / sqrt(d)
-                const float x = xc[i] * inv_sd;
-#pragma unroll
-                for (int j = 0; j < T; ++j)
-                    if (j == ks) b[j][i] = x;
-            }
-        }
-        float lc[T], br[T];
-#pragma unroll
-        for (int j = 0; j < T; ++j) {
-            const float v = rq[j] * inv_d;
-            lc[j] = v;
-            br[j] = (q + G * j > k) ? v : 0.0f;  // rows <= k of B are finished
-        }
-#pragma unroll
-        for (int i = 0; i < T; ++i)
-#pragma unroll
-            for (int j = 0; j < T; ++j) {
-                a[i][j] -= lr[i] * lc[j];
-                b[i][j] -= br[i] * xc[j];
-            }
     }
     __syncthreads();
 
-#pragma unroll
-    for (int i = 0; i < T; ++i)
-#pragma unroll
-        for (int j = 0; j < T; ++j) {
-            const int r = q + G * i, c = p + G * j;
-            Lout[(uint64_t)r * ldl + c] = (c <= r) ? Ls[r * kLd + c] : 0.0f;
-            Linv_out[(uint64_t)r * ldl + c] = (c <= r) ? b[i][j] : 0.0f;
+    constexpr int kBlocks = NB / kSub;
+    for (int p = 0; p < kBlocks; ++p) {
+        const int base = kSub * p;
+        if (wave == 0) factor_sub_block(As, Xs, base, lane, block_index * NB + base, status);
+        __syncthreads();
+        const int below = kBlocks - 1 - p;  // sub-blocks under the diagonal one
+        if (below == 0) break;
+        // L[t][p] = A[t][p] X_pp^T, one sub-block per wave (at most three)
+        if (wave < below) {
+            float* tile = As + (base + kSub * (1 + wave)) * kPitch + base;
+            const floatx16 acc = tile_product<true>(tile, kPitch, Xs + base * kPitch + base, kPitch, kSub, 1.0f,
+                                                    tile_zero(), lane);
+            tile_store(tile, kPitch, acc, lane);  // every read of the tile precedes this in the wave's LDS order
         }
+        __syncthreads();
+        // A[ti][tj] -= L[ti][p] L[tj][p]^T for the sub-blocks tj <= ti below and right of (p, p)
+        const int tiles = below * (below + 1) / 2;
+        for (int t = wave; t < tiles; t += 4) {
+            const int ti = t < 1 ? 0 : (t < 3 ? 1 : 2), tj = t - ti * (ti + 1) / 2;
+            const int ri = base + kSub * (1 + ti), rj = base + kSub * (1 + tj);
+            float* tile = As + ri * kPitch + rj;
+            const floatx16 acc = tile_product<true>(As + ri * kPitch + base, kPitch, As + rj * kPitch + base, kPitch,
+                                                    kSub, -1.0f, tile_load(tile, kPitch, lane), lane);
+            tile_store(tile, kPitch, acc, lane);
+        }
+        __syncthreads();
+    }
+
+    // halving, level 1: sub-block pairs (0, 1) and (2, 3) on waves 0 and 1
+    if (wave < 2) {
+        const int lo = 2 * kSub * wave, mid = lo + kSub;
+        float* scratch = Ts + kSub * wave * kTPitch;
+        const floatx16 t = tile_product<false>(As + mid * kPitch + lo, kPitch, Xs + lo * kPitch + lo, kPitch, kSub, 1.0f,
+                                               tile_zero(), lane);
+        tile_store(scratch, kTPitch, t, lane);
+    }
+    __syncthreads();
+    if (wave < 2) {
+        const int lo = 2 * kSub * wave, mid = lo + kSub;
+        const float* scratch = Ts + kSub * wave * kTPitch;
+        const floatx16 r = tile_product<false>(Xs + mid * kPitch + mid, kPitch, scratch, kTPitch, kSub, -1.0f,
+                                               tile_zero(), lane);
+        tile_store(Xs + mid * kPitch + lo, kPitch, r, lane);
+    }
+    __syncthreads();
+    // level 2: the 64 x 64 block under the diagonal, one 32 x 32 tile per wave
+    {
+        const int ti = wave >> 1, tj = wave & 1, half = 2 * kSub;
+        const floatx16 t = tile_product<false>(As + (half + kSub * ti) * kPitch, kPitch, Xs + kSub * tj, kPitch, half,
+                                               1.0f, tile_zero(), lane);
+        tile_store(Ts + kSub * ti * kTPitch + kSub * tj, kTPitch, t, lane);
+        __syncthreads();
+        const floatx16 r = tile_product<false>(Xs + (half + kSub * ti) * kPitch + half, kPitch, Ts + kSub * tj, kTPitch,
+                                               half, -1.0f, tile_zero(), lane);
+        tile_store(Xs + (half + kSub * ti) * kPitch + kSub * tj, kPitch, r, lane);
+    }
+    __syncthreads();
+
+    {
+        const int r0 = tid >> 5, c = 4 * (tid & 31);
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            const int r = r0 + 8 * i;
+            const float* a = As + r * kPitch + c;
+            const float* x = Xs + r * kPitch + c;
+            const float a0 = a[0], a1 = a[1], a2 = a[2], a3 = a[3];  // read first, then select: no branches
+            const float x0 = x[0], x1 = x[1], x2 = x[2], x3 = x[3];
+            float4 l, li;
+            l.x = (c + 0 <= r) ? a0 : 0.0f, li.x = (c + 0 <= r) ? x0 : 0.0f;
+            l.y = (c + 1 <= r) ? a1 : 0.0f, li.y = (c + 1 <= r) ? x1 : 0.0f;
+            l.z = (c + 2 <= r) ? a2 : 0.0f, li.z = (c + 2 <= r) ? x2 : 0.0f;
+            l.w = (c + 3 <= r) ? a3 : 0.0f, li.w = (c + 3 <= r) ? x3 : 0.0f;
+            *reinterpret_cast<float4*>(Lout + (uint64_t)r * ldl + c) = l;
+            *reinterpret_cast<float4*>(Linv_out + (uint64_t)r * ldl + c) = li;
+        }
+    }
 }
 
 __global__ __launch_bounds__(256) void abs_sum_kernel(const float* __restrict__ M, uint64_t ld, uint64_t n,
@@ -309,7 +414,7 @@ int spd_inverse(const float* A, uint64_t lda, float lambda, float* inv, uint64_t
 
     for (uint64_t j = 0; j < nblk; ++j) {
         const uint64_t off = j * NB * np + j * NB;
-        hipLaunchKernelGGL(spd_diag_kernel, dim3(1), dim3(1024), 0, s, W + off, np, L + off, Li + off, np,
+        hipLaunchKernelGGL(spd_diag_kernel, dim3(1), dim3(256), 0, s, W + off, np, L + off, Li + off, np,
                            (int32_t)j, status);
         if (hipGetLastError() != hipSuccess) return TRAKHIP_ERR_LAUNCH;
         if (j + 1 == nblk) break;
