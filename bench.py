@@ -345,7 +345,7 @@ def bench_scoring(torch, dev, reps=3):
             best = ms if best is None else min(best, ms)
         return r, best
 
-    from trak_amd.utils import gemm_nt, gemm_nt16, gemm_nt_split, gemm_tn, gram_split, spd_inverse, split_rows
+    from trak_amd.utils import gemm_nt, gemm_nt16, gemm_nt_split, gemm_tn, gram_split, spd_inverse, split2_rows, split_rows
 
     # the fp32 MFMA instruction (v_mfma_f32_32x32x2_f32): priced against the 157.3 TFLOP/s fp32 peak
     xtx, t_xtx = timed(lambda: gemm_tn(X, X))
@@ -362,6 +362,12 @@ def bench_scoring(torch, dev, reps=3):
     _, s_feat = timed(lambda: gemm_nt_split(split_rows(X), split_rows(inv)))
     _, s_sc = timed(lambda: gemm_nt_split(split_rows(feats), split_rows(Xt), row_scale=otl))
     split_ms = s_xtx + s_feat + s_sc
+    # opt-in cheaper split (BasicScoreComputer(gemm="split2")): rows scaled by powers of two, two fp16
+    # planes, three fp16 MFMAs per k step; entries keep 22 significand bits relative to their row's maximum
+    _, q_xtx = timed(lambda: gram_split(split2_rows(X, transposed=True)))
+    _, q_feat = timed(lambda: gemm_nt_split(split2_rows(X), split2_rows(inv)))
+    _, q_sc = timed(lambda: gemm_nt_split(split2_rows(feats), split2_rows(Xt), row_scale=otl))
+    split2_ms = q_xtx + q_feat + q_sc
     # TRAKer's default stores gradients and features as fp16 (use_half_precision): the same products
     # with one MFMA per k step and exact products; X^T X from one fp16 plane (the transposed operand
     # needs the re-layout), the two row-major products read in place (what BasicScoreComputer runs)
@@ -387,6 +393,12 @@ def bench_scoring(torch, dev, reps=3):
             "bf16_mfma_tflops_executed": 6 * split_flop / (split_ms * 1e-3) / 1e12,
             "frac_bf16_mfma_peak": 6 * split_flop / (split_ms * 1e-3) / 1e12 / PEAK_FP16_TFLOPS,
             "xtx_note": "symmetric product: lower-triangle tiles computed and mirrored, flops counted as computed",
+        },
+        "split_fp16x2_opt_in": {
+            "xtx_ms": q_xtx, "x_xtx_inv_ms": q_feat, "scores_ms": q_sc,
+            "gemm_tflops_algorithmic": gemm_flop / (split2_ms * 1e-3) / 1e12,
+            "gemm_tflops_fp32_equivalent": split_flop / (split2_ms * 1e-3) / 1e12,
+            "note": "not the default: operand error up to 2^-22 relative to the row maximum (three-plane split: exact)",
         },
         "fp16_inputs": {
             "xtx_ms": h_xtx, "x_xtx_inv_ms": h_feat, "scores_ms": h_sc,

@@ -165,6 +165,30 @@ int trakhip_gemm_nt_split(const void* A_planes_dev, uint64_t M, const void* B_pl
 int trakhip_gram_split(const void* A_planes_dev, uint64_t N, uint64_t K, int src_dtype, float* C_dev, uint64_t ldc,
                        float alpha, float beta, void* stream);
 
+/* An opt-in cheaper form of the split products for fp32 operands: two fp16 planes per operand and
+ * three fp16 MFMAs per k step instead of three bf16 planes and six MFMAs (about 1.75 times the speed).
+ * trakhip_split2_rows multiplies every operand row by the power of two that brings its largest
+ * magnitude into [2^14, 2^15) and stores x * 2^s = h1 + h2 (fp16, round to nearest even): 22 significand
+ * bits for entries within 2^-18 of the row's largest, fewer below (absolute error <= 2^-26 of the
+ * row's largest magnitude), against all 24 bits of the three-plane split.  The product leaves out
+ * h2 * h2' (below 2^-22 of a product); the powers of two are removed again in the epilogue (exact).
+ * Not a replacement for the exact split where inputs may hold rows of very uneven magnitude.
+ *   trakhip_split2_bytes    bytes of the planes of a [rows, K] fp32 operand
+ *   trakhip_split2_rows     src_dev as for trakhip_split_rows; scales_dev: 2 * rows floats, the first
+ *                           `rows` of them are the inverse row factors that the products take, the rest
+ *                           is scratch
+ *   trakhip_gemm_nt_split2, trakhip_gram_split2   as trakhip_gemm_nt_split / trakhip_gram_split, with
+ *                           each operand's scales_dev
+ * Stand in for the same three matmuls (trak/score_computers.py:153, :176, trak/utils.py:131). */
+size_t trakhip_split2_bytes(uint64_t rows, uint64_t K);
+int trakhip_split2_rows(const float* src_dev, uint64_t ld, uint64_t rows, uint64_t K, int transposed, void* planes_dev,
+                        size_t planes_bytes, float* scales_dev, void* stream);
+int trakhip_gemm_nt_split2(const void* A_planes_dev, const float* A_scales_dev, uint64_t M, const void* B_planes_dev,
+                           const float* B_scales_dev, uint64_t N, uint64_t K, float* C_dev, uint64_t ldc, float alpha,
+                           float beta, const float* row_scale_dev, void* stream);
+int trakhip_gram_split2(const void* A_planes_dev, const float* A_scales_dev, uint64_t N, uint64_t K, float* C_dev,
+                        uint64_t ldc, float alpha, float beta, void* stream);
+
 /* C[M, N] (fp32) = alpha * A[M, K] * B[N, K]^T + beta * C, row i *= row_scale[i], for fp16 or bf16
  * operands read where they are: no planes, no extra pass.  For the two products of a TRAKer that
  * stores half precision whose operands are row-major along the contraction: `block @ xtx_inv`

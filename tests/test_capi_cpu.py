@@ -130,6 +130,34 @@ def test_store_entry_points_validate_before_touching_the_device():
     assert "page-locked" in _lib.strerror(-11)
 
 
+def test_split2_entry_points_validate_before_touching_the_device():
+    lib = _lib.load()
+    p = ctypes.c_void_p(4096)
+    # two fp16 planes x octets padded to 8 x rows padded to 256 x 16 bytes
+    assert lib.trakhip_split2_bytes(1, 1) == 2 * 8 * 256 * 16
+    assert lib.trakhip_split2_bytes(50_000, 4096) == 2 * 512 * 50_176 * 16
+    assert lib.trakhip_split2_bytes(0, 5) == 0 and lib.trakhip_split2_bytes(5, 0) == 0
+    sp = lambda **kw: lib.trakhip_split2_rows(
+        kw.get("src", p), kw.get("ld", 64), kw.get("rows", 10), kw.get("K", 64), kw.get("tr", 0), kw.get("out", p),
+        kw.get("bytes", 1 << 30), kw.get("scales", p), None)
+    assert sp(rows=0) == -2 and sp(K=0) == -2 and sp(ld=63) == -2 and sp(tr=1, ld=9) == -2
+    assert sp(src=None) == -5 and sp(out=None) == -5 and sp(scales=None) == -5
+    assert sp(bytes=100) == -6
+    assert sp(src=ctypes.c_void_p(4098)) == -7 and sp(out=ctypes.c_void_p(4104)) == -7
+    assert sp(scales=ctypes.c_void_p(4097)) == -7
+    mm = lambda **kw: lib.trakhip_gemm_nt_split2(
+        kw.get("a", p), kw.get("sa", p), kw.get("M", 8), kw.get("b", p), kw.get("sb", p), kw.get("N", 8),
+        kw.get("K", 16), kw.get("c", p), kw.get("ldc", 8), 1.0, 0.0, None, None)
+    assert mm(sa=None) == -5 and mm(sb=None) == -5
+    assert mm(M=0) == 0 and mm(N=0) == 0
+    assert mm(K=0) == -2 and mm(ldc=7) == -2
+    assert mm(a=None) == -5 and mm(b=None) == -5 and mm(c=None) == -5
+    assert mm(a=ctypes.c_void_p(4104)) == -7 and mm(c=ctypes.c_void_p(4098)) == -7
+    gr = lambda **kw: lib.trakhip_gram_split2(kw.get("a", p), kw.get("sa", p), kw.get("N", 8), kw.get("K", 16),
+                                              kw.get("c", p), kw.get("ldc", 8), 1.0, 0.0, None)
+    assert gr(N=0) == 0 and gr(sa=None) == -5 and gr(a=None) == -5 and gr(ldc=7) == -2
+
+
 def test_gemm_nt16_validates_before_touching_the_device():
     lib = _lib.load()
     p = ctypes.c_void_p(4096)

@@ -9,7 +9,17 @@ import torch
 
 from oracle import score_oracle as so
 from trak_amd import BasicScoreComputer, get_matrix_mult
-from trak_amd.utils import gemm_nt, gemm_nt16, gemm_nt_split, gemm_tn, gram_split, matmul_nt, spd_inverse, split_rows
+from trak_amd.utils import (
+    gemm_nt,
+    gemm_nt16,
+    gemm_nt_split,
+    gemm_tn,
+    gram_split,
+    matmul_nt,
+    spd_inverse,
+    split2_rows,
+    split_rows,
+)
 
 pytestmark = pytest.mark.gpu
 
@@ -244,6 +254,79 @@ def test_gemm_nt16_refuses_what_it_cannot_read_in_place(gpu):
     assert rel_max(matmul_nt(a, b.bfloat16()).cpu().numpy(), want.cpu().numpy()) < gemm_tol(128)
 
 
+def split2_planes_to_numpy(op):
+    """[2, padded rows, padded K] float64 values of the two fp16 planes of a split2 operand."""
+    Rp, K8 = (op.rows + 255) // 256 * 256, (op.K + 63) // 64 * 8
+    raw = op.planes.cpu().numpy()[: 2 * K8 * Rp * 16].view(np.float16).reshape(2, K8, Rp, 8)
+    return raw.astype(np.float64).transpose(0, 2, 1, 3).reshape(2, Rp, K8 * 8)
+
+
+@pytest.mark.parametrize("rows,K,transposed", [(5, 9, False), (300, 70, False), (70, 300, True), (257, 33, True), (256, 64, False)])
+def test_split2_rows_scales_and_planes(gpu, rows, K, transposed):
+    """Two fp16 planes of the row-scaled operand: the row factor is the power of two that puts the
+    row's largest magnitude into [2^14, 2^15); h1 + h2 equals the scaled value up to 2^-11 of the
+    smaller term (2^-26 of the row's largest magnitude at worst); padding is zero."""
+    gen = torch.Generator(device="cpu").manual_seed(rows * K + 1)
+    t = torch.randn((rows, K), generator=gen)
+    t *= (10.0 ** torch.randint(-20, 20, (rows, 1), generator=gen).float())      # rows of very different size
+    t[0, :] = 0.0                                                              # a row of zeros
+    if rows > 3:
+        t[3, 1:] *= 1e-9                                                       # one large entry, the rest tiny
+    src = (t.T.contiguous() if transposed else t).to(gpu)
+    op = split2_rows(src, transposed=transposed)
+    assert op.rows == rows and op.K == K and op.scales is not None
+    planes = split2_planes_to_numpy(op)
+    unscale = op.scales[:rows].cpu().double().numpy()
+    amax = t.abs().max(dim=1).values.double().numpy()
+    want_unscale = np.where(amax > 0, 2.0 ** (np.floor(np.log2(np.where(amax > 0, amax, 1.0))) - 14), 1.0)
+    assert np.array_equal(unscale, want_unscale)
+    scaled = t.double().numpy() / unscale[:, None]
+    assert np.abs(scaled).max() < 2.0 ** 15
+    got = planes[0, :rows, :K] + planes[1, :rows, :K]
+    # h1 carries 11 bits; h2 the next 11 unless it is subnormal in fp16 (absolute error 2^-25 then)
+    err = np.abs(got - scaled)
+    assert np.all(err <= np.maximum(np.abs(scaled) * 2.0 ** -21, 2.0 ** -25))
+    assert np.array_equal(planes[0, :rows, :K], scaled.astype(np.float16).astype(np.float64))   # RNE first term
+    assert np.count_nonzero(planes[:, rows:, :]) == 0 and np.count_nonzero(planes[:, :, K:]) == 0
+
+
+@pytest.mark.parametrize("M,N,K", [(1, 1, 1), (130, 70, 33), (256, 512, 64), (1000, 513, 257), (64, 2048, 4096), (129, 257, 8200)])
+def test_gemm_nt_split2(gpu, M, N, K):
+    """Three fp16 MFMAs on two planes per operand: error bounded by 2^-21 of sum |a||b| plus the fp32
+    accumulation; alpha, beta, row scale; rows of very different magnitude keep their relative accuracy."""
+    gen = torch.Generator(device="cpu").manual_seed(M + N * 3 + K + 2)
+    a, b = torch.randn(M, K, generator=gen), torch.randn(N, K, generator=gen)
+    a *= 10.0 ** torch.randint(-12, 12, (M, 1), generator=gen).float()
+    b *= 10.0 ** torch.randint(-12, 12, (N, 1), generator=gen).float()
+    a64, b64 = a.double().numpy(), b.double().numpy()
+    want = a64 @ b64.T
+    bound = np.abs(a64) @ np.abs(b64).T                       # sum |a||b| per entry
+    sa, sb = split2_rows(a.to(gpu)), split2_rows(b.to(gpu))
+    got = gemm_nt_split(sa, sb).cpu().double().numpy()
+    assert np.all(np.abs(got - want) <= bound * (2.0 ** -20 + 2e-7 * math.sqrt(K)) + 1e-300)
+    rs = torch.rand(M, generator=gen)
+    c0 = torch.randn(M, N, generator=gen) * float(np.abs(want).max())
+    got = gemm_nt_split(sa, sb, out=c0.clone().to(gpu), alpha=2.0, beta=0.5, row_scale=rs.to(gpu)).cpu().double().numpy()
+    want2 = (2.0 * want + 0.5 * c0.double().numpy()) * rs.double().numpy()[:, None]
+    tol = (2.0 * bound + 0.5 * np.abs(c0.double().numpy())) * (2.0 ** -20 + 2e-7 * math.sqrt(K)) + 1e-300
+    assert np.all(np.abs(got - want2) <= tol)
+    assert torch.equal(matmul_nt(a.to(gpu), b.to(gpu), two_planes=True), gemm_nt_split(sa, sb))
+    with pytest.raises(RuntimeError):
+        gemm_nt_split(sa, split_rows(b.to(gpu)))              # operands of different formats
+
+
+@pytest.mark.parametrize("N,K", [(1, 1), (100, 37), (256, 64), (257, 300), (700, 1030)])
+def test_gram_split2_is_symmetric(gpu, N, K):
+    gen = torch.Generator(device="cpu").manual_seed(N + K)
+    x = torch.randn(K, N, generator=gen)                       # the operand is x^T, read in place
+    g = gram_split(split2_rows(x.to(gpu), transposed=True))
+    want = x.double().numpy().T @ x.double().numpy()
+    assert torch.equal(g, g.T)
+    assert rel_max(g.cpu().numpy(), want) < 2.0 ** -19 + gemm_tol(K)
+    acc = gram_split(split2_rows(x.to(gpu), transposed=True), out=g.clone(), alpha=1.0, beta=1.0)
+    assert torch.equal(acc, acc.T) and rel_max(acc.cpu().numpy(), 2 * want) < 2.0 ** -19 + gemm_tol(K)
+
+
 @pytest.mark.parametrize("M,N,K", [(1, 1, 1), (130, 70, 33), (256, 512, 64), (1000, 513, 257), (64, 2048, 4096), (129, 257, 8200)])
 def test_gemm_nt_split(gpu, M, N, K):
     gen = torch.Generator(device="cpu").manual_seed(M * 7 + N + K)
@@ -305,7 +388,7 @@ def test_gemm_nt_split_keeps_small_terms(gpu):
     assert np.abs(got - K * (1.0 - 2.0 ** -18)).max() <= 2.0 ** -23 * K
 
 
-@pytest.mark.parametrize("gemm", ["split", "fp32"])
+@pytest.mark.parametrize("gemm", ["split", "split2", "fp32"])
 @pytest.mark.parametrize("N,k,M,lam,max_dim", [(700, 512, 90, 1e-3, 20_000), (2500, 1024, 300, 0.0, 1000), (333, 100, 17, 1e-2, 100)])
 def test_score_computer_matches_float64_oracle(gpu, N, k, M, lam, max_dim, gemm):
     gen = torch.Generator(device="cpu").manual_seed(N + k)
@@ -337,7 +420,7 @@ def test_score_computer_matches_float64_oracle(gpu, N, k, M, lam, max_dim, gemm)
     assert rel_max(get_matrix_mult(feats, Xt.to(gpu)).cpu().numpy(), scores_want) < 1e-4
 
 
-@pytest.mark.parametrize("gemm", ["split", "fp32"])
+@pytest.mark.parametrize("gemm", ["split", "split2", "fp32"])
 def test_full_size_scoring_shape(gpu, gemm):
     """N = 50 000 training rows, k = 4096, M = 10 000 targets, lambda = 1e-3: the float64 oracle does not
     finish in seconds on a CPU at this size, so the check uses what does not depend on size: the

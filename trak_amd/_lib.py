@@ -66,6 +66,14 @@ def load():
     lib.trakhip_gemm_nt_split.restype = i32
     lib.trakhip_gram_split.argtypes = [vp, u64, u64, i32, vp, u64, f32, f32, vp]
     lib.trakhip_gram_split.restype = i32
+    lib.trakhip_split2_bytes.argtypes = [u64, u64]
+    lib.trakhip_split2_bytes.restype = sz
+    lib.trakhip_split2_rows.argtypes = [vp, u64, u64, u64, i32, vp, sz, vp, vp]
+    lib.trakhip_split2_rows.restype = i32
+    lib.trakhip_gemm_nt_split2.argtypes = [vp, vp, u64, vp, vp, u64, u64, vp, u64, f32, f32, vp, vp]
+    lib.trakhip_gemm_nt_split2.restype = i32
+    lib.trakhip_gram_split2.argtypes = [vp, vp, u64, u64, vp, u64, f32, f32, vp]
+    lib.trakhip_gram_split2.restype = i32
     lib.trakhip_gemm_nt16.argtypes = [vp, u64, vp, u64, i32, vp, u64, u64, u64, u64, f32, f32, vp, vp]
     lib.trakhip_gemm_nt16.restype = i32
     lib.trakhip_spd_inverse_workspace.argtypes = [u64]

@@ -112,6 +112,27 @@ int trakhip_gram_split(const void* A_planes_dev, uint64_t N, uint64_t K, int dty
     return trakhip::gram_split(A_planes_dev, N, K, dtype, C_dev, ldc, alpha, beta, static_cast<hipStream_t>(stream));
 }
 
+size_t trakhip_split2_bytes(uint64_t rows, uint64_t K) { return trakhip::split2_bytes(rows, K); }
+
+int trakhip_split2_rows(const float* src_dev, uint64_t ld, uint64_t rows, uint64_t K, int transposed, void* planes_dev,
+                        size_t planes_bytes, float* scales_dev, void* stream) {
+    return trakhip::split2_rows(src_dev, ld, rows, K, transposed, planes_dev, planes_bytes, scales_dev,
+                                static_cast<hipStream_t>(stream));
+}
+
+int trakhip_gemm_nt_split2(const void* A_planes_dev, const float* A_scales_dev, uint64_t M, const void* B_planes_dev,
+                           const float* B_scales_dev, uint64_t N, uint64_t K, float* C_dev, uint64_t ldc, float alpha,
+                           float beta, const float* row_scale_dev, void* stream) {
+    return trakhip::gemm_nt_split2(A_planes_dev, A_scales_dev, M, B_planes_dev, B_scales_dev, N, K, C_dev, ldc, alpha,
+                                   beta, row_scale_dev, static_cast<hipStream_t>(stream));
+}
+
+int trakhip_gram_split2(const void* A_planes_dev, const float* A_scales_dev, uint64_t N, uint64_t K, float* C_dev,
+                        uint64_t ldc, float alpha, float beta, void* stream) {
+    return trakhip::gram_split2(A_planes_dev, A_scales_dev, N, K, C_dev, ldc, alpha, beta,
+                                static_cast<hipStream_t>(stream));
+}
+
 int trakhip_gemm_nt16(const void* A_dev, uint64_t lda, const void* B_dev, uint64_t ldb, int dtype, float* C_dev,
                       uint64_t ldc, uint64_t M, uint64_t N, uint64_t K, float alpha, float beta,
                       const float* row_scale_dev, void* stream) {

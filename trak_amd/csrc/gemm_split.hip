@@ -12,6 +12,12 @@
 // cost of the fp32 instruction.  The three terms left out are each below 2^-24 |a b|, the rounding
 // a single fp32 multiplication makes.
 // fp16 or bf16 operands (both of the same type): one plane, one MFMA, nothing left out.
+// An opt-in cheaper variant for fp32 operands ("two fp16 planes"): every row is scaled by a power of two
+// that brings its largest magnitude to [2^14, 2^15), then x = h1 + h2 with fp16 terms (22 significand
+// bits for entries within 2^-18 of the row's largest, fewer below), and
+//     a * b = a1 b1 + (a1 b2 + a2 b1) + O(2^-22 |a b|)
+// with three fp16 MFMAs; the powers of two are taken out again in the epilogue.  Half the MFMAs of the
+// three-plane product at four times its operand error bound.
 //
 // Operands are brought once, outside the GEMM, into "planes": plane p, k-octet o (8 consecutive k),
 // row r is one 16-byte piece at ((p * K8 + o) * Rp + r) * 16 bytes, rows padded with zeros to a
@@ -123,6 +129,106 @@ __global__ __launch_bounds__(256) void relayout16_kernel(const uint16_t* __restr
     planes[o * Rp + r] = w;
 }
 
+// ---- two fp16 planes with a power-of-two scale per row ------------------------------------------
+
+// Largest magnitude of every operand row as binary32 bits (non-negative floats order like unsigned
+// integers).  Row-major operand: one wave per row.
+__global__ __launch_bounds__(256) void absmax_rows_kernel(const float* __restrict__ src, uint64_t ld, uint64_t rows,
+                                                          uint64_t K, uint32_t* __restrict__ maxbits) {
+    const uint64_t r = (uint64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (r >= rows) return;
+    const int lane = threadIdx.x & 63;
+    uint32_t m = 0;
+    for (uint64_t k = lane; k < K; k += 64) {
+        const uint32_t b = __float_as_uint(src[r * ld + k]) & 0x7FFFFFFFu;
+        m = b > m ? b : m;
+    }
+#pragma unroll
+    for (int w = 32; w > 0; w >>= 1) {
+        const uint32_t o = (uint32_t)__shfl_xor((int)m, w);
+        m = o > m ? o : m;
+    }
+    if (lane == 0) maxbits[r] = m;
+}
+
+// Transposed operand (row r of the operand is column r of src[K, rows]): a thread walks one column over
+// one chunk of k and merges with an atomic maximum (order independent); maxbits starts at zero.
+constexpr int kColChunks = 64;
+__global__ __launch_bounds__(256) void absmax_cols_kernel(const float* __restrict__ src, uint64_t ld, uint64_t rows,
+                                                          uint64_t K, uint32_t* __restrict__ maxbits) {
+    const uint64_t r = (uint64_t)blockIdx.x * 256 + threadIdx.x;
+    if (r >= rows) return;
+    const uint64_t per = (K + kColChunks - 1) / kColChunks;
+    const uint64_t k0 = (uint64_t)blockIdx.y * per, k1 = k0 + per < K ? k0 + per : K;
+    uint32_t m = 0;
+    for (uint64_t k = k0; k < k1; ++k) {
+        const uint32_t b = __float_as_uint(src[k * ld + r]) & 0x7FFFFFFFu;
+        m = b > m ? b : m;
+    }
+    if (m) atomicMax(maxbits + r, m);
+}
+
+__global__ __launch_bounds__(256) void zero_u32_kernel(uint32_t* __restrict__ p, uint64_t n) {
+    const uint64_t i = (uint64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < n) p[i] = 0u;
+}
+
+// Power of two that brings a row whose largest magnitude has these bits into [2^14, 2^15) (fp16 tops
+// out at 65504), and its inverse.  A row of zeros, or one that holds an infinity or a NaN, is left alone.
+__device__ __forceinline__ void row_factors(uint32_t maxbits, float& scale, float& unscale) {
+    int sh = 0;
+    if (maxbits != 0u && maxbits < 0x7F800000u) {
+        sh = 14 - ((int)(maxbits >> 23) - 127);
+        sh = sh > 126 ? 126 : sh;
+    }
+    scale = __uint_as_float((uint32_t)(127 + sh) << 23);
+    unscale = __uint_as_float((uint32_t)(127 - sh) << 23);
+}
+
+// One thread per (row r, octet o), as split_kernel: x * scale = h1 + h2 with fp16 terms, planes 0 and 1.
+template <bool TRANS, bool ALIGNED>
+__global__ __launch_bounds__(256) void split2_kernel(const float* __restrict__ src, uint64_t ld, uint64_t rows,
+                                                     uint64_t K, uint64_t Rp, uint64_t K8, uint32_t row_blocks,
+                                                     const uint32_t* __restrict__ maxbits, uint4* __restrict__ planes,
+                                                     float* __restrict__ unscale_out) {
+    const uint64_t r = (uint64_t)(blockIdx.x % row_blocks) * 64 + (threadIdx.x & 63);
+    const uint64_t o = (uint64_t)(blockIdx.x / row_blocks) * 4 + (threadIdx.x >> 6);
+    if (r >= Rp || o >= K8) return;
+    float scale = 1.0f, unscale = 1.0f;
+    if (r < rows) row_factors(maxbits[r], scale, unscale);
+    if (o == 0 && r < rows) unscale_out[r] = unscale;
+    float v[8];
+    if (!TRANS && ALIGNED && r < rows && 8 * o + 8 <= K) {
+        const float4* q = reinterpret_cast<const float4*>(src + r * ld + 8 * o);
+        const float4 lo = q[0], hi = q[1];
+        v[0] = lo.x, v[1] = lo.y, v[2] = lo.z, v[3] = lo.w;
+        v[4] = hi.x, v[5] = hi.y, v[6] = hi.z, v[7] = hi.w;
+    } else {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const uint64_t k = 8 * o + i;
+            v[i] = (r < rows && k < K) ? (TRANS ? src[k * ld + r] : src[r * ld + k]) : 0.0f;
+        }
+    }
+    uint32_t w[2][4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        uint32_t t[2][2];
+#pragma unroll
+        for (int e = 0; e < 2; ++e) {
+            const float x = v[2 * i + e] * scale;  // exact: a power of two, no overflow by construction
+            const _Float16 h1 = (_Float16)x;       // round to nearest even
+            const _Float16 h2 = (_Float16)(x - (float)h1);
+            t[0][e] = (uint32_t)__builtin_bit_cast(uint16_t, h1);
+            t[1][e] = (uint32_t)__builtin_bit_cast(uint16_t, h2);
+        }
+        w[0][i] = t[0][0] | (t[0][1] << 16);
+        w[1][i] = t[1][0] | (t[1][1] << 16);
+    }
+#pragma unroll
+    for (int p = 0; p < 2; ++p) planes[((uint64_t)p * K8 + o) * Rp + r] = make_uint4(w[p][0], w[p][1], w[p][2], w[p][3]);
+}
+
 // ---- GEMM ----------------------------------------------------------------------------------
 
 template <bool F16>
@@ -139,46 +245,57 @@ __device__ __forceinline__ floatx16 mfma16(const piece& a, const piece& b, float
 // n = lane % 32; register r holds row 8*(r/4) + 4*(lane/32) + r%4.  When C is accumulated into (ACCUM),
 // its old values are fetched for 32 rows at a time before any of them is overwritten (loads and stores
 // through one pointer would otherwise alternate, one memory round trip per element).
-template <bool ACCUM, int JT>
+// SCALED: the accumulators are products of operands whose rows were multiplied by powers of two;
+// a_unscale[row] and b_unscale[col] are the inverse factors (applied one after the other, so that no
+// intermediate leaves the binary32 range when the result does not).
+template <bool ACCUM, int JT, bool SCALED = false>
 __device__ __forceinline__ void store_c(const floatx16 (&acc)[2][JT], float* __restrict__ C, uint64_t ldc, uint64_t M,
                                         uint64_t N, uint64_t row_base, uint64_t col0, int h, float alpha, float beta,
-                                        const float* __restrict__ row_scale) {
-    if constexpr (!ACCUM) {
+                                        const float* __restrict__ row_scale,
+                                        const float* __restrict__ a_unscale = nullptr,
+                                        const float* __restrict__ b_unscale = nullptr) {
+    float ub[JT];
 #pragma unroll
-        for (int i = 0; i < 2; ++i) {
+    for (int j = 0; j < JT; ++j) ub[j] = (SCALED && col0 + 32 * j < N) ? b_unscale[col0 + 32 * j] : 1.0f;
 #pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const uint64_t row = row_base + 32 * i + 8 * (r >> 2) + 4 * h + (r & 3);
-                if (row >= M) continue;
-                const float rs = row_scale ? row_scale[row] : 1.0f;
+    for (int i = 0; i < 2; ++i) {
+        const uint64_t row0 = row_base + 32 * i + 4 * h;
+        float ua[16];
 #pragma unroll
-                for (int j = 0; j < JT; ++j) {
-                    const uint64_t col = col0 + 32 * j;
-                    if (col < N) C[row * ldc + col] = alpha * acc[i][j][r] * rs;
-                }
-            }
+        for (int r = 0; r < 16; ++r) {
+            const uint64_t row = row0 + 8 * (r >> 2) + (r & 3);
+            ua[r] = (SCALED && row < M) ? a_unscale[row] : 1.0f;
         }
-    } else {
+        // old values of C: fetched for a group of columns before any of them is overwritten (all four
+        // 32-column groups at once, two at a time when the unscale factors take registers as well)
+        constexpr int JG = (ACCUM && SCALED) ? (JT + 1) / 2 : JT;
 #pragma unroll
-        for (int i = 0; i < 2; ++i) {
-            const uint64_t row0 = row_base + 32 * i + 4 * h;
-            floatx16 prev[JT];
+        for (int j0 = 0; j0 < JT; j0 += JG) {
+            floatx16 prev[ACCUM ? JG : 1];
+            if constexpr (ACCUM) {
 #pragma unroll
-            for (int j = 0; j < JT; ++j)
+                for (int j = 0; j < JG; ++j)
 #pragma unroll
-                for (int r = 0; r < 16; ++r) {
-                    const uint64_t row = row0 + 8 * (r >> 2) + (r & 3), col = col0 + 32 * j;
-                    prev[j][r] = (row < M && col < N) ? C[row * ldc + col] : 0.0f;
-                }
+                    for (int r = 0; r < 16; ++r) {
+                        const uint64_t row = row0 + 8 * (r >> 2) + (r & 3), col = col0 + 32 * (j0 + j);
+                        prev[j][r] = (j0 + j < JT && row < M && col < N) ? C[row * ldc + col] : 0.0f;
+                    }
+            }
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
                 const uint64_t row = row0 + 8 * (r >> 2) + (r & 3);
                 if (row >= M) continue;
                 const float rs = row_scale ? row_scale[row] : 1.0f;
 #pragma unroll
-                for (int j = 0; j < JT; ++j) {
-                    const uint64_t col = col0 + 32 * j;
-                    if (col < N) C[row * ldc + col] = (alpha * acc[i][j][r] + beta * prev[j][r]) * rs;
+                for (int j = 0; j < JG; ++j) {
+                    const uint64_t col = col0 + 32 * (j0 + j);
+                    if (j0 + j >= JT || col >= N) continue;
+                    float v = acc[i][j0 + j][r];
+                    if constexpr (SCALED) v = (v * ua[r]) * ub[j0 + j];
+                    if constexpr (ACCUM)
+                        C[row * ldc + col] = (alpha * v + beta * prev[j][r]) * rs;
+                    else
+                        C[row * ldc + col] = alpha * v * rs;
                 }
             }
         }
@@ -221,7 +338,8 @@ template <int P, bool F16, int S, bool ACCUM>
 __global__ __launch_bounds__(64 * kWaves, 2) void gemm_split_kernel(
     const piece* __restrict__ A, uint64_t Rpa, const piece* __restrict__ B, uint64_t Rpb, uint64_t K8,
     float* __restrict__ C, uint64_t ldc, uint64_t M, uint64_t N, float alpha, float beta,
-    const float* __restrict__ row_scale, uint32_t tiles_n, uint32_t flags) {
+    const float* __restrict__ row_scale, uint32_t tiles_n, uint32_t flags, const float* __restrict__ a_unscale,
+    const float* __restrict__ b_unscale) {
     constexpr int JT = BN / kWavesN / 32;            // 32-column MFMA tiles per wave
     constexpr int kAPieces = P * 2 * BM;             // [plane][half][row]
     constexpr int kSubPieces = P * 2 * (BM + BN);    // three planes: 3072 pieces = 48 KB
@@ -280,6 +398,15 @@ __global__ __launch_bounds__(64 * kWaves, 2) void gemm_split_kernel(
 #pragma unroll
                         for (int i = 0; i < 2; ++i)
                             acc[i][j] = mfma16<F16>(fa[i][kPa[t6]], fb[kPb[t6]], acc[i][j]);
+                } else if constexpr (P == 2) {
+                    // the three plane pairs with pa + pb <= 1, smaller terms first
+                    constexpr int kPa[3] = {0, 1, 0};
+                    constexpr int kPb[3] = {1, 0, 0};
+#pragma unroll
+                    for (int t3 = 0; t3 < 3; ++t3)
+#pragma unroll
+                        for (int i = 0; i < 2; ++i)
+                            acc[i][j] = mfma16<F16>(fa[i][kPa[t3]], fb[kPb[t3]], acc[i][j]);
                 } else {
 #pragma unroll
                     for (int i = 0; i < 2; ++i) acc[i][j] = mfma16<F16>(fa[i][0], fb[0], acc[i][j]);
@@ -290,7 +417,8 @@ __global__ __launch_bounds__(64 * kWaves, 2) void gemm_split_kernel(
         __syncthreads();
     }
 
-    store_c<ACCUM, JT>(acc, C, ldc, M, N, m0 + wm * 64, n0 + wn * (32 * JT) + x, h, alpha, beta, row_scale);
+    store_c<ACCUM, JT, P == 2>(acc, C, ldc, M, N, m0 + wm * 64, n0 + wn * (32 * JT) + x, h, alpha, beta, row_scale,
+                               a_unscale, b_unscale);
 }
 
 // ---- 16-bit operands read in place -----------------------------------------------------------
@@ -453,9 +581,21 @@ int split_rows(const void* src, int dtype, uint64_t ld, uint64_t rows, uint64_t 
     return hipGetLastError() == hipSuccess ? TRAKHIP_OK : TRAKHIP_ERR_LAUNCH;
 }
 
-int gemm_nt_split(const void* A_planes, uint64_t M, const void* B_planes, uint64_t N, uint64_t K, int dtype, float* C,
-                  uint64_t ldc, float alpha, float beta, const float* row_scale, hipStream_t s, uint32_t flags) {
-    if (!known_dtype(dtype)) return TRAKHIP_ERR_DTYPE;
+}  // namespace trakhip
+
+namespace {
+
+// completes a symmetric matrix whose lower-triangle tiles were computed
+int mirror_lower(float* C, uint64_t ldc, uint64_t N, hipStream_t s) {
+    const uint64_t blocks = (N + 31) / 32;
+    if (blocks > 65535) return TRAKHIP_ERR_SHAPE;
+    hipLaunchKernelGGL(mirror_lower_kernel, dim3((uint32_t)blocks, (uint32_t)blocks), dim3(256), 0, s, C, ldc, N);
+    return hipGetLastError() == hipSuccess ? TRAKHIP_OK : TRAKHIP_ERR_LAUNCH;
+}
+
+int launch_split(const void* A_planes, uint64_t M, const void* B_planes, uint64_t N, uint64_t K, int dtype, float* C,
+                 uint64_t ldc, float alpha, float beta, const float* row_scale, hipStream_t s, uint32_t flags,
+                 const float* a_unscale, const float* b_unscale) {
     if (M == 0 || N == 0) return TRAKHIP_OK;
     if (K == 0 || ldc < N) return TRAKHIP_ERR_SHAPE;
     if (!A_planes || !B_planes || !C) return TRAKHIP_ERR_NULL;
@@ -470,17 +610,88 @@ int gemm_nt_split(const void* A_planes, uint64_t M, const void* B_planes, uint64
     const uint64_t Rpa = padded_rows(M), Rpb = padded_rows(N), K8 = octets(K);
     // ACCUM (beta != 0) fetches the old C in the epilogue; kept out of the plain kernel
     void (*kernel)(const piece*, uint64_t, const piece*, uint64_t, uint64_t, float*, uint64_t, uint64_t, uint64_t, float,
-                   float, const float*, uint32_t, uint32_t);
+                   float, const float*, uint32_t, uint32_t, const float*, const float*);
     const bool accum = beta != 0.0f;
-    if (dtype == TRAKHIP_F32)
+    if (a_unscale)
+        kernel = accum ? gemm_split_kernel<2, true, 2, true> : gemm_split_kernel<2, true, 2, false>;
+    else if (dtype == TRAKHIP_F32)
         kernel = accum ? gemm_split_kernel<3, false, 1, true> : gemm_split_kernel<3, false, 1, false>;
     else if (dtype == TRAKHIP_F16)
         kernel = accum ? gemm_split_kernel<1, true, 4, true> : gemm_split_kernel<1, true, 4, false>;
     else
         kernel = accum ? gemm_split_kernel<1, false, 4, true> : gemm_split_kernel<1, false, 4, false>;
     hipLaunchKernelGGL(kernel, grid, block, 0, s, a, Rpa, b, Rpb, K8, C, ldc, M, N, alpha, beta, row_scale,
-                       (uint32_t)tiles_n, flags);
+                       (uint32_t)tiles_n, flags, a_unscale, b_unscale);
     return hipGetLastError() == hipSuccess ? TRAKHIP_OK : TRAKHIP_ERR_LAUNCH;
+}
+
+}  // namespace
+
+namespace trakhip {
+
+int gemm_nt_split(const void* A_planes, uint64_t M, const void* B_planes, uint64_t N, uint64_t K, int dtype, float* C,
+                  uint64_t ldc, float alpha, float beta, const float* row_scale, hipStream_t s, uint32_t flags) {
+    if (!known_dtype(dtype)) return TRAKHIP_ERR_DTYPE;
+    return launch_split(A_planes, M, B_planes, N, K, dtype, C, ldc, alpha, beta, row_scale, s, flags, nullptr, nullptr);
+}
+
+size_t split2_bytes(uint64_t rows, uint64_t K) {
+    if (rows == 0 || K == 0) return 0;
+    return (size_t)(2 * octets(K) * padded_rows(rows) * 16);
+}
+
+int split2_rows(const float* src, uint64_t ld, uint64_t rows, uint64_t K, int transposed, void* planes,
+                size_t planes_bytes, float* scales, hipStream_t s) {
+    if (rows == 0 || K == 0) return TRAKHIP_ERR_SHAPE;
+    if (ld < (transposed ? rows : K)) return TRAKHIP_ERR_SHAPE;
+    if (!src || !planes || !scales) return TRAKHIP_ERR_NULL;
+    if (planes_bytes < split2_bytes(rows, K)) return TRAKHIP_ERR_WORKSPACE;
+    if ((reinterpret_cast<uintptr_t>(src) % 4) || (reinterpret_cast<uintptr_t>(planes) % 16) ||
+        (reinterpret_cast<uintptr_t>(scales) % 4))
+        return TRAKHIP_ERR_ALIGN;
+    const uint64_t Rp = padded_rows(rows), K8 = octets(K);
+    const uint64_t gx = Rp / 64, gy = (K8 + 3) / 4;
+    if (gx * gy > 0x7FFFFFFFull || rows > 0x7FFFFFFFull) return TRAKHIP_ERR_SHAPE;
+    // scales[0 .. rows) receives the inverse factors; scales[rows .. 2 rows) holds the row maxima meanwhile
+    uint32_t* maxbits = reinterpret_cast<uint32_t*>(scales + rows);
+    if (transposed) {
+        hipLaunchKernelGGL(zero_u32_kernel, dim3((uint32_t)((rows + 255) / 256)), dim3(256), 0, s, maxbits, rows);
+        hipLaunchKernelGGL(absmax_cols_kernel, dim3((uint32_t)((rows + 255) / 256), kColChunks), dim3(256), 0, s, src, ld,
+                           rows, K, maxbits);
+    } else {
+        hipLaunchKernelGGL(absmax_rows_kernel, dim3((uint32_t)((rows + 3) / 4)), dim3(256), 0, s, src, ld, rows, K,
+                           maxbits);
+    }
+    const dim3 grid((uint32_t)(gx * gy)), block(256);
+    uint4* out = static_cast<uint4*>(planes);
+    const bool aligned = reinterpret_cast<uintptr_t>(src) % 16 == 0 && (ld * 4) % 16 == 0;
+    if (transposed)
+        hipLaunchKernelGGL((split2_kernel<true, false>), grid, block, 0, s, src, ld, rows, K, Rp, K8, (uint32_t)gx, maxbits,
+                           out, scales);
+    else if (aligned)
+        hipLaunchKernelGGL((split2_kernel<false, true>), grid, block, 0, s, src, ld, rows, K, Rp, K8, (uint32_t)gx, maxbits,
+                           out, scales);
+    else
+        hipLaunchKernelGGL((split2_kernel<false, false>), grid, block, 0, s, src, ld, rows, K, Rp, K8, (uint32_t)gx,
+                           maxbits, out, scales);
+    return hipGetLastError() == hipSuccess ? TRAKHIP_OK : TRAKHIP_ERR_LAUNCH;
+}
+
+int gemm_nt_split2(const void* A_planes, const float* a_scales, uint64_t M, const void* B_planes, const float* b_scales,
+                   uint64_t N, uint64_t K, float* C, uint64_t ldc, float alpha, float beta, const float* row_scale,
+                   hipStream_t s, uint32_t flags) {
+    if ((M && !a_scales) || (N && !b_scales)) return TRAKHIP_ERR_NULL;
+    return launch_split(A_planes, M, B_planes, N, K, TRAKHIP_F32, C, ldc, alpha, beta, row_scale, s, flags, a_scales,
+                        b_scales);
+}
+
+int gram_split2(const void* A_planes, const float* a_scales, uint64_t N, uint64_t K, float* C, uint64_t ldc, float alpha,
+                float beta, hipStream_t s) {
+    if (N == 0) return TRAKHIP_OK;
+    const int e = gemm_nt_split2(A_planes, a_scales, N, A_planes, a_scales, N, K, C, ldc, alpha, beta, nullptr, s,
+                                 kGemmLowerTilesOnly);
+    if (e) return e;
+    return mirror_lower(C, ldc, N, s);
 }
 
 int gemm_nt16(const void* A, uint64_t lda, const void* B, uint64_t ldb, int dtype, float* C, uint64_t ldc, uint64_t M,
@@ -512,10 +723,7 @@ int gram_split(const void* A_planes, uint64_t N, uint64_t K, int dtype, float* C
     if (N == 0) return TRAKHIP_OK;
     const int e = gemm_nt_split(A_planes, N, A_planes, N, K, dtype, C, ldc, alpha, beta, nullptr, s, kGemmLowerTilesOnly);
     if (e) return e;
-    const uint64_t blocks = (N + 31) / 32;
-    if (blocks > 65535) return TRAKHIP_ERR_SHAPE;
-    hipLaunchKernelGGL(mirror_lower_kernel, dim3((uint32_t)blocks, (uint32_t)blocks), dim3(256), 0, s, C, ldc, N);
-    return hipGetLastError() == hipSuccess ? TRAKHIP_OK : TRAKHIP_ERR_LAUNCH;
+    return mirror_lower(C, ldc, N, s);
 }
 
 }  // namespace trakhip

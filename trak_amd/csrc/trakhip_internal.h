@@ -57,6 +57,14 @@ int gemm_nt_split(const void* A_planes, uint64_t M, const void* B_planes, uint64
                   uint64_t ldc, float alpha, float beta, const float* row_scale, hipStream_t s, uint32_t flags = 0);
 int gram_split(const void* A_planes, uint64_t N, uint64_t K, int dtype, float* C, uint64_t ldc, float alpha, float beta,
                hipStream_t s);
+size_t split2_bytes(uint64_t rows, uint64_t K);
+int split2_rows(const float* src, uint64_t ld, uint64_t rows, uint64_t K, int transposed, void* planes,
+                size_t planes_bytes, float* scales, hipStream_t s);
+int gemm_nt_split2(const void* A_planes, const float* a_scales, uint64_t M, const void* B_planes, const float* b_scales,
+                   uint64_t N, uint64_t K, float* C, uint64_t ldc, float alpha, float beta, const float* row_scale,
+                   hipStream_t s, uint32_t flags = 0);
+int gram_split2(const void* A_planes, const float* a_scales, uint64_t N, uint64_t K, float* C, uint64_t ldc, float alpha,
+                float beta, hipStream_t s);
 int gemm_nt16(const void* A, uint64_t lda, const void* B, uint64_t ldb, int dtype, float* C, uint64_t ldc, uint64_t M,
               uint64_t N, uint64_t K, float alpha, float beta, const float* row_scale, hipStream_t s);
 size_t spd_inverse_workspace_bytes(uint64_t n);

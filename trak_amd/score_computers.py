@@ -21,6 +21,7 @@ from .utils import (
     matmul_nt,
     scores_finalize,
     spd_inverse,
+    split2_rows,
     split_rows,
 )
 
@@ -59,7 +60,10 @@ class BasicScoreComputer(AbstractScoreComputer):
     `gemm` selects how the three matrix products are computed: "split" (default) splits every
     fp32 operand exactly into three bf16 terms and runs six bf16 MFMAs per k step with fp32
     accumulation (same error as the fp32 instruction, 1.7 times its speed); "fp32" uses the fp32
-    MFMA instruction directly.
+    MFMA instruction directly; "split2" is an opt-in cheaper split for fp32 operands (rows scaled by a
+    power of two, two fp16 planes, three MFMAs per k step: entries keep 22 significand bits relative
+    to their row's largest magnitude instead of all 24; 1.75 times the speed of "split").  fp16 / bf16
+    operands are multiplied as they are (exact products) under "split" and "split2".
     """
 
     def __init__(
@@ -72,8 +76,8 @@ class BasicScoreComputer(AbstractScoreComputer):
         gemm: str = "split",
     ) -> None:
         super().__init__(dtype, device)
-        if gemm not in ("split", "fp32"):
-            raise ValueError('gemm must be "split" or "fp32"')
+        if gemm not in ("split", "split2", "fp32"):
+            raise ValueError('gemm must be "split", "split2" or "fp32"')
         self.gemm = gemm
         self.CUDA_MAX_DIM_SIZE = CUDA_MAX_DIM_SIZE
         self.logger = logging.getLogger("ScoreComputer")
@@ -94,9 +98,9 @@ class BasicScoreComputer(AbstractScoreComputer):
         result = ch.zeros(self.proj_dim, self.proj_dim, dtype=ch.float32, device=self._dev)
         for block in self._blocks(grads):
             block = block.to(self._dev)
-            if self.gemm == "split":
+            if self.gemm != "fp32":
                 # the operand is block^T, read in place; lower-triangle tiles + mirror image
-                gram_split(split_rows(block, transposed=True), out=result, alpha=1.0, beta=1.0)
+                gram_split(self._split(block, transposed=True), out=result, alpha=1.0, beta=1.0)
             else:
                 gemm_tn(block, block, out=result, alpha=1.0, beta=1.0)
         return result.to(self.dtype)
@@ -115,14 +119,14 @@ class BasicScoreComputer(AbstractScoreComputer):
         for block in self._blocks(grads):
             end = start + block.shape[0]
             # the inverse is symmetric, so block @ inv == block @ inv^T
-            if self.gemm == "split":
+            if self.gemm != "fp32":
                 block = block.to(self._dev)
                 if half and _nt16_ok(block, xtx_inv):
                     gemm_nt16(block, xtx_inv, out=result[start:end])
                 else:
                     if inv_split is None:
-                        inv_split = split_rows(xtx_inv if half else xtx_inv.float())
-                    gemm_nt_split(split_rows(block if half else block.float()), inv_split, out=result[start:end])
+                        inv_split = self._split(xtx_inv if half else xtx_inv.float())
+                    gemm_nt_split(self._split(block if half else block.float()), inv_split, out=result[start:end])
             else:
                 gemm_nt(block.to(self._dev), xtx_inv, out=result[start:end])
             start = end
@@ -157,9 +161,17 @@ class BasicScoreComputer(AbstractScoreComputer):
             features.to(self._dev), target_grads.to(self._dev), alpha=scale, row_scale=out_to_loss.reshape(-1)
         )
 
+    def _split(self, t, transposed=False):
+        """Operand format of the chosen product: 16-bit matrices stay one plane; fp32 ones become three
+        exact bf16 planes ("split") or two scaled fp16 planes ("split2")."""
+        if self.gemm == "split2" and t.dtype not in (ch.float16, ch.bfloat16):
+            return split2_rows(t, transposed=transposed)
+        return split_rows(t, transposed=transposed)
+
     def _matmul_nt(self, a, b, out=None, alpha=1.0, beta=0.0, row_scale=None):
-        if self.gemm == "split":
-            return matmul_nt(a, b, out=out, alpha=alpha, beta=beta, row_scale=row_scale)
+        if self.gemm != "fp32":
+            return matmul_nt(a, b, out=out, alpha=alpha, beta=beta, row_scale=row_scale,
+                             two_planes=self.gemm == "split2")
         return gemm_nt(a, b, out=out, alpha=alpha, beta=beta, row_scale=row_scale)
 
 

@@ -154,10 +154,11 @@ def gemm_tn(a, b, out=None, alpha=1.0, beta=0.0):
 
 class SplitOperand:
     """A matrix [rows, K] in the operand format of `gemm_nt_split`: three bf16 planes whose sum is
-    the matrix exactly (fp32 source) or the matrix itself as one plane (fp16 / bf16 source)."""
+    the matrix exactly (fp32 source), the matrix itself as one plane (fp16 / bf16 source), or - from
+    `split2_rows` - two fp16 planes of the row-scaled matrix with the inverse row factors in `scales`."""
 
-    def __init__(self, planes, rows, K, dtype):
-        self.planes, self.rows, self.K, self.dtype = planes, int(rows), int(K), dtype
+    def __init__(self, planes, rows, K, dtype, scales=None):
+        self.planes, self.rows, self.K, self.dtype, self.scales = planes, int(rows), int(K), dtype, scales
 
     @property
     def device(self):
@@ -191,6 +192,33 @@ def split_rows(t, transposed=False):
     return SplitOperand(planes, rows, K, t.dtype)
 
 
+def split2_rows(t, transposed=False):
+    """The cheaper, slightly less accurate operand format for an fp32 CUDA matrix: every row times a power
+    of two, then two fp16 planes (22 significand bits for entries within 2^-18 of the row's largest
+    magnitude).  `gemm_nt_split` / `gram_split` of two such operands run three fp16 MFMAs per k step
+    instead of six bf16 ones.  Arguments as for `split_rows`."""
+    if t.dim() != 2:
+        raise RuntimeError("t must be 2D")
+    t = t.float()
+    if t.stride(1) != 1 or (t.shape[0] > 1 and t.stride(0) < t.shape[1]):
+        t = t.contiguous()
+    if not t.is_cuda:
+        raise RuntimeError("split2_rows needs a CUDA tensor")
+    rows, K = (t.shape[1], t.shape[0]) if transposed else (t.shape[0], t.shape[1])
+    lib = _lib.load()
+    nbytes = lib.trakhip_split2_bytes(rows, K)
+    with torch.cuda.device(t.device):
+        planes = torch.empty(max(nbytes, 16), dtype=torch.uint8, device=t.device)
+        scales = torch.empty(2 * max(rows, 1), dtype=torch.float32, device=t.device)
+        stream = torch.cuda.current_stream(t.device).cuda_stream
+        code = lib.trakhip_split2_rows(
+            ctypes.c_void_p(t.data_ptr()), _ld(t), rows, K, int(bool(transposed)), ctypes.c_void_p(planes.data_ptr()),
+            planes.numel(), ctypes.c_void_p(scales.data_ptr()), ctypes.c_void_p(stream),
+        )
+    _lib.check(code)
+    return SplitOperand(planes, rows, K, torch.float32, scales=scales)
+
+
 def split_pair(a, b, a_transposed=False):
     """Both operands of one product in a common format: 16-bit operands of one type stay as they
     are (one plane each), any other combination is multiplied from fp32 splits."""
@@ -205,8 +233,8 @@ def gemm_nt_split(a, b, out=None, alpha=1.0, beta=0.0, row_scale=None):
     accumulation, fp32-level accuracy."""
     if not isinstance(a, SplitOperand) or not isinstance(b, SplitOperand):
         raise TypeError("gemm_nt_split takes SplitOperand arguments (see split_rows)")
-    if a.K != b.K or a.device != b.device or a.dtype != b.dtype:
-        raise RuntimeError("operands must share the inner dimension, the device and the source dtype")
+    if a.K != b.K or a.device != b.device or a.dtype != b.dtype or (a.scales is None) != (b.scales is None):
+        raise RuntimeError("operands must share the inner dimension, the device, the source dtype and the format")
     M, N, K = a.rows, b.rows, a.K
     if out is None:
         out = torch.empty((M, N), dtype=torch.float32, device=a.device)
@@ -221,11 +249,19 @@ def gemm_nt_split(a, b, out=None, alpha=1.0, beta=0.0, row_scale=None):
     lib = _lib.load()
     with torch.cuda.device(a.device):
         stream = torch.cuda.current_stream(a.device).cuda_stream
-        code = lib.trakhip_gemm_nt_split(
-            ctypes.c_void_p(a.planes.data_ptr()), M, ctypes.c_void_p(b.planes.data_ptr()), N, K,
-            _STORE_DTYPES[a.dtype], ctypes.c_void_p(out.data_ptr()), _ld(out), float(alpha), float(beta),
-            ctypes.c_void_p(rs.data_ptr()) if rs is not None else None, ctypes.c_void_p(stream),
-        )
+        rs_ptr = ctypes.c_void_p(rs.data_ptr()) if rs is not None else None
+        if a.scales is not None:
+            code = lib.trakhip_gemm_nt_split2(
+                ctypes.c_void_p(a.planes.data_ptr()), ctypes.c_void_p(a.scales.data_ptr()), M,
+                ctypes.c_void_p(b.planes.data_ptr()), ctypes.c_void_p(b.scales.data_ptr()), N, K,
+                ctypes.c_void_p(out.data_ptr()), _ld(out), float(alpha), float(beta), rs_ptr, ctypes.c_void_p(stream),
+            )
+        else:
+            code = lib.trakhip_gemm_nt_split(
+                ctypes.c_void_p(a.planes.data_ptr()), M, ctypes.c_void_p(b.planes.data_ptr()), N, K,
+                _STORE_DTYPES[a.dtype], ctypes.c_void_p(out.data_ptr()), _ld(out), float(alpha), float(beta),
+                rs_ptr, ctypes.c_void_p(stream),
+            )
     _lib.check(code)
     return out
 
@@ -273,12 +309,15 @@ def gemm_nt16(a, b, out=None, alpha=1.0, beta=0.0, row_scale=None):
     return out
 
 
-def matmul_nt(a, b, out=None, alpha=1.0, beta=0.0, row_scale=None):
+def matmul_nt(a, b, out=None, alpha=1.0, beta=0.0, row_scale=None, two_planes=False):
     """alpha * a @ b.T + beta * out with fp32 accuracy on the 16-bit matrix cores, whatever the operand
     types: two fp16 or two bf16 matrices that qualify are multiplied where they are (`gemm_nt16`),
-    other 16-bit pairs as single planes, anything else from fp32 splits (`gemm_nt_split`)."""
+    other 16-bit pairs as single planes, anything else from fp32 splits (`gemm_nt_split`; the exact
+    three-plane split, or the two-plane one of `split2_rows` when `two_planes` is set)."""
     if _nt16_ok(a, b):
         return gemm_nt16(a, b, out=out, alpha=alpha, beta=beta, row_scale=row_scale)
+    if two_planes and not (a.dtype == b.dtype and a.dtype in (torch.float16, torch.bfloat16)):
+        return gemm_nt_split(split2_rows(a), split2_rows(b), out=out, alpha=alpha, beta=beta, row_scale=row_scale)
     return gemm_nt_split(*split_pair(a, b), out=out, alpha=alpha, beta=beta, row_scale=row_scale)
 
 
@@ -297,10 +336,16 @@ def gram_split(a, out=None, alpha=1.0, beta=0.0):
     lib = _lib.load()
     with torch.cuda.device(a.device):
         stream = torch.cuda.current_stream(a.device).cuda_stream
-        code = lib.trakhip_gram_split(
-            ctypes.c_void_p(a.planes.data_ptr()), N, a.K, _STORE_DTYPES[a.dtype], ctypes.c_void_p(out.data_ptr()),
-            _ld(out), float(alpha), float(beta), ctypes.c_void_p(stream),
-        )
+        if a.scales is not None:
+            code = lib.trakhip_gram_split2(
+                ctypes.c_void_p(a.planes.data_ptr()), ctypes.c_void_p(a.scales.data_ptr()), N, a.K,
+                ctypes.c_void_p(out.data_ptr()), _ld(out), float(alpha), float(beta), ctypes.c_void_p(stream),
+            )
+        else:
+            code = lib.trakhip_gram_split(
+                ctypes.c_void_p(a.planes.data_ptr()), N, a.K, _STORE_DTYPES[a.dtype], ctypes.c_void_p(out.data_ptr()),
+                _ld(out), float(alpha), float(beta), ctypes.c_void_p(stream),
+            )
     _lib.check(code)
     return out
 
