@@ -20,6 +20,7 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include "short_k_tile.h"
 #include "trakhip_internal.h"
 
 namespace {
@@ -234,126 +235,23 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_nn_batched_kernel(const floa
 // MFMAs run back to back.  Needs 16-byte aligned rows and K a multiple of 8.
 // ROWS = 128: 2 x 2 waves of 64 x 64, 135 KB of LDS, one workgroup per CU.  ROWS = 32: 1 x 4 waves of
 // 32 x 32 for products with few rows of tiles (the panel: N = 128), four times as many workgroups.
-constexpr int kShortK = 128;
-constexpr int kShortStride = kShortK + 4;  // floats; 528-byte rows keep 16-byte reads conflict free
-
 template <int ROWS>
 __global__ __launch_bounds__(kThreads, 1) void gemm_nt_short_k_kernel(const float* __restrict__ A, uint64_t lda,
                                                                       const float* __restrict__ B, uint64_t ldb,
                                                                       float* __restrict__ C, uint64_t ldc, uint64_t M,
                                                                       uint64_t N, uint32_t K, float alpha, float beta,
                                                                       uint32_t tiles_n, uint32_t flags) {
-    constexpr int WM = ROWS >= 64 ? 2 : 1, WNV = 4 / WM;           // wave grid
-    constexpr int IT = ROWS / WM / 32, JT = BM / WNV / 32;          // 32 x 32 MFMA tiles per wave
-    __shared__ __attribute__((aligned(16))) float lds[(ROWS + BM) * kShortStride];
+    __shared__ __attribute__((aligned(16))) float lds[short_k::lds_floats<ROWS>()];
     // With kGemmLowerTilesOnly (square tiles only) the grid holds the lower-triangle tiles alone, numbered
     // row by row (a workgroup that only returns would still wait for a CU with this much LDS free).
     uint32_t tile_m, tile_n;
     if (ROWS == BM && (flags & trakhip::kGemmLowerTilesOnly)) {
-        tile_m = (uint32_t)((sqrtf(8.0f * (float)blockIdx.x + 1.0f) - 1.0f) * 0.5f);
-        while (tile_m * (tile_m + 1) / 2 > blockIdx.x) --tile_m;
-        while ((tile_m + 1) * (tile_m + 2) / 2 <= blockIdx.x) ++tile_m;
-        tile_n = blockIdx.x - tile_m * (tile_m + 1) / 2;
+        short_k::triangle_tile(blockIdx.x, tile_m, tile_n);
     } else {
         tile_m = blockIdx.x / tiles_n;
         tile_n = blockIdx.x % tiles_n;
     }
-    const uint64_t m0 = (uint64_t)tile_m * ROWS, n0 = (uint64_t)tile_n * BM;
-    const int tid = threadIdx.x;
-    const int wave = tid >> 6, lane = tid & 63;
-    const int wm = wave / WNV, wn = wave % WNV;
-    const int x = lane & 31, h = lane >> 5;
-
-    // rows x 32 float4 per operand, all loads in flight at once
-    constexpr int kPiecesA = ROWS * (kShortK / 4) / kThreads, kPiecesB = BM * (kShortK / 4) / kThreads;
-    float4 ra[kPiecesA], rb[kPiecesB];
-#pragma unroll
-    for (int i = 0; i < kPiecesA; ++i) {
-        const int id = tid + kThreads * i;
-        const uint32_t row = id >> 5, k4 = 4 * (id & 31);
-        ra[i] = (m0 + row < M && k4 < K) ? *reinterpret_cast<const float4*>(A + (m0 + row) * lda + k4)
-                                         : make_float4(0.f, 0.f, 0.f, 0.f);
-    }
-#pragma unroll
-    for (int i = 0; i < kPiecesB; ++i) {
-        const int id = tid + kThreads * i;
-        const uint32_t row = id >> 5, k4 = 4 * (id & 31);
-        rb[i] = (n0 + row < N && k4 < K) ? *reinterpret_cast<const float4*>(B + (n0 + row) * ldb + k4)
-                                         : make_float4(0.f, 0.f, 0.f, 0.f);
-    }
-    float* as = lds;
-    float* bs = lds + ROWS * kShortStride;
-#pragma unroll
-    for (int i = 0; i < kPiecesA; ++i) {
-        const int id = tid + kThreads * i;
-        *reinterpret_cast<float4*>(as + (id >> 5) * kShortStride + 4 * (id & 31)) = ra[i];
-    }
-#pragma unroll
-    for (int i = 0; i < kPiecesB; ++i) {
-        const int id = tid + kThreads * i;
-        *reinterpret_cast<float4*>(bs + (id >> 5) * kShortStride + 4 * (id & 31)) = rb[i];
-    }
-    __syncthreads();
-
-    const uint64_t row_base = m0 + wm * (32 * IT) + 4 * h, col_base = n0 + wn * (32 * JT) + x;
-    floatx16 acc[IT][JT];
-#pragma unroll
-    for (int i = 0; i < IT; ++i)
-#pragma unroll
-        for (int j = 0; j < JT; ++j)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
-    // the old values of C are fetched here, so that their latency passes under the MFMAs
-    floatx16 prev[IT][JT];
-    if (beta != 0.0f) {
-#pragma unroll
-        for (int i = 0; i < IT; ++i)
-#pragma unroll
-            for (int j = 0; j < JT; ++j)
-#pragma unroll
-                for (int r = 0; r < 16; ++r) {
-                    const uint64_t row = row_base + 32 * i + 8 * (r >> 2) + (r & 3);
-                    const uint64_t col = col_base + 32 * j;
-                    prev[i][j][r] = (row < M && col < N) ? C[row * ldc + col] : 0.f;
-                }
-    }
-    // lane half h takes k = 8 s + 4 h + t for the t-th MFMA of sub-step s, as in the general kernel
-    for (uint32_t s = 0; s < K / 8; ++s) {
-        float4 fa[IT], fb[JT];
-#pragma unroll
-        for (int i = 0; i < IT; ++i)
-            fa[i] = *reinterpret_cast<const float4*>(as + (wm * (32 * IT) + 32 * i + x) * kShortStride + 8 * s + 4 * h);
-#pragma unroll
-        for (int j = 0; j < JT; ++j)
-            fb[j] = *reinterpret_cast<const float4*>(bs + (wn * (32 * JT) + 32 * j + x) * kShortStride + 8 * s + 4 * h);
-#pragma unroll
-        for (int t = 0; t < 4; ++t)
-#pragma unroll
-            for (int i = 0; i < IT; ++i)
-#pragma unroll
-                for (int j = 0; j < JT; ++j) {
-                    const float av = t == 0 ? fa[i].x : (t == 1 ? fa[i].y : (t == 2 ? fa[i].z : fa[i].w));
-                    const float bv = t == 0 ? fb[j].x : (t == 1 ? fb[j].y : (t == 2 ? fb[j].z : fb[j].w));
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(av, bv, acc[i][j], 0, 0, 0);
-                }
-    }
-#pragma unroll
-    for (int i = 0; i < IT; ++i) {
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-            const uint64_t row = row_base + 32 * i + 8 * (r >> 2) + (r & 3);
-            if (row >= M) continue;
-#pragma unroll
-            for (int j = 0; j < JT; ++j) {
-                const uint64_t col = col_base + 32 * j;
-                if (col >= N) continue;
-                float* c = C + row * ldc + col;
-                float v = alpha * acc[i][j][r];
-                if (beta != 0.0f) v += beta * prev[i][j][r];
-                *c = v;
-            }
-        }
-    }
+    short_k::tile<ROWS>(A, lda, B, ldb, C, ldc, M, N, K, alpha, beta, tile_m, tile_n, lds);
 }
 
 template <bool AK, bool BK, int WN>
@@ -397,7 +295,7 @@ int gemm_nt(const float* A, uint64_t lda, const float* B, uint64_t ldb, float* C
             uint64_t N, uint64_t K, float alpha, float beta, const float* row_scale, hipStream_t s, uint32_t flags) {
     const bool aligned = A && B && (reinterpret_cast<uintptr_t>(A) % 16 == 0) &&
                          (reinterpret_cast<uintptr_t>(B) % 16 == 0) && (lda % 4 == 0) && (ldb % 4 == 0);
-    if (M && N && C && aligned && !row_scale && K >= 8 && K <= kShortK && K % 8 == 0 && lda >= K && ldb >= K &&
+    if (M && N && C && aligned && !row_scale && K >= 8 && K <= short_k::kMaxK && K % 8 == 0 && lda >= K && ldb >= K &&
         ldc >= N) {
         const uint64_t tm = (M + BM - 1) / BM, tn = (N + BM - 1) / BM;
         // Lower tiles only: a square tile grid is launched as its triangle; otherwise the flag is dropped

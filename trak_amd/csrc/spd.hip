@@ -8,7 +8,8 @@
 //   1. W = A + lambda I, padded with an identity block up to a multiple of 128;
 //   2. for every 128-block column j:  one workgroup factors the diagonal block in LDS
 //      (L_jj) and inverts it; the panel below it is  W[j+1:, j] * L_jj^-T  and the trailing
-//      matrix gets  W -= panel * panel^T   (both MFMA GEMMs from gemm.hip);
+//      matrix gets  W -= panel * panel^T   (MFMA products; the trailing update and the next
+//      diagonal block share one launch, see spd_step_kernel);
 //   3. L^-1 by recursive halving: inv([[A,0],[B,C]]) = [[A^-1,0],[-C^-1 B A^-1, C^-1]]
 //      (two GEMMs per node of the recursion tree);
 //   4. inverse = L^-T L^-1 (one GEMM), then the mean of |.| by a two-stage reduction in a
@@ -18,6 +19,7 @@
 
 #include <vector>
 
+#include "short_k_tile.h"
 #include "trakhip_internal.h"
 
 namespace {
@@ -162,13 +164,18 @@ __device__ __forceinline__ floatx16 tile_zero() {
     return acc;
 }
 
-__global__ __launch_bounds__(256) void spd_diag_kernel(const float* __restrict__ W, uint64_t ldw,
-                                                       float* __restrict__ Lout, float* __restrict__ Linv_out,
-                                                       uint64_t ldl, int32_t block_index,
-                                                       int32_t* __restrict__ status) {
-    __shared__ float As[NB * kPitch];           // the block, overwritten by its factor
-    __shared__ float Xs[NB * kPitch];           // the inverse of the factor
-    __shared__ float Ts[2 * kSub * kTPitch];    // B A^-1 of the halving steps
+constexpr int kDiagLdsFloats = 2 * NB * kPitch + 2 * kSub * kTPitch;  // 148 736 bytes
+
+// `panel`, when not null, is the 128 x 128 block of the factor to the left of this diagonal block
+// (row pitch ldp) whose contribution has not been taken off W yet: the block that is factored is
+// W - panel panel^T (its lower triangle).
+__device__ __forceinline__ void diag_block(const float* __restrict__ W, uint64_t ldw, float* __restrict__ Lout,
+                                           float* __restrict__ Linv_out, uint64_t ldl, int32_t block_index,
+                                           int32_t* __restrict__ status, const float* __restrict__ panel,
+                                           uint64_t ldp, float* __restrict__ lds) {
+    float* As = lds;                        // the block, overwritten by its factor
+    float* Xs = As + NB * kPitch;           // the inverse of the factor
+    float* Ts = Xs + NB * kPitch;           // B A^-1 of the halving steps
     const int tid = threadIdx.x;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;  // wave index in a scalar register
 
@@ -191,9 +198,36 @@ __global__ __launch_bounds__(256) void spd_diag_kernel(const float* __restrict__
             x[0] = x[1] = x[2] = x[3] = 0.0f;
         }
     }
+    constexpr int kBlocks = NB / kSub;
+    if (panel) {
+        // Xs borrows the panel block; the ten 32 x 32 sub-blocks on or under the diagonal get
+        // A -= P P^T (what is left above the diagonal is never read); then Xs is cleared again
+        const int r0 = tid >> 5, c = 4 * (tid & 31);
+        float4 v[16];
+#pragma unroll
+        for (int i = 0; i < 16; ++i) v[i] = *reinterpret_cast<const float4*>(panel + (uint64_t)(r0 + 8 * i) * ldp + c);
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            float* x = Xs + (r0 + 8 * i) * kPitch + c;
+            x[0] = v[i].x, x[1] = v[i].y, x[2] = v[i].z, x[3] = v[i].w;
+        }
+        __syncthreads();
+        for (int t = wave; t < kBlocks * (kBlocks + 1) / 2; t += 4) {
+            const int ti = t < 1 ? 0 : (t < 3 ? 1 : (t < 6 ? 2 : 3)), tj = t - ti * (ti + 1) / 2;
+            float* tile = As + kSub * ti * kPitch + kSub * tj;
+            const floatx16 acc = tile_product<true>(Xs + kSub * ti * kPitch, kPitch, Xs + kSub * tj * kPitch, kPitch, NB,
+                                                    -1.0f, tile_load(tile, kPitch, lane), lane);
+            tile_store(tile, kPitch, acc, lane);
+        }
+        __syncthreads();
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            float* x = Xs + (r0 + 8 * i) * kPitch + c;
+            x[0] = x[1] = x[2] = x[3] = 0.0f;
+        }
+    }
     __syncthreads();
 
-    constexpr int kBlocks = NB / kSub;
     for (int p = 0; p < kBlocks; ++p) {
         const int base = kSub * p;
         if (wave == 0) factor_sub_block(As, Xs, base, lane, block_index * NB + base, status);
@@ -268,6 +302,36 @@ __global__ __launch_bounds__(256) void spd_diag_kernel(const float* __restrict__
             *reinterpret_cast<float4*>(Lout + (uint64_t)r * ldl + c) = l;
             *reinterpret_cast<float4*>(Linv_out + (uint64_t)r * ldl + c) = li;
         }
+    }
+}
+
+__global__ __launch_bounds__(256) void spd_diag_kernel(const float* __restrict__ W, uint64_t ldw,
+                                                       float* __restrict__ Lout, float* __restrict__ Linv_out,
+                                                       uint64_t ldl, int32_t block_index,
+                                                       int32_t* __restrict__ status) {
+    __shared__ __attribute__((aligned(16))) float lds[kDiagLdsFloats];
+    diag_block(W, ldw, Lout, Linv_out, ldl, block_index, status, nullptr, 0, lds);
+}
+
+// One step of the factorization in one launch, after the panel below diagonal block j is known:
+// workgroup 0 takes the next diagonal block (j+1, j+1) - its own trailing update, then factor and
+// inverse - while workgroups 1 .. T-1 apply the trailing update W -= panel panel^T to the other
+// lower-triangle tiles (tile numbers in the triangle's row-by-row order; number 0 is that diagonal
+// block).  Nothing in the launch depends on anything else in it, and the 31 us of the sequential
+// diagonal work no longer sit between two launches but beside the trailing update.
+//   Wt    trailing matrix, block (j+1, j+1) at its origin;  panel  L[j+1:, j] (rows x 128, pitch np)
+__global__ __launch_bounds__(256, 1) void spd_step_kernel(float* __restrict__ Wt, const float* __restrict__ panel,
+                                                          uint64_t np, uint64_t rows, float* __restrict__ Lout,
+                                                          float* __restrict__ Linv_out, int32_t block_index,
+                                                          int32_t* __restrict__ status) {
+    constexpr int kLds = kDiagLdsFloats > short_k::lds_floats<NB>() ? kDiagLdsFloats : short_k::lds_floats<NB>();
+    __shared__ __attribute__((aligned(16))) float lds[kLds];
+    if (blockIdx.x == 0) {
+        diag_block(Wt, np, Lout, Linv_out, np, block_index, status, panel, np, lds);
+    } else {
+        uint32_t tile_m, tile_n;
+        short_k::triangle_tile(blockIdx.x, tile_m, tile_n);
+        short_k::tile<NB>(panel, np, panel, np, Wt, np, rows, rows, NB, -1.0f, 1.0f, tile_m, tile_n, lds);
     }
 }
 
@@ -412,22 +476,33 @@ int spd_inverse(const float* A, uint64_t lda, float lambda, float* inv, uint64_t
                        np, W, L, Li, status);
     if (hipGetLastError() != hipSuccess) return TRAKHIP_ERR_LAUNCH;
 
-    for (uint64_t j = 0; j < nblk; ++j) {
+    // Diagonal block 0 alone; then per block column j: the panel below it, and one launch that holds both
+    // the trailing update and the next diagonal block (spd_step_kernel).  Trailing updates of more than
+    // 512 tiles (n > 4096) go through the general product, with the diagonal block in a launch of its own.
+    hipLaunchKernelGGL(spd_diag_kernel, dim3(1), dim3(256), 0, s, W, np, L, Li, np, 0, status);
+    if (hipGetLastError() != hipSuccess) return TRAKHIP_ERR_LAUNCH;
+    for (uint64_t j = 0; j + 1 < nblk; ++j) {
         const uint64_t off = j * NB * np + j * NB;
-        hipLaunchKernelGGL(spd_diag_kernel, dim3(1), dim3(256), 0, s, W + off, np, L + off, Li + off, np,
-                           (int32_t)j, status);
-        if (hipGetLastError() != hipSuccess) return TRAKHIP_ERR_LAUNCH;
-        if (j + 1 == nblk) break;
-        const uint64_t rows = np - (j + 1) * NB;
+        const uint64_t rows = np - (j + 1) * NB, blocks = rows / NB;
         const uint64_t below = (j + 1) * NB * np + j * NB;
+        const uint64_t tr = (j + 1) * NB * np + (j + 1) * NB;
         // panel = W[j+1:, j] * (L_jj^-1)^T
         int e = gemm_nt(W + below, np, Li + off, np, L + below, np, rows, NB, NB, 1.0f, 0.0f, nullptr, s);
         if (e) return e;
-        // trailing matrix -= panel * panel^T
-        const uint64_t tr = (j + 1) * NB * np + (j + 1) * NB;
+        const uint64_t tiles = blocks * (blocks + 1) / 2;
+        if (tiles <= 512) {
+            hipLaunchKernelGGL(spd_step_kernel, dim3((uint32_t)tiles), dim3(256), 0, s, W + tr, L + below, np, rows,
+                               L + tr, Li + tr, (int32_t)(j + 1), status);
+            if (hipGetLastError() != hipSuccess) return TRAKHIP_ERR_LAUNCH;
+            continue;
+        }
+        // trailing matrix -= panel * panel^T (only the lower triangle of W is ever read)
         e = gemm_nt(L + below, np, L + below, np, W + tr, np, rows, rows, NB, -1.0f, 1.0f, nullptr, s,
-                    kGemmLowerTilesOnly);  // only the lower triangle of W is ever read
+                    kGemmLowerTilesOnly);
         if (e) return e;
+        hipLaunchKernelGGL(spd_diag_kernel, dim3(1), dim3(256), 0, s, W + tr, np, L + tr, Li + tr, np,
+                           (int32_t)(j + 1), status);
+        if (hipGetLastError() != hipSuccess) return TRAKHIP_ERR_LAUNCH;
     }
 
     Ctx c = {W, L, Li, np, s};
