@@ -8,6 +8,8 @@ import pytest
 import torch
 
 from oracle import score_oracle as so
+import trak_amd.score_computers as score_computers_module
+import trak_amd.utils as utils_module
 from trak_amd import BasicScoreComputer, get_matrix_mult
 from trak_amd.utils import (
     gemm_nt,
@@ -487,3 +489,52 @@ def test_score_computer_half_precision_flow(gpu):
     sc.get_scores(feats, Xt.to(gpu), accumulator=acc)
     want = feats.double().cpu().numpy() @ Xt.double().numpy().T
     assert rel_max(acc.cpu().numpy(), want) < gemm_tol(k)                    # exact products, fp32 sums
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+@pytest.mark.parametrize("where", ["cpu", "gpu"])
+def test_blockwise_product_collects_on_the_host(gpu, dtype, where):
+    """The host-collected block product (results too large for the device; trak/utils.py:135-245): ragged
+    blocks in both directions, operands on either side, a CPU result of the target type, accumulation."""
+    gen = torch.Generator(device="cpu").manual_seed(11)
+    N, M, K = 300, 150, 128
+    f, t = torch.randn(N, K, generator=gen).to(dtype), torch.randn(M, K, generator=gen).to(dtype)
+    want = f.double().numpy() @ t.double().numpy().T
+    src_f, src_t = (f, t) if where == "cpu" else (f.to(gpu), t.to(gpu))
+    tol = gemm_tol(K) if dtype == torch.float32 else 1e-3                      # the result is rounded to fp16
+    got = utils_module.get_matrix_mult_blockwise(src_f, src_t, dtype, bs=64, block_bytes=64 * 64 * 4)
+    assert got.device.type == "cpu" and got.dtype == dtype and got.shape == (N, M)
+    assert rel_max(got.numpy(), want) < tol
+    # the same through the public entry point, and one block when it fits
+    assert torch.equal(get_matrix_mult(src_f, src_t, use_blockwise=True, batch_size=8096), utils_module.get_matrix_mult_blockwise(src_f, src_t))
+    acc = torch.ones(N, M)
+    utils_module.get_matrix_mult_blockwise(src_f, src_t, out=acc, accumulate=True, bs=64, block_bytes=64 * 64 * 4)
+    utils_module.get_matrix_mult_blockwise(src_f, src_t, out=acc, accumulate=True, bs=100, block_bytes=100 * 100 * 4)
+    assert rel_max(acc.numpy(), 1.0 + 2.0 * want) < tol + 1e-6
+
+
+def test_get_scores_goes_blockwise_when_the_result_does_not_fit(gpu, monkeypatch):
+    gen = torch.Generator(device="cpu").manual_seed(12)
+    N, M, k = 500, 70, 256
+    feats, Xt = torch.randn(N, k, generator=gen) / 16, torch.randn(M, k, generator=gen) / 16
+    want = feats.double().numpy() @ Xt.double().numpy().T
+    calls = []
+    real = utils_module.get_matrix_mult_blockwise
+
+    def spy(*args, **kwargs):
+        calls.append(1)
+        return real(*args, bs=64, block_bytes=128 * 64 * 4, **kwargs)
+
+    monkeypatch.setattr(score_computers_module, "output_fits_on_device", lambda *a, **k: False)
+    monkeypatch.setattr(score_computers_module, "get_matrix_mult_blockwise", spy)
+    for gemm in ("split", "split2", "fp32"):
+        sc = BasicScoreComputer(dtype=torch.float32, device="cuda:0", gemm=gemm)
+        acc = torch.zeros(N, M)
+        sc.get_scores(feats.to(gpu), Xt.to(gpu), accumulator=acc)
+        sc.get_scores(feats, Xt, accumulator=acc)                                 # host-resident operands
+        assert rel_max(acc.numpy(), 2 * want) < 1e-5
+    assert len(calls) == 6
+    # a device accumulator never takes this path
+    dev_acc = torch.zeros(N, M, device=gpu)
+    BasicScoreComputer(dtype=torch.float32, device="cuda:0").get_scores(feats.to(gpu), Xt.to(gpu), accumulator=dev_acc)
+    assert len(calls) == 6 and rel_max(dev_acc.cpu().numpy(), want) < 1e-5

@@ -17,8 +17,10 @@ from .utils import (
     gemm_nt16,
     gemm_nt_split,
     gemm_tn,
+    get_matrix_mult_blockwise,
     gram_split,
     matmul_nt,
+    output_fits_on_device,
     scores_finalize,
     spd_inverse,
     split2_rows,
@@ -147,6 +149,11 @@ class BasicScoreComputer(AbstractScoreComputer):
             # accumulator on the GPU: the sum over checkpoints happens in the GEMM epilogue and the
             # [N, M] matrix never crosses PCIe per checkpoint (trak/traker.py:641-668 moves it each time)
             self._matmul_nt(f, t, out=accumulator, beta=1.0)
+            return
+        if not accumulator.is_cuda and not output_fits_on_device(train_dim, target_dim, self._dev):
+            # too large for the device: block by block into the host accumulator (trak/utils.py:135-245)
+            get_matrix_mult_blockwise(f, t, out=accumulator, accumulate=True,
+                                      product=lambda a, b, o: self._matmul_nt(a, b, out=o))
             return
         scores = self._matmul_nt(f, t)
         if accumulator.is_cuda:

@@ -436,15 +436,109 @@ def scores_finalize(acc, divisor, row_factor, out):
     return out
 
 
-def get_matrix_mult(features, target_grads, target_dtype=None, batch_size=8096, use_blockwise=False):
-    """features @ target_grads.T (trak/utils.py:248-294).  On the GPU this is one GEMM of fp32 accuracy
-    on the matrix cores (operands split into bf16 terms, see gemm_nt_split);
-    CPU inputs take torch's matmul as in the reference (trak/utils.py:128-132).  The reference's
-    blockwise host-staged variant exists to fit small GPU memories; `use_blockwise` and
-    `batch_size` are accepted for signature compatibility and ignored."""
+def output_fits_on_device(n_rows, n_cols, device, reserve=0.25):
+    """Whether an fp32 [n_rows, n_cols] result can be held on `device` next to what is there, keeping
+    `reserve` of the free memory for operands in their product format."""
+    free, _ = torch.cuda.mem_get_info(device)
+    return n_rows * n_cols * 4 <= free * (1.0 - reserve)
+
+
+def _block_extents(total, size):
+    return [(lo, min(lo + size, total)) for lo in range(0, total, size)]
+
+
+def get_matrix_mult_blockwise(features, target_grads, target_dtype=None, bs=8096, out=None, accumulate=False,
+                              product=None, block_bytes=1 << 30):
+    """features @ target_grads.T computed block by block on the GPU and collected on the host, for
+    results that do not fit in device memory (trak/utils.py:135-245).  Operands may live on the host
+    or on the device; the result is a CPU tensor (`out`, when given: written, or added to with
+    `accumulate`).  Two device blocks and two page-locked host blocks: while block i is copied out and
+    stored by the host, block i + 1 is being multiplied.  `bs` is the least block edge (the reference's
+    meaning); blocks are grown to about `block_bytes` of fp32 results, since there is no small device
+    memory to fit here.  `product(a, b, out)` overrides the product used for a block."""
     if target_dtype is None:
         target_dtype = features.dtype
+    if product is None:
+        product = lambda a, b, o: matmul_nt(a, b, out=o)  # noqa: E731
+    N, M = features.shape[0], target_grads.shape[0]
+    if features.is_cuda:
+        dev = features.device
+    elif target_grads.is_cuda:
+        dev = target_grads.device
+    else:
+        dev = torch.device("cuda", torch.cuda.current_device())
+    final = out if out is not None else torch.empty((N, M), dtype=target_dtype, device="cpu")
+    if final.device.type != "cpu" or tuple(final.shape) != (N, M):
+        raise RuntimeError("out must be a CPU tensor of shape [features rows, target rows]")
+    if N == 0 or M == 0:
+        return final
+    bs, elements = max(int(bs), 1), max(int(block_bytes) // 4, 1)
+    cb = min(M, max(bs, elements // bs))
+    rb = min(N, max(bs, elements // cb))
+    row_blocks, col_blocks = _block_extents(N, rb), _block_extents(M, cb)
+    with torch.cuda.device(dev):
+        main = torch.cuda.current_stream(dev)
+        copy_stream = torch.cuda.Stream(device=dev)
+        dbuf = [torch.empty((rb, cb), dtype=torch.float32, device=dev) for _ in range(2)]
+        pbuf = [torch.empty((rb, cb), dtype=final.dtype, pin_memory=True) for _ in range(2)]
+        computed = [torch.cuda.Event() for _ in range(2)]
+        copied = [None, None]
+        targets_on_device = {}
+        pending = None  # (event, pinned view, destination view) of the block before
+
+        def consume(p):
+            event, src, dst = p
+            event.synchronize()
+            if accumulate:
+                dst += src
+            else:
+                dst.copy_(src)
+
+        idx = 0
+        for r0, r1 in row_blocks:
+            f = features[r0:r1].to(dev, non_blocking=True)
+            for c0, c1 in col_blocks:
+                if len(col_blocks) == 1:
+                    t = targets_on_device.setdefault(0, target_grads.to(dev, non_blocking=True))
+                else:
+                    t = target_grads[c0:c1].to(dev, non_blocking=True)
+                slot = idx % 2
+                if copied[slot] is not None:
+                    main.wait_event(copied[slot])  # the copy that read this device block two blocks ago
+                d = dbuf[slot][: r1 - r0, : c1 - c0]
+                product(f, t, d)
+                converted = d if final.dtype == torch.float32 else d.to(final.dtype)
+                computed[slot].record(main)
+                # (the host finished with pinned block `slot` when it stored block idx - 2, one iteration ago)
+                with torch.cuda.stream(copy_stream):
+                    copy_stream.wait_event(computed[slot])
+                    p = pbuf[slot][: r1 - r0, : c1 - c0]
+                    p.copy_(converted, non_blocking=True)
+                    converted.record_stream(copy_stream)
+                    ev = torch.cuda.Event()
+                    ev.record(copy_stream)
+                    copied[slot] = ev
+                if pending is not None:
+                    consume(pending)  # overlaps with the product and the copy just queued
+                pending = (ev, p, final[r0:r1, c0:c1])
+                idx += 1
+        consume(pending)
+    return final
+
+
+def get_matrix_mult(features, target_grads, target_dtype=None, batch_size=8096, use_blockwise=False):
+    """features @ target_grads.T (trak/utils.py:248-294).  On the GPU this is one GEMM of fp32 accuracy
+    on the matrix cores (see `matmul_nt`); CPU inputs take torch's matmul as in the reference
+    (trak/utils.py:128-132).  A result that does not fit in device memory, or `use_blockwise`, goes
+    block by block to the host (`get_matrix_mult_blockwise`; a CPU tensor comes back, as in the
+    reference)."""
+    if target_dtype is None:
+        target_dtype = features.dtype
+    if use_blockwise:
+        return get_matrix_mult_blockwise(features, target_grads, target_dtype, batch_size)
     if features.device.type == "cpu":
         return (features @ target_grads.t()).clone().to(target_dtype)
+    if not output_fits_on_device(features.shape[0], target_grads.shape[0], features.device):
+        return get_matrix_mult_blockwise(features, target_grads, target_dtype, batch_size)
     out = matmul_nt(features, target_grads.to(features.device))
     return out.to(target_dtype)
