@@ -12,7 +12,6 @@ import torch
 from torch import Tensor
 
 from .utils import (
-    _nt16_ok,
     gemm_nt,
     gemm_nt16,
     gemm_nt_split,
@@ -20,6 +19,7 @@ from .utils import (
     get_matrix_mult_blockwise,
     gram_split,
     matmul_nt,
+    nt16_ok,
     output_fits_on_device,
     scores_finalize,
     spd_inverse,
@@ -123,7 +123,7 @@ class BasicScoreComputer(AbstractScoreComputer):
             # the inverse is symmetric, so block @ inv == block @ inv^T
             if self.gemm != "fp32":
                 block = block.to(self._dev)
-                if half and _nt16_ok(block, xtx_inv):
+                if half and nt16_ok(block, xtx_inv):
                     gemm_nt16(block, xtx_inv, out=result[start:end])
                 else:
                     if inv_split is None:

@@ -266,7 +266,7 @@ def gemm_nt_split(a, b, out=None, alpha=1.0, beta=0.0, row_scale=None):
     return out
 
 
-def _nt16_ok(a, b):
+def nt16_ok(a, b):
     """Whether `gemm_nt16` can read these operands where they are."""
     if a.dtype != b.dtype or a.dtype not in (torch.float16, torch.bfloat16):
         return False
@@ -284,7 +284,7 @@ def gemm_nt16(a, b, out=None, alpha=1.0, beta=0.0, row_scale=None):
     """out[M, N] (fp32) = alpha * a @ b.T + beta * out (rows optionally scaled) for fp16 or bf16 CUDA
     matrices a [M, K], b [N, K] read in place: K a multiple of 64, rows 16-byte aligned (see
     `matmul_nt` for the general case).  Exact products, fp32 accumulation."""
-    if not _nt16_ok(a, b):
+    if not nt16_ok(a, b):
         raise RuntimeError("gemm_nt16 needs two fp16 or two bf16 CUDA matrices with K % 64 == 0 and 16-byte aligned rows")
     M, N, K = a.shape[0], b.shape[0], a.shape[1]
     if out is None:
@@ -314,7 +314,7 @@ def matmul_nt(a, b, out=None, alpha=1.0, beta=0.0, row_scale=None, two_planes=Fa
     types: two fp16 or two bf16 matrices that qualify are multiplied where they are (`gemm_nt16`),
     other 16-bit pairs as single planes, anything else from fp32 splits (`gemm_nt_split`; the exact
     three-plane split, or the two-plane one of `split2_rows` when `two_planes` is set)."""
-    if _nt16_ok(a, b):
+    if nt16_ok(a, b):
         return gemm_nt16(a, b, out=out, alpha=alpha, beta=beta, row_scale=row_scale)
     if two_planes and not (a.dtype == b.dtype and a.dtype in (torch.float16, torch.bfloat16)):
         return gemm_nt_split(split2_rows(a), split2_rows(b), out=out, alpha=alpha, beta=beta, row_scale=row_scale)
