@@ -153,7 +153,14 @@ int trakhip_gemm_tn(const float* A_dev, uint64_t lda, const float* B_dev, uint64
  *   trakhip_gram_split             C[N, N] = alpha * A * A^T + beta * C: only the tiles that touch
  *                                  the lower triangle are computed, then the strict upper triangle
  *                                  is overwritten with the mirror image, so C is exactly
- *                                  symmetric; with beta != 0, C must have been produced this way
+ *                                  symmetric; with beta != 0, C must have been produced this way.
+ *                                  workspace_dev (may be NULL): trakhip_gram_split_workspace bytes,
+ *                                  16-byte aligned.  A product with few tiles (N up to 4608) leaves
+ *                                  CUs idle; with the workspace its k range is shared out over three
+ *                                  sets of workgroups whose sums are added in a fixed order
+ *   trakhip_gram_split_workspace   bytes that trakhip_gram_split (two_planes == 0) or
+ *                                  trakhip_gram_split2 (two_planes != 0) can use for these sizes; 0
+ *                                  when they would not use any
  * Stand in, like trakhip_gemm_nt / trakhip_gemm_tn, for trak/score_computers.py:153 (the Gram
  * product, A = the planes of block^T), :176 and trak/utils.py:131. */
 size_t trakhip_split_bytes(uint64_t rows, uint64_t K, int src_dtype);
@@ -162,8 +169,9 @@ int trakhip_split_rows(const void* src_dev, int src_dtype, uint64_t ld, uint64_t
 int trakhip_gemm_nt_split(const void* A_planes_dev, uint64_t M, const void* B_planes_dev, uint64_t N, uint64_t K,
                           int src_dtype, float* C_dev, uint64_t ldc, float alpha, float beta,
                           const float* row_scale_dev, void* stream);
+size_t trakhip_gram_split_workspace(uint64_t N, uint64_t K, int src_dtype, int two_planes);
 int trakhip_gram_split(const void* A_planes_dev, uint64_t N, uint64_t K, int src_dtype, float* C_dev, uint64_t ldc,
-                       float alpha, float beta, void* stream);
+                       float alpha, float beta, void* workspace_dev, size_t workspace_bytes, void* stream);
 
 /* An opt-in cheaper form of the split products for fp32 operands: two fp16 planes per operand and
  * three fp16 MFMAs per k step instead of three bf16 planes and six MFMAs (about 1.75 times the speed).
@@ -187,7 +195,8 @@ int trakhip_gemm_nt_split2(const void* A_planes_dev, const float* A_scales_dev, 
                            const float* B_scales_dev, uint64_t N, uint64_t K, float* C_dev, uint64_t ldc, float alpha,
                            float beta, const float* row_scale_dev, void* stream);
 int trakhip_gram_split2(const void* A_planes_dev, const float* A_scales_dev, uint64_t N, uint64_t K, float* C_dev,
-                        uint64_t ldc, float alpha, float beta, void* stream);
+                        uint64_t ldc, float alpha, float beta, void* workspace_dev, size_t workspace_bytes,
+                        void* stream);
 
 /* C[M, N] (fp32) = alpha * A[M, K] * B[N, K]^T + beta * C, row i *= row_scale[i], for fp16 or bf16
  * operands read where they are: no planes, no extra pass.  For the two products of a TRAKer that

@@ -154,8 +154,11 @@ def test_split2_entry_points_validate_before_touching_the_device():
     assert mm(a=None) == -5 and mm(b=None) == -5 and mm(c=None) == -5
     assert mm(a=ctypes.c_void_p(4104)) == -7 and mm(c=ctypes.c_void_p(4098)) == -7
     gr = lambda **kw: lib.trakhip_gram_split2(kw.get("a", p), kw.get("sa", p), kw.get("N", 8), kw.get("K", 16),
-                                              kw.get("c", p), kw.get("ldc", 8), 1.0, 0.0, None)
+                                              kw.get("c", p), kw.get("ldc", 8), 1.0, 0.0, kw.get("ws", None),
+                                              kw.get("wsb", 0), None)
     assert gr(N=0) == 0 and gr(sa=None) == -5 and gr(a=None) == -5 and gr(ldc=7) == -2
+    # with a workspace the k range is shared out when there is enough of it: same validation
+    assert gr(K=4096, N=300, ws=p, wsb=1 << 30, ldc=299) == -2 and gr(K=4096, N=300, ws=p, wsb=1 << 30, c=None) == -5
 
 
 def test_gemm_nt16_validates_before_touching_the_device():
@@ -202,5 +205,14 @@ def test_split_gemm_entry_points_validate_before_touching_the_device():
     assert mm(a=None) == -5 and mm(b=None) == -5 and mm(c=None) == -5
     assert mm(a=ctypes.c_void_p(4104)) == -7 and mm(c=ctypes.c_void_p(4098)) == -7
     gr = lambda **kw: lib.trakhip_gram_split(kw.get("a", p), kw.get("N", 8), kw.get("K", 16), kw.get("dt", F32),
-                                             kw.get("c", p), kw.get("ldc", 8), 1.0, 0.0, None)
+                                             kw.get("c", p), kw.get("ldc", 8), 1.0, 0.0, kw.get("ws", None),
+                                             kw.get("wsb", 0), None)
     assert gr(N=0) == 0 and gr(dt=5) == -3 and gr(ldc=7) == -2 and gr(a=None) == -5
+    # scratch for sharing the k range of a product with few tiles: three N x N fp32 matrices, or none
+    ws = lib.trakhip_gram_split_workspace
+    assert ws(4096, 50_000, F32, 0) == 3 * 4096 * 4096 * 4 and ws(4096, 50_000, F16, 0) == 3 * 4096 * 4096 * 4
+    assert ws(4096, 50_000, F32, 1) == 3 * 4096 * 4096 * 4
+    assert ws(8192, 50_000, F32, 0) == 0            # 528 lower tiles keep every CU busy as they are
+    assert ws(4096, 256, F32, 0) == 0 and ws(4096, 1024, F16, 0) == 0      # too few k steps to share out
+    assert ws(0, 5, F32, 0) == 0 and ws(5, 0, F32, 0) == 0 and ws(5, 5, 9, 0) == 0
+    assert gr(K=4096, N=300, ws=p, wsb=1 << 30, ldc=299) == -2 and gr(K=4096, N=300, ws=p, wsb=1 << 30, c=None) == -5

@@ -64,7 +64,9 @@ def load():
     lib.trakhip_split_rows.restype = i32
     lib.trakhip_gemm_nt_split.argtypes = [vp, u64, vp, u64, u64, i32, vp, u64, f32, f32, vp, vp]
     lib.trakhip_gemm_nt_split.restype = i32
-    lib.trakhip_gram_split.argtypes = [vp, u64, u64, i32, vp, u64, f32, f32, vp]
+    lib.trakhip_gram_split_workspace.argtypes = [u64, u64, i32, i32]
+    lib.trakhip_gram_split_workspace.restype = sz
+    lib.trakhip_gram_split.argtypes = [vp, u64, u64, i32, vp, u64, f32, f32, vp, sz, vp]
     lib.trakhip_gram_split.restype = i32
     lib.trakhip_split2_bytes.argtypes = [u64, u64]
     lib.trakhip_split2_bytes.restype = sz
@@ -72,7 +74,7 @@ def load():
     lib.trakhip_split2_rows.restype = i32
     lib.trakhip_gemm_nt_split2.argtypes = [vp, vp, u64, vp, vp, u64, u64, vp, u64, f32, f32, vp, vp]
     lib.trakhip_gemm_nt_split2.restype = i32
-    lib.trakhip_gram_split2.argtypes = [vp, vp, u64, u64, vp, u64, f32, f32, vp]
+    lib.trakhip_gram_split2.argtypes = [vp, vp, u64, u64, vp, u64, f32, f32, vp, sz, vp]
     lib.trakhip_gram_split2.restype = i32
     lib.trakhip_gemm_nt16.argtypes = [vp, u64, vp, u64, i32, vp, u64, u64, u64, u64, f32, f32, vp, vp]
     lib.trakhip_gemm_nt16.restype = i32

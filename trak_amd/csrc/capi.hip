@@ -107,9 +107,14 @@ int trakhip_gemm_nt_split(const void* A_planes_dev, uint64_t M, const void* B_pl
                                   static_cast<hipStream_t>(stream));
 }
 
+size_t trakhip_gram_split_workspace(uint64_t N, uint64_t K, int dtype, int two_planes) {
+    return trakhip::gram_split_workspace_bytes(N, K, dtype, two_planes);
+}
+
 int trakhip_gram_split(const void* A_planes_dev, uint64_t N, uint64_t K, int dtype, float* C_dev, uint64_t ldc,
-                       float alpha, float beta, void* stream) {
-    return trakhip::gram_split(A_planes_dev, N, K, dtype, C_dev, ldc, alpha, beta, static_cast<hipStream_t>(stream));
+                       float alpha, float beta, void* workspace_dev, size_t workspace_bytes, void* stream) {
+    return trakhip::gram_split(A_planes_dev, N, K, dtype, C_dev, ldc, alpha, beta, workspace_dev, workspace_bytes,
+                               static_cast<hipStream_t>(stream));
 }
 
 size_t trakhip_split2_bytes(uint64_t rows, uint64_t K) { return trakhip::split2_bytes(rows, K); }
@@ -128,9 +133,10 @@ int trakhip_gemm_nt_split2(const void* A_planes_dev, const float* A_scales_dev, 
 }
 
 int trakhip_gram_split2(const void* A_planes_dev, const float* A_scales_dev, uint64_t N, uint64_t K, float* C_dev,
-                        uint64_t ldc, float alpha, float beta, void* stream) {
-    return trakhip::gram_split2(A_planes_dev, A_scales_dev, N, K, C_dev, ldc, alpha, beta,
-                                static_cast<hipStream_t>(stream));
+                        uint64_t ldc, float alpha, float beta, void* workspace_dev, size_t workspace_bytes,
+                        void* stream) {
+    return trakhip::gram_split2(A_planes_dev, A_scales_dev, N, K, C_dev, ldc, alpha, beta, workspace_dev,
+                                workspace_bytes, static_cast<hipStream_t>(stream));
 }
 
 int trakhip_gemm_nt16(const void* A_dev, uint64_t lda, const void* B_dev, uint64_t ldb, int dtype, float* C_dev,

@@ -35,6 +35,7 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include "short_k_tile.h"
 #include "trakhip_internal.h"
 
 namespace {
@@ -47,6 +48,7 @@ typedef uint32_t piece __attribute__((ext_vector_type(4)));  // 16 bytes = 8 x 1
 constexpr int kWavesM = 4, kWavesN = 2;            // 4 x 2 waves, each owns 64 x 128 of C
 constexpr int BM = 64 * kWavesM, BN = 128 * kWavesN;
 constexpr int kWaves = kWavesM * kWavesN;
+constexpr uint32_t kGemmTriangleGrid = 2u;          // kernel flag: the grid lists the lower-triangle tiles only
 constexpr int kRowPad = 256;                       // rows of an operand are padded to this
 constexpr int kOctetPad = 8;                       // octets (64 values of k) are padded to this
 
@@ -339,14 +341,29 @@ __global__ __launch_bounds__(64 * kWaves, 2) void gemm_split_kernel(
     const piece* __restrict__ A, uint64_t Rpa, const piece* __restrict__ B, uint64_t Rpb, uint64_t K8,
     float* __restrict__ C, uint64_t ldc, uint64_t M, uint64_t N, float alpha, float beta,
     const float* __restrict__ row_scale, uint32_t tiles_n, uint32_t flags, const float* __restrict__ a_unscale,
-    const float* __restrict__ b_unscale) {
+    const float* __restrict__ b_unscale, uint32_t parts, uint64_t part_stride) {
     constexpr int JT = BN / kWavesN / 32;            // 32-column MFMA tiles per wave
     constexpr int kAPieces = P * 2 * BM;             // [plane][half][row]
     constexpr int kSubPieces = P * 2 * (BM + BN);    // three planes: 3072 pieces = 48 KB
     constexpr int kBufPieces = S * kSubPieces;
     __shared__ piece lds[2][kBufPieces];
 
-    const uint32_t tile_m = blockIdx.x / tiles_n, tile_n = blockIdx.x % tiles_n;
+    // parts > 1: the grid is `parts` copies of the tile list; copy p multiplies the p-th share of the k
+    // steps and writes its sums to the p-th matrix at C (a later pass adds the shares in order)
+    uint32_t tile_id = blockIdx.x, part = 0;
+    if (parts > 1) {
+        const uint32_t per_part = gridDim.x / parts;
+        part = blockIdx.x / per_part;
+        tile_id = blockIdx.x % per_part;
+        C += (uint64_t)part * part_stride;
+    }
+    uint32_t tile_m, tile_n;
+    if (flags & kGemmTriangleGrid) {  // the tile list is the lower triangle, row by row
+        short_k::triangle_tile(tile_id, tile_m, tile_n);
+    } else {
+        tile_m = tile_id / tiles_n;
+        tile_n = tile_id % tiles_n;
+    }
     const uint64_t m0 = (uint64_t)tile_m * BM, n0 = (uint64_t)tile_n * BN;
     // a symmetric product needs only the tiles that touch the lower triangle
     if ((flags & trakhip::kGemmLowerTilesOnly) && n0 > m0 + BM - 1) return;
@@ -363,8 +380,9 @@ __global__ __launch_bounds__(64 * kWaves, 2) void gemm_split_kernel(
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
-    const uint64_t steps = K8 / (2 * S);
-    dma_step<P, S>(A, Rpa, B, Rpb, K8, m0, n0, 0, wave, lane, lds[0]);
+    const uint64_t all_steps = K8 / (2 * S);
+    const uint64_t first = all_steps * part / parts, steps = all_steps * (part + 1) / parts;  // [first, steps)
+    dma_step<P, S>(A, Rpa, B, Rpb, K8, m0, n0, first, wave, lane, lds[0]);
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
 
@@ -372,8 +390,8 @@ __global__ __launch_bounds__(64 * kWaves, 2) void gemm_split_kernel(
     const int a_lane = h * BM + wm * 64 + x;
     const int b_lane = kAPieces + h * BN + wn * (32 * JT) + x;
 
-    for (uint64_t s = 0; s < steps; ++s) {
-        const int cur = (int)(s & 1);
+    for (uint64_t s = first; s < steps; ++s) {
+        const int cur = (int)((s - first) & 1);
         // the other buffer was last read before the barrier that ended the previous step
         if (s + 1 < steps) dma_step<P, S>(A, Rpa, B, Rpb, K8, m0, n0, s + 1, wave, lane, lds[cur ^ 1]);
 #pragma unroll
@@ -531,6 +549,35 @@ __global__ __launch_bounds__(256) void mirror_lower_kernel(float* __restrict__ C
     }
 }
 
+// C = alpha * (P_0 + P_1 + ... in this order) + beta * C on the lower triangle, mirrored into the upper
+// one: closes a symmetric product whose k range was shared out over `parts` matrices at P.
+__global__ __launch_bounds__(256) void gram_combine_kernel(const float* __restrict__ P, uint64_t part_stride,
+                                                           uint32_t parts, float* __restrict__ C, uint64_t ldc,
+                                                           uint64_t n, float alpha, float beta) {
+    __shared__ float t[32][33];
+    const uint32_t bi = blockIdx.y, bj = blockIdx.x;  // 32 x 32 block (bi, bj) on or under the diagonal
+    if (bj > bi) return;
+    const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;
+#pragma unroll
+    for (int r = ty; r < 32; r += 8) {
+        const uint64_t row = (uint64_t)bi * 32 + r, col = (uint64_t)bj * 32 + tx;
+        float v = 0.0f;
+        if (row < n && col <= row) {
+            for (uint32_t p = 0; p < parts; ++p) v += P[(uint64_t)p * part_stride + row * n + col];
+            v *= alpha;
+            if (beta != 0.0f) v += beta * C[row * ldc + col];
+            C[row * ldc + col] = v;
+        }
+        t[r][tx] = v;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int r = ty; r < 32; r += 8) {
+        const uint64_t row = (uint64_t)bj * 32 + r, col = (uint64_t)bi * 32 + tx;  // the mirror image
+        if (row < n && col < n && col > row) C[row * ldc + col] = t[tx][r];
+    }
+}
+
 uint64_t padded_rows(uint64_t rows) { return (rows + kRowPad - 1) / kRowPad * kRowPad; }
 uint64_t octets(uint64_t K) { return (K + 8 * kOctetPad - 1) / (8 * kOctetPad) * kOctetPad; }
 int planes_of(int dtype) { return dtype == TRAKHIP_F32 ? 3 : 1; }
@@ -593,9 +640,14 @@ int mirror_lower(float* C, uint64_t ldc, uint64_t N, hipStream_t s) {
     return hipGetLastError() == hipSuccess ? TRAKHIP_OK : TRAKHIP_ERR_LAUNCH;
 }
 
+// sub-steps per barrier of each operand format
+int sub_steps(int dtype, bool two_planes) { return two_planes ? 2 : (dtype == TRAKHIP_F32 ? 1 : 4); }
+
+// parts > 1 (symmetric products only): the k steps are shared out over `parts` launches' worth of
+// workgroups that write plain sums into `parts` N x N matrices at C; see gram_combine_kernel.
 int launch_split(const void* A_planes, uint64_t M, const void* B_planes, uint64_t N, uint64_t K, int dtype, float* C,
                  uint64_t ldc, float alpha, float beta, const float* row_scale, hipStream_t s, uint32_t flags,
-                 const float* a_unscale, const float* b_unscale) {
+                 const float* a_unscale, const float* b_unscale, uint32_t parts = 1) {
     if (M == 0 || N == 0) return TRAKHIP_OK;
     if (K == 0 || ldc < N) return TRAKHIP_ERR_SHAPE;
     if (!A_planes || !B_planes || !C) return TRAKHIP_ERR_NULL;
@@ -604,13 +656,18 @@ int launch_split(const void* A_planes, uint64_t M, const void* B_planes, uint64_
         return TRAKHIP_ERR_ALIGN;
     const uint64_t tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
     if (tiles_m * tiles_n > 0x7FFFFFFFull) return TRAKHIP_ERR_SHAPE;
-    const dim3 grid((uint32_t)(tiles_m * tiles_n)), block(64 * kWaves);
+    uint64_t workgroups = tiles_m * tiles_n;
+    if (parts > 1) {
+        flags = kGemmTriangleGrid;
+        workgroups = tiles_m * (tiles_m + 1) / 2 * parts;
+    }
+    const dim3 grid((uint32_t)workgroups), block(64 * kWaves);
     const piece* a = static_cast<const piece*>(A_planes);
     const piece* b = static_cast<const piece*>(B_planes);
     const uint64_t Rpa = padded_rows(M), Rpb = padded_rows(N), K8 = octets(K);
     // ACCUM (beta != 0) fetches the old C in the epilogue; kept out of the plain kernel
     void (*kernel)(const piece*, uint64_t, const piece*, uint64_t, uint64_t, float*, uint64_t, uint64_t, uint64_t, float,
-                   float, const float*, uint32_t, uint32_t, const float*, const float*);
+                   float, const float*, uint32_t, uint32_t, const float*, const float*, uint32_t, uint64_t);
     const bool accum = beta != 0.0f;
     if (a_unscale)
         kernel = accum ? gemm_split_kernel<2, true, 2, true> : gemm_split_kernel<2, true, 2, false>;
@@ -621,8 +678,43 @@ int launch_split(const void* A_planes, uint64_t M, const void* B_planes, uint64_
     else
         kernel = accum ? gemm_split_kernel<1, false, 4, true> : gemm_split_kernel<1, false, 4, false>;
     hipLaunchKernelGGL(kernel, grid, block, 0, s, a, Rpa, b, Rpb, K8, C, ldc, M, N, alpha, beta, row_scale,
-                       (uint32_t)tiles_n, flags, a_unscale, b_unscale);
+                       (uint32_t)tiles_n, flags, a_unscale, b_unscale, parts, (uint64_t)N * N);
     return hipGetLastError() == hipSuccess ? TRAKHIP_OK : TRAKHIP_ERR_LAUNCH;
+}
+
+// A symmetric product has (tiles + 1) tiles / 2 workgroups' worth of work; up to 170 of them leave a third of
+// the CUs idle, and the k range is long enough to share out: three shares, a round and a half of
+// workgroups of a third of the work each.
+constexpr uint32_t kGramParts = 3;
+uint32_t gram_parts(uint64_t N, uint64_t K, int dtype, bool two_planes) {
+    const uint64_t tiles = (N + BM - 1) / BM, lower = tiles * (tiles + 1) / 2;
+    const uint64_t steps = octets(K) / (2 * sub_steps(dtype, two_planes));
+    return (lower <= 170 && steps >= 8 * kGramParts) ? kGramParts : 1;
+}
+
+int gram_impl(const void* A_planes, const float* a_scales, uint64_t N, uint64_t K, int dtype, float* C, uint64_t ldc,
+              float alpha, float beta, void* ws, size_t ws_bytes, hipStream_t s) {
+    if (N == 0) return TRAKHIP_OK;
+    const bool two_planes = a_scales != nullptr;
+    const uint32_t parts = gram_parts(N, K, dtype, two_planes);
+    const size_t need = (size_t)parts * N * N * sizeof(float);
+    if (parts > 1 && ws && ws_bytes >= need && reinterpret_cast<uintptr_t>(ws) % 16 == 0) {
+        if (!C) return TRAKHIP_ERR_NULL;
+        if (ldc < N) return TRAKHIP_ERR_SHAPE;
+        float* shares = static_cast<float*>(ws);
+        const int e = launch_split(A_planes, N, A_planes, N, K, dtype, shares, N, 1.0f, 0.0f, nullptr, s, 0u, a_scales,
+                                   a_scales, parts);
+        if (e) return e;
+        const uint64_t blocks = (N + 31) / 32;
+        if (blocks > 65535) return TRAKHIP_ERR_SHAPE;
+        hipLaunchKernelGGL(gram_combine_kernel, dim3((uint32_t)blocks, (uint32_t)blocks), dim3(256), 0, s, shares,
+                           (uint64_t)N * N, parts, C, ldc, N, alpha, beta);
+        return hipGetLastError() == hipSuccess ? TRAKHIP_OK : TRAKHIP_ERR_LAUNCH;
+    }
+    const int e = launch_split(A_planes, N, A_planes, N, K, dtype, C, ldc, alpha, beta, nullptr, s, trakhip::kGemmLowerTilesOnly,
+                               a_scales, a_scales);
+    if (e) return e;
+    return mirror_lower(C, ldc, N, s);
 }
 
 }  // namespace
@@ -685,13 +777,16 @@ int gemm_nt_split2(const void* A_planes, const float* a_scales, uint64_t M, cons
                         b_scales);
 }
 
+size_t gram_split_workspace_bytes(uint64_t N, uint64_t K, int dtype, int two_planes) {
+    if (N == 0 || K == 0 || !known_dtype(dtype)) return 0;
+    const uint32_t parts = gram_parts(N, K, dtype, two_planes != 0);
+    return parts > 1 ? (size_t)parts * N * N * sizeof(float) : 0;
+}
+
 int gram_split2(const void* A_planes, const float* a_scales, uint64_t N, uint64_t K, float* C, uint64_t ldc, float alpha,
-                float beta, hipStream_t s) {
-    if (N == 0) return TRAKHIP_OK;
-    const int e = gemm_nt_split2(A_planes, a_scales, N, A_planes, a_scales, N, K, C, ldc, alpha, beta, nullptr, s,
-                                 kGemmLowerTilesOnly);
-    if (e) return e;
-    return mirror_lower(C, ldc, N, s);
+                float beta, void* ws, size_t ws_bytes, hipStream_t s) {
+    if (N && !a_scales) return TRAKHIP_ERR_NULL;
+    return gram_impl(A_planes, a_scales, N, K, TRAKHIP_F32, C, ldc, alpha, beta, ws, ws_bytes, s);
 }
 
 int gemm_nt16(const void* A, uint64_t lda, const void* B, uint64_t ldb, int dtype, float* C, uint64_t ldc, uint64_t M,
@@ -719,11 +814,9 @@ int gemm_nt16(const void* A, uint64_t lda, const void* B, uint64_t ldb, int dtyp
 }
 
 int gram_split(const void* A_planes, uint64_t N, uint64_t K, int dtype, float* C, uint64_t ldc, float alpha, float beta,
-               hipStream_t s) {
-    if (N == 0) return TRAKHIP_OK;
-    const int e = gemm_nt_split(A_planes, N, A_planes, N, K, dtype, C, ldc, alpha, beta, nullptr, s, kGemmLowerTilesOnly);
-    if (e) return e;
-    return mirror_lower(C, ldc, N, s);
+               void* ws, size_t ws_bytes, hipStream_t s) {
+    if (!known_dtype(dtype)) return TRAKHIP_ERR_DTYPE;
+    return gram_impl(A_planes, nullptr, N, K, dtype, C, ldc, alpha, beta, ws, ws_bytes, s);
 }
 
 }  // namespace trakhip

@@ -514,7 +514,7 @@ int spd_inverse(const float* A, uint64_t lda, float lambda, float* inv, uint64_t
     // exactly symmetric.  The planes go where W and L were (or behind the scratch for small n).
     void* planes = planes_tail_bytes(n, np) ? static_cast<void*>(mean_dev + 4) : static_cast<void*>(W);
     e = split_rows(Li, TRAKHIP_F32, np, n, n, 1, planes, split_bytes(n, n, TRAKHIP_F32), s);
-    if (!e) e = gram_split(planes, n, n, TRAKHIP_F32, inv, ldi, 1.0f, 0.0f, s);
+    if (!e) e = gram_split(planes, n, n, TRAKHIP_F32, inv, ldi, 1.0f, 0.0f, nullptr, 0, s);
     if (e) return e;
 
     if (normalize || mean_abs) {

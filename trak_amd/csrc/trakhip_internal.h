@@ -55,8 +55,10 @@ int split_rows(const void* src, int dtype, uint64_t ld, uint64_t rows, uint64_t 
                size_t planes_bytes, hipStream_t s);
 int gemm_nt_split(const void* A_planes, uint64_t M, const void* B_planes, uint64_t N, uint64_t K, int dtype, float* C,
                   uint64_t ldc, float alpha, float beta, const float* row_scale, hipStream_t s, uint32_t flags = 0);
+// ws (may be null): gram_split_workspace_bytes() bytes that let a product with few tiles share its k range out
+size_t gram_split_workspace_bytes(uint64_t N, uint64_t K, int dtype, int two_planes);
 int gram_split(const void* A_planes, uint64_t N, uint64_t K, int dtype, float* C, uint64_t ldc, float alpha, float beta,
-               hipStream_t s);
+               void* ws, size_t ws_bytes, hipStream_t s);
 size_t split2_bytes(uint64_t rows, uint64_t K);
 int split2_rows(const float* src, uint64_t ld, uint64_t rows, uint64_t K, int transposed, void* planes,
                 size_t planes_bytes, float* scales, hipStream_t s);
@@ -64,7 +66,7 @@ int gemm_nt_split2(const void* A_planes, const float* a_scales, uint64_t M, cons
                    uint64_t N, uint64_t K, float* C, uint64_t ldc, float alpha, float beta, const float* row_scale,
                    hipStream_t s, uint32_t flags = 0);
 int gram_split2(const void* A_planes, const float* a_scales, uint64_t N, uint64_t K, float* C, uint64_t ldc, float alpha,
-                float beta, hipStream_t s);
+                float beta, void* ws, size_t ws_bytes, hipStream_t s);
 int gemm_nt16(const void* A, uint64_t lda, const void* B, uint64_t ldb, int dtype, float* C, uint64_t ldc, uint64_t M,
               uint64_t N, uint64_t K, float alpha, float beta, const float* row_scale, hipStream_t s);
 size_t spd_inverse_workspace_bytes(uint64_t n);

@@ -336,15 +336,21 @@ def gram_split(a, out=None, alpha=1.0, beta=0.0):
     lib = _lib.load()
     with torch.cuda.device(a.device):
         stream = torch.cuda.current_stream(a.device).cuda_stream
-        if a.scales is not None:
+        # scratch that lets a product with few tiles share its k range out over the idle CUs
+        two = a.scales is not None
+        ws_bytes = lib.trakhip_gram_split_workspace(N, a.K, _STORE_DTYPES[a.dtype], int(two))
+        ws = torch.empty(ws_bytes, dtype=torch.uint8, device=a.device) if ws_bytes else None
+        ws_ptr = ctypes.c_void_p(ws.data_ptr()) if ws is not None else None
+        if two:
             code = lib.trakhip_gram_split2(
                 ctypes.c_void_p(a.planes.data_ptr()), ctypes.c_void_p(a.scales.data_ptr()), N, a.K,
-                ctypes.c_void_p(out.data_ptr()), _ld(out), float(alpha), float(beta), ctypes.c_void_p(stream),
+                ctypes.c_void_p(out.data_ptr()), _ld(out), float(alpha), float(beta), ws_ptr, ws_bytes,
+                ctypes.c_void_p(stream),
             )
         else:
             code = lib.trakhip_gram_split(
                 ctypes.c_void_p(a.planes.data_ptr()), N, a.K, _STORE_DTYPES[a.dtype], ctypes.c_void_p(out.data_ptr()),
-                _ld(out), float(alpha), float(beta), ctypes.c_void_p(stream),
+                _ld(out), float(alpha), float(beta), ws_ptr, ws_bytes, ctypes.c_void_p(stream),
             )
     _lib.check(code)
     return out
