@@ -311,3 +311,58 @@ def test_projection_and_scoring_replay_from_a_hip_graph(gpu):
         assert torch.equal(got_feats, feats) and torch.equal(got_scores, scores), rep
         assert float(got_scores.abs().sum()) > 0
         _ = split_rows(targets)                  # unrelated eager work between replays
+
+
+def test_gram_and_inverse_replay_from_a_hip_graph(gpu):
+    """X^T X (operand split, k range shared out over three sets of workgroups, fixed-order combine) and the
+    regularized inverse (about a hundred dependent launches, one of them heterogeneous) through the C
+    ABI with caller-owned buffers: captured once, replayed with new inputs, equal to the eager result
+    bit for bit, status word included."""
+    lib = _lib.load()
+    N, n, lam = 1500, 384, 1e-2
+    gen = torch.Generator(device=gpu).manual_seed(9)
+    x_static = torch.zeros(N, n, device=gpu)
+    planes = torch.empty(lib.trakhip_split_bytes(n, N, _lib.F32), dtype=torch.uint8, device=gpu)
+    gram_ws_bytes = lib.trakhip_gram_split_workspace(n, N, _lib.F32, 0)
+    assert gram_ws_bytes == 3 * n * n * 4
+    gram_ws = torch.empty(gram_ws_bytes, dtype=torch.uint8, device=gpu)
+    xtx = torch.empty(n, n, device=gpu)
+    inv = torch.empty(n, n, device=gpu)
+    mean_abs = torch.zeros(1, device=gpu)
+    status = torch.full((1,), -1, dtype=torch.int32, device=gpu)
+    spd_ws = torch.empty(lib.trakhip_spd_inverse_workspace(n), dtype=torch.uint8, device=gpu)
+    vp = lambda t: ctypes.c_void_p(t.data_ptr())
+
+    def work():
+        stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+        assert lib.trakhip_split_rows(vp(x_static), _lib.F32, n, n, N, 1, vp(planes), planes.numel(), stream) == 0
+        assert lib.trakhip_gram_split(vp(planes), n, N, _lib.F32, vp(xtx), n, 1.0, 0.0, vp(gram_ws), gram_ws_bytes,
+                                      stream) == 0
+        assert lib.trakhip_spd_inverse(vp(xtx), n, lam, vp(inv), n, n, 1, vp(mean_abs), vp(status), vp(spd_ws),
+                                       spd_ws.numel(), stream) == 0
+
+    x_static.copy_(torch.randn(N, n, generator=gen, device=gpu))
+    work()
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            work()
+    torch.cuda.current_stream().wait_stream(side)
+    for rep in range(3):
+        x_static.copy_(torch.randn(N, n, generator=gen, device=gpu) * (1.0 + rep))
+        status.fill_(-1)
+        graph.replay()
+        torch.cuda.synchronize()
+        got = (xtx.clone(), inv.clone(), mean_abs.clone(), int(status.item()))
+        status.fill_(-1)
+        work()                                   # eager, same buffers
+        torch.cuda.synchronize()
+        assert got[3] == 0 and int(status.item()) == 0
+        assert torch.equal(got[0], xtx) and torch.equal(got[1], inv) and torch.equal(got[2], mean_abs), rep
+        a64 = x_static.double().T @ x_static.double() + lam * torch.eye(n, device=gpu, dtype=torch.float64)
+        resid = a64 @ (got[1].double() * got[2].double()) - torch.eye(n, device=gpu, dtype=torch.float64)
+        assert float(resid.abs().max()) < 1e-4
+        _ = torch.randn(64, 64, device=gpu) @ torch.randn(64, 64, device=gpu)      # unrelated eager work
