@@ -29,8 +29,7 @@ constexpr int kSumBlocks = 1024;
 
 __global__ __launch_bounds__(256) void spd_init_kernel(const float* __restrict__ A, uint64_t lda, float lambda,
                                                        uint64_t n, uint64_t np, float* __restrict__ W,
-                                                       float* __restrict__ L, float* __restrict__ Li,
-                                                       int32_t* __restrict__ status) {
+                                                       float* __restrict__ Li, int32_t* __restrict__ status) {
     const uint64_t idx = (uint64_t)blockIdx.x * 256 + threadIdx.x;
     if (idx == 0 && status) *status = 0;
     if (idx >= np * np) return;
@@ -41,8 +40,8 @@ __global__ __launch_bounds__(256) void spd_init_kernel(const float* __restrict__
     else
         v = (i == j) ? 1.0f : 0.0f;
     W[idx] = v;
-    L[idx] = 0.0f;
-    Li[idx] = 0.0f;
+    Li[idx] = 0.0f;  // the blocks above the diagonal stay zero: the final product reads all of Li
+    // (every block of L that is read later - diagonal blocks, panels - is written first)
 }
 
 // One workgroup of four waves: Cholesky of the 128x128 diagonal block at W (lower triangle used),
@@ -473,7 +472,7 @@ int spd_inverse(const float* A, uint64_t lda, float lambda, float* inv, uint64_t
 
     const uint64_t total = np * np;
     hipLaunchKernelGGL(spd_init_kernel, dim3((uint32_t)((total + 255) / 256)), dim3(256), 0, s, A, lda, lambda, n,
-                       np, W, L, Li, status);
+                       np, W, Li, status);
     if (hipGetLastError() != hipSuccess) return TRAKHIP_ERR_LAUNCH;
 
     // Diagonal block 0 alone; then per block column j: the panel below it, and one launch that holds both
