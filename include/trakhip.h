@@ -42,6 +42,7 @@ extern "C" {
 #define TRAKHIP_ERR_NOT_SPD -9   /* matrix handed to the SPD inverse is not positive definite */
 #define TRAKHIP_ERR_NO_DEVICE -10
 #define TRAKHIP_ERR_POINTER -11  /* destination is neither device memory nor page-locked host memory */
+#define TRAKHIP_ERR_STATIC_LIMIT -12 /* trakhip_project_static: shape needs more than its static scratch */
 
 const char* trakhip_strerror(int code);
 
@@ -67,6 +68,21 @@ size_t trakhip_project_workspace(uint64_t B, uint64_t P, uint32_t proj_dim, uint
 int trakhip_project(const void* in_dev, int in_dtype, uint64_t B, uint64_t P, uint64_t ld_in,
                     float* out_dev, void* workspace_dev, size_t workspace_bytes, uint32_t proj_dim,
                     uint32_t seed, uint32_t num_feature_tiles, int proj_type, void* stream);
+
+/* trakhip_project for callers that cannot allocate or hand over a workspace (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference:
+ * fast_jl allocates its intermediate with torch::zeros on every call (fast_jl/fast_jl.cu:48-49).
+ * Same arguments, checks and results (bit for bit) as trakhip_project, minus the workspace: the
+ * partial sums live in a static device array of trakhip_project_static_limit() bytes (36 MiB) that
+ * each GPU the library runs on holds until the process ends.  A shape whose
+ * trakhip_project_workspace() exceeds that is refused with TRAKHIP_ERR_STATIC_LIMIT (every shape
+ * with proj_dim <= 65536 fits).  Calls no hipMalloc / hipFree or any allocating routine.  All calls
+ * on one GPU share the one array: calls that overlap in time on the same GPU (different streams
+ * or threads) race and give wrong results; calls that follow one another on a stream do not. */
+size_t trakhip_project_static_limit(void);
+int trakhip_project_static(const void* in_dev, int in_dtype, uint64_t B, uint64_t P, uint64_t ld_in,
+                           float* out_dev, uint32_t proj_dim, uint32_t seed, uint32_t num_feature_tiles,
+                           int proj_type, void* stream);
 
 /* The two phases of trakhip_project as separate calls, for B <= 32 rows: phase 1 writes partial
  * sums [G, B, proj_dim] over G runs of consecutive features to the workspace (the kernel of

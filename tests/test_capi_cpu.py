@@ -34,7 +34,7 @@ def test_abi_version_and_strerror():
     assert _lib.strerror(0) == "success"
     # the text the reference throws at fast_jl/fast_jl_kernel.cuh:113-115
     assert _lib.strerror(-1) == "Invalid Number of JL dimensions it has to be a multiple of 512"
-    for code in range(-11, 0):
+    for code in range(-12, 0):
         assert "unknown trakhip error" not in _lib.strerror(code)
     assert "unknown trakhip error" in _lib.strerror(-999)
 
@@ -57,6 +57,21 @@ def test_project_argument_validation_needs_no_device():
         _lib.check(-1)
     with pytest.raises(RuntimeError):
         _lib.check(-2)
+
+
+def test_static_entry_point_validates_before_touching_the_device():
+    lib = _lib.load()
+    p = ctypes.c_void_p(4096)
+    call = lambda **kw: lib.trakhip_project_static(
+        kw.get("inp", p), kw.get("dtype", 0), kw.get("B", 32), kw.get("P", 1024), kw.get("ld", 1024),
+        kw.get("out", p), kw.get("k", 512), 0, kw.get("tiles", 2), kw.get("pt", 0), None)
+    assert lib.trakhip_project_static_limit() == 36 << 20
+    assert call(k=100) == -1 and call(B=0) == -2 and call(dtype=5) == -3 and call(pt=9) == -4
+    assert call(inp=None) == -5 and call(out=None) == -5 and call(out=ctypes.c_void_p(4100)) == -7
+    # two runs of 150 column blocks: 37.5 MiB of partial sums, more than the 36 MiB array
+    assert lib.trakhip_project_workspace(32, 1024, 153_600, 2) == 2 * 32 * 153_600 * 4
+    assert call(k=153_600) == -12
+    assert "static" in _lib.strerror(-12)
 
 
 def test_workspace_size():

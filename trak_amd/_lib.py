@@ -42,6 +42,10 @@ def load():
     lib.trakhip_project_workspace.restype = sz
     lib.trakhip_project.argtypes = [vp, i32, u64, u64, u64, vp, vp, sz, u32, u32, u32, i32, vp]
     lib.trakhip_project.restype = i32
+    lib.trakhip_project_static_limit.argtypes = []
+    lib.trakhip_project_static_limit.restype = sz
+    lib.trakhip_project_static.argtypes = [vp, i32, u64, u64, u64, vp, u32, u32, u32, i32, vp]
+    lib.trakhip_project_static.restype = i32
     lib.trakhip_project_partials.argtypes = [vp, i32, u64, u64, u64, vp, sz, u32, u32, u32, i32, vp]
     lib.trakhip_project_partials.restype = i32
     lib.trakhip_project_gather_partials.argtypes = [vp, u32, i32, u64, u64, vp, sz, u32, u32, u32, i32, vp]

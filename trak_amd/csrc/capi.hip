@@ -19,6 +19,8 @@ const char* trakhip_strerror(int code) {
         case TRAKHIP_ERR_NO_DEVICE: return "no HIP device";
         case TRAKHIP_ERR_POINTER:
             return "destination is neither device memory nor page-locked host memory";
+        case TRAKHIP_ERR_STATIC_LIMIT:
+            return "shape needs more scratch than the static array of trakhip_project_static holds";
         default: return "unknown trakhip error";
     }
 }
@@ -34,6 +36,15 @@ int trakhip_project(const void* in_dev, int in_dtype, uint64_t B, uint64_t P, ui
                     uint32_t num_feature_tiles, int proj_type, void* stream) {
     return trakhip::project(in_dev, in_dtype, B, P, ld_in, out_dev, workspace_dev, workspace_bytes, proj_dim,
                             seed, num_feature_tiles, proj_type, static_cast<hipStream_t>(stream));
+}
+
+size_t trakhip_project_static_limit(void) { return trakhip::project_static_limit_bytes(); }
+
+int trakhip_project_static(const void* in_dev, int in_dtype, uint64_t B, uint64_t P, uint64_t ld_in, float* out_dev,
+                           uint32_t proj_dim, uint32_t seed, uint32_t num_feature_tiles, int proj_type,
+                           void* stream) {
+    return trakhip::project_static(in_dev, in_dtype, B, P, ld_in, out_dev, proj_dim, seed, num_feature_tiles,
+                                   proj_type, static_cast<hipStream_t>(stream));
 }
 
 int trakhip_project_partials(const void* in_dev, int in_dtype, uint64_t B, uint64_t P, uint64_t ld_in,

@@ -27,6 +27,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <atomic>
+
 #include "jl_stream.h"
 #include "store_cast.h"
 #include "trakhip_internal.h"
@@ -741,6 +743,13 @@ LaunchFn pick(const Plan& pl, int dtype, int proj_type, bool gather) {
 
 }  // namespace
 
+// Scratch of trakhip_project_static (see project_static below): 36 MiB, enough for every shape with
+// proj_dim <= 65536.
+constexpr size_t kStaticScratchBytes = 36u << 20;
+constexpr int kMaxDevices = 64;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+static std::atomic<void*> static_scratch_ptr[kMaxDevices];
+
 namespace trakhip {
 
 size_t project_workspace_bytes(uint64_t B, uint64_t P, uint32_t k, uint32_t num_feature_tiles) {
@@ -839,6 +848,48 @@ int project(const void* in, int dtype, uint64_t B, uint64_t P, uint64_t ld, floa
         if (r) return r;
     }
     return TRAKHIP_OK;
+}
+
+// ---- projection without any allocation ------------------------------------------------------
+//
+// For callers that cannot provide or allocate a workspace (code under HIP graph capture, tight
+// serving loops): the partial sums go to a file-scope device array instead.  Every device the
+// library runs on holds its own copy of the array, at its own address, until the process ends.
+// In host code the array's name is only a handle for hipGetSymbolAddress: the address that kernels
+// and copies use is looked up once per device (with that device current) and kept in
+// static_scratch_ptr[]; the name itself is never passed to a kernel.
+
+size_t project_static_limit_bytes() { return kStaticScratchBytes; }
+
+// Address of the current device's copy of `scratch` (nullptr + error code on failure).
+static int static_scratch(void** ptr) {
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return TRAKHIP_ERR_NO_DEVICE;
+    void* p = static_scratch_ptr[dev].load(std::memory_order_acquire);
+    if (!p) {
+        // two threads racing here look up the same address; the store is idempotent
+        if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess || !p) return TRAKHIP_ERR_NO_DEVICE;
+        static_scratch_ptr[dev].store(p, std::memory_order_release);
+    }
+    *ptr = p;
+    return TRAKHIP_OK;
+}
+
+int project_static(const void* in, int dtype, uint64_t B, uint64_t P, uint64_t ld, float* out, uint32_t k,
+                   uint32_t seed, uint32_t num_feature_tiles, int proj_type, hipStream_t s) {
+    // host-only validation first (a dummy non-null, aligned workspace of unlimited size)
+    const int e = check_project_args(in, dtype, B, P, ld, reinterpret_cast<const void*>(uintptr_t(256)), SIZE_MAX, k,
+                                     num_feature_tiles, proj_type);
+    if (e) return e;
+    if (!out) return TRAKHIP_ERR_NULL;
+    if (reinterpret_cast<uintptr_t>(out) % 16) return TRAKHIP_ERR_ALIGN;
+    if (project_workspace_bytes(B, P, k, num_feature_tiles) > kStaticScratchBytes) return TRAKHIP_ERR_STATIC_LIMIT;
+    void* ws = nullptr;
+    const int d = static_scratch(&ws);
+    if (d) return d;
+    // every partial block that the reduction reads is written by the projection kernel of the same
+    // call, so nothing in the array has to start at zero
+    return project(in, dtype, B, P, ld, out, ws, kStaticScratchBytes, k, seed, num_feature_tiles, proj_type, s);
 }
 
 int materialize_device(uint32_t seed, uint32_t num_feature_tiles, uint64_t P, uint64_t f0, uint64_t nf,

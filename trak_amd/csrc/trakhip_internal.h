@@ -12,6 +12,10 @@ size_t project_workspace_bytes(uint64_t B, uint64_t P, uint32_t k, uint32_t num_
 int project(const void* in, int dtype, uint64_t B, uint64_t P, uint64_t ld, float* out, void* ws,
             size_t ws_bytes, uint32_t k, uint32_t seed, uint32_t num_feature_tiles, int proj_type,
             hipStream_t s);
+// the same without a workspace argument: partial sums go to a per-device static array
+size_t project_static_limit_bytes();
+int project_static(const void* in, int dtype, uint64_t B, uint64_t P, uint64_t ld, float* out, uint32_t k,
+                   uint32_t seed, uint32_t num_feature_tiles, int proj_type, hipStream_t s);
 int project_partials(const void* in, int dtype, uint64_t B, uint64_t P, uint64_t ld, void* ws, size_t ws_bytes,
                      uint32_t k, uint32_t seed, uint32_t num_feature_tiles, int proj_type, hipStream_t s);
 int project_gather_partials(const trakhip_segment* segs, uint32_t n_segs, int dtype, uint64_t B, uint64_t P,
