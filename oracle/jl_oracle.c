@@ -19,7 +19,7 @@
  *                         this build (the reference's XORWOW draw order cannot be reproduced);
  *                         what it keeps from fast_jl/random.cuh:27-60 -- one stream per
  *                         (column, tile), entries in feature order, one bit per Rademacher
- *                         entry with bit set -> +1, Box-Muller normals rounded to fp16 -- is
+ *                         entry with bit set -> +1, Box-Muller normals in fp16 -- is
  *                         PINNED by a second independent implementation (oracle/jl_oracle.py),
  *                         by exhaustive "every bit of a block used exactly once" checks, by the
  *                         parity property of tests/test_rademacher.py:65-108 and by
@@ -85,10 +85,10 @@ static uint32_t float_to_bits(float f) {
     return b;
 }
 
-/* Radius of the Box-Muller pair: sqrt(-2 ln u) with u = (2*(w>>9)+1) / 2^24, evaluated in
- * binary32 by a fixed sequence of IEEE operations. */
-static float radius_from_word(uint32_t w) {
-    uint32_t odd = 2u * (w >> 9) + 1u;
+/* Radius of a Box-Muller pair for the 15-bit index x: sqrt(-2 ln u) with u = (x + 1/2) / 2^15
+ * = (2x + 1) / 2^16, evaluated in binary32 by a fixed sequence of IEEE operations. */
+static float radius_from_index(uint32_t x) {
+    uint32_t odd = 2u * x + 1u;
     float xf = (float)odd;
     uint32_t xb = float_to_bits(xf);
     int expo = (int)((xb >> 23) & 0xFFu) - 127;
@@ -108,7 +108,7 @@ static float radius_from_word(uint32_t w) {
     float y = t * zp;
     y = fmaf(-0.5f, z, y);
     float ln_m = t + y;
-    float ln_u = fmaf((float)(expo - 24), 0.693147182f, ln_m);
+    float ln_u = fmaf((float)(expo - 16), 0.693147182f, ln_m);
     float s = -2.0f * ln_u;
     float guess = bits_to_float(0x5f3759dfu - (float_to_bits(s) >> 1));
     float half_s = 0.5f * s;
@@ -120,11 +120,13 @@ static float radius_from_word(uint32_t w) {
     return s * guess;
 }
 
-static void cos_sin_from_word(uint32_t w, float* c, float* s) {
-    uint32_t quadrant = w >> 30;
-    float frac = (float)((w >> 6) & 0xFFFFFFu);
-    float d = frac - 8388608.0f;
-    float y = d * 9.36266447e-8f;
+/* cos and sin of the angle (a + 1/2) * (pi/2) / 2^13 for the 13-bit index a.  Angles above pi/4
+ * are evaluated at their mirror image pi/2 - angle (index 8191 - a) with cos and sin exchanged. */
+static void cos_sin_from_index(uint32_t a, float* c, float* s) {
+    int upper = a > 4095u;
+    uint32_t idx = upper ? 8191u - a : a;
+    float steps = (float)idx + 0.5f;
+    float y = steps * 1.91747604e-4f; /* pi / 2^14 */
     float y2 = y * y;
     float ps = fmaf(-1.9515295891e-4f, y2, 8.3321608736e-3f);
     ps = fmaf(ps, y2, -1.6666654611e-1f);
@@ -135,11 +137,12 @@ static void cos_sin_from_word(uint32_t w, float* c, float* s) {
     float pcy2 = pc * y2;
     float base = fmaf(-0.5f, y2, 1.0f);
     float cs = fmaf(pcy2, y2, base);
-    switch (quadrant) {
-        case 0: *c = cs; *s = sn; break;
-        case 1: *c = -sn; *s = cs; break;
-        case 2: *c = -cs; *s = -sn; break;
-        default: *c = sn; *s = -cs; break;
+    if (upper) {
+        *c = sn;
+        *s = cs;
+    } else {
+        *c = cs;
+        *s = sn;
     }
 }
 
@@ -186,6 +189,44 @@ static float half_bits_to_float(uint16_t h) {
     return (float)(sign ? -v : v);
 }
 
+/* The three factor tables as fp16 bit patterns (tests compare them with a float64 math library). */
+uint16_t jlo_radius_half(uint32_t x) { return half_bits_rne(radius_from_index(x & 0x7FFFu)); }
+uint16_t jlo_cos_half(uint32_t a) {
+    float c, s;
+    cos_sin_from_index(a & 0x1FFFu, &c, &s);
+    return half_bits_rne(c);
+}
+uint16_t jlo_sin_half(uint32_t a) {
+    float c, s;
+    cos_sin_from_index(a & 0x1FFFu, &c, &s);
+    return half_bits_rne(s);
+}
+
+/* One normal entry from one random word: radius index = bits 16..30, angle index = bits 2..14;
+ * the cosine entry takes its sign from bit 15, the sine entry from bit 31 (bit set: negative).
+ * The two fp16 factors are multiplied exactly (22-bit product, exact in double) and rounded once. */
+float jlo_normal_from_word(uint32_t w, int sine) {
+    static uint16_t rtab[1 << 15], ctab[1 << 13], stab[1 << 13];
+    static int ready = 0;
+    if (!ready) {
+        for (uint32_t x = 0; x < (1u << 15); ++x) rtab[x] = jlo_radius_half(x);
+        for (uint32_t a = 0; a < (1u << 13); ++a) {
+            ctab[a] = jlo_cos_half(a);
+            stab[a] = jlo_sin_half(a);
+        }
+        ready = 1;
+    }
+    uint32_t x = (w >> 16) & 0x7FFFu;
+    uint32_t a = (w >> 2) & 0x1FFFu;
+    double radius = (double)half_bits_to_float(rtab[x]);
+    double trig = (double)half_bits_to_float(sine ? stab[a] : ctab[a]);
+    double prod = radius * trig;
+    float pf = (float)prod; /* exact: 22 significant bits, well inside the binary32 range */
+    float mag = half_bits_to_float(half_bits_rne(pf));
+    int negative = sine ? (int)(w >> 31) : (int)((w >> 15) & 1u);
+    return negative ? -mag : mag;
+}
+
 /* Value of S[f, c] (as float; always exactly an fp16 value). */
 float jlo_entry(uint32_t seed, uint32_t num_feature_tiles, uint64_t P, uint64_t f, uint32_t c,
                 int proj_type) {
@@ -206,25 +247,12 @@ float jlo_entry(uint32_t seed, uint32_t num_feature_tiles, uint64_t P, uint64_t 
         uint32_t bitpos = (slot % 2u ? 31u : 15u) - mfma_index;
         return ((word >> bitpos) & 1u) ? 1.0f : -1.0f;
     } else {
-        uint32_t ctr[4] = {offset / 4u, 0u, 0u, 0u};
+        /* eight entries per block; word i of the block makes entries 2i (cosine) and 2i+1 (sine) */
+        uint32_t ctr[4] = {offset / 8u, 0u, 0u, 0u};
         jlo_philox4x32_10(ctr, key, out);
-        uint32_t e = offset % 4u;
-        uint32_t wa = e < 2u ? out[0] : out[2];
-        uint32_t wb = e < 2u ? out[1] : out[3];
-        float r = radius_from_word(wa);
-        float c_, s_;
-        cos_sin_from_word(wb, &c_, &s_);
-        float z = (e % 2u) ? r * s_ : r * c_;
-        return half_bits_to_float(half_bits_rne(z));
+        uint32_t e = offset % 8u;
+        return jlo_normal_from_word(out[e / 2u], (int)(e % 2u));
     }
-}
-
-/* The binary32 normal before rounding to fp16 (for checks against a float64 Box-Muller). */
-float jlo_normal_unrounded(uint32_t wa, uint32_t wb, int second) {
-    float r = radius_from_word(wa);
-    float c_, s_;
-    cos_sin_from_word(wb, &c_, &s_);
-    return second ? r * s_ : r * c_;
 }
 
 uint16_t jlo_half_bits(float v) { return half_bits_rne(v); }

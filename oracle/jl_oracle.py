@@ -9,7 +9,8 @@ Restated reference behaviour (MadryLab/trak):
   * stream_seed   -- fast_jl/random.cuh:15-17
   * tiling        -- fast_jl/fast_jl.cu:42, fast_jl/fast_jl_kernel.cuh:124
   * Rademacher: one random bit per entry, bit set -> +1 -- fast_jl/random.cuh:33-37
-  * Normal: Box-Muller normal rounded to fp16 -- fast_jl/random.cuh:50-60
+  * Normal: Box-Muller normal in fp16 (fp16 radius times fp16 cos/sin, rounded once)
+    -- fast_jl/random.cuh:50-60
 The generator is Philox4x32-10 (Random123), pinned by Random123's known-answer vectors in
 tests/test_oracle_philox.py; the position -> (block, bit) map is this build's definition and
 is pinned by agreement of this file with oracle/jl_oracle.c and by the property tests.
@@ -99,14 +100,14 @@ def _f32(x):
     return np.asarray(x, dtype=np.float32)
 
 
-def box_muller_unrounded(wa, wb):
-    """Two float32 normals (cos branch, sin branch) from two uint32 words, following the
-    specified binary32 operation sequence."""
-    wa = np.asarray(wa, dtype=np.uint32)
-    wb = np.asarray(wb, dtype=np.uint32)
+def radius_f32(x):
+    """sqrt(-2 ln u), u = (x + 1/2) / 2^15, for 15-bit indices x: the specified binary32
+    operation sequence (log by exponent/mantissa split and a degree-9 polynomial, square root by
+    three Newton steps on the reciprocal root)."""
+    x = np.asarray(x, dtype=np.uint32)
     one = np.float32(1.0)
-    odd = ((wa >> np.uint32(9)) << np.uint32(1)) | np.uint32(1)
-    xf = odd.astype(np.float32)  # exact, < 2^24
+    odd = (x << np.uint32(1)) | np.uint32(1)
+    xf = odd.astype(np.float32)  # exact, < 2^16
     xb = xf.view(np.uint32)
     expo = (xb >> np.uint32(23)).astype(np.int32) - 127
     mant = ((xb & np.uint32(0x7FFFFF)) | np.uint32(0x3F800000)).view(np.float32)
@@ -132,7 +133,7 @@ def box_muller_unrounded(wa, wb):
     y = (t * (z * poly).astype(np.float32)).astype(np.float32)
     y = _fma32(np.float32(-0.5), z, y)
     ln_m = (t + y).astype(np.float32)
-    ln_u = _fma32((expo - 24).astype(np.float32), np.float32(0.693147182), ln_m)
+    ln_u = _fma32((expo - 16).astype(np.float32), np.float32(0.693147182), ln_m)
     s = (np.float32(-2.0) * ln_u).astype(np.float32)
     guess = (np.uint32(0x5F3759DF) - (s.view(np.uint32) >> np.uint32(1))).view(np.float32)
     half_s = (np.float32(0.5) * s).astype(np.float32)
@@ -140,11 +141,17 @@ def box_muller_unrounded(wa, wb):
         gg = (guess * guess).astype(np.float32)
         corr = _fma32(-half_s, gg, np.float32(1.5))
         guess = (guess * corr).astype(np.float32)
-    radius = (s * guess).astype(np.float32)
+    return (s * guess).astype(np.float32)
 
-    quadrant = wb >> np.uint32(30)
-    frac = ((wb >> np.uint32(6)) & np.uint32(0xFFFFFF)).astype(np.float32)
-    yv = ((frac - np.float32(8388608.0)).astype(np.float32) * np.float32(9.36266447e-8)).astype(np.float32)
+
+def cos_sin_f32(a):
+    """cos and sin of (a + 1/2) * (pi/2) / 2^13 for 13-bit indices a, as binary32: polynomials on
+    (0, pi/4); the upper half of the range is the mirror image (index 8191 - a, cos <-> sin)."""
+    a = np.asarray(a, dtype=np.uint32)
+    one = np.float32(1.0)
+    mirror = a >= np.uint32(4096)
+    am = np.where(mirror, np.uint32(8191) - a, a).astype(np.uint32)
+    yv = ((am.astype(np.float32) + np.float32(0.5)).astype(np.float32) * np.float32(1.91747604e-4)).astype(np.float32)
     y2 = (yv * yv).astype(np.float32)
     ps = _fma32(np.float32(-1.9515295891e-4), y2, np.float32(8.3321608736e-3))
     ps = _fma32(ps, y2, np.float32(-1.6666654611e-1))
@@ -152,11 +159,36 @@ def box_muller_unrounded(wa, wb):
     pc = _fma32(np.float32(2.443315711809948e-5), y2, np.float32(-1.388731625493765e-3))
     pc = _fma32(pc, y2, np.float32(4.166664568298827e-2))
     cs = _fma32((pc * y2).astype(np.float32), y2, _fma32(np.float32(-0.5), y2, one))
-    cosv = np.select([quadrant == 0, quadrant == 1, quadrant == 2], [cs, -sn, -cs], default=sn)
-    sinv = np.select([quadrant == 0, quadrant == 1, quadrant == 2], [sn, cs, -sn], default=-cs)
-    z0 = (radius * cosv.astype(np.float32)).astype(np.float32)
-    z1 = (radius * sinv.astype(np.float32)).astype(np.float32)
-    return z0, z1
+    return np.where(mirror, sn, cs).astype(np.float32), np.where(mirror, cs, sn).astype(np.float32)
+
+
+_TABLES = None
+
+
+def normal_tables():
+    """(R, C, S): the fp16 factor tables of the normal entries (round to nearest even of the
+    binary32 sequences above), as float16 arrays of 2^15, 2^13 and 2^13 entries."""
+    global _TABLES
+    if _TABLES is None:
+        r = radius_f32(np.arange(1 << 15, dtype=np.uint32)).astype(np.float16)
+        c, s = cos_sin_f32(np.arange(1 << 13, dtype=np.uint32))
+        _TABLES = (r, c.astype(np.float16), s.astype(np.float16))
+    return _TABLES
+
+
+def normal_from_word(w, sine):
+    """fp16 normal entries (returned as float16) from random words w: radius index bits 16..30,
+    angle index bits 2..14; sign of the cosine entry bit 15, of the sine entry bit 31 (set ->
+    negative).  The product of the two fp16 factors is exact in float64 and rounded once."""
+    w = np.asarray(w, dtype=np.uint32)
+    sine = np.asarray(sine, dtype=bool)
+    R, C, S = normal_tables()
+    x = ((w >> np.uint32(16)) & np.uint32(0x7FFF)).astype(np.int64)
+    a = ((w >> np.uint32(2)) & np.uint32(0x1FFF)).astype(np.int64)
+    trig = np.where(sine, S[a], C[a]).astype(np.float64)
+    mag = (R[x].astype(np.float64) * trig).astype(np.float16)  # numpy rounds float64 -> float16 once, to nearest even
+    neg = np.where(sine, w >> np.uint32(31), (w >> np.uint32(15)) & np.uint32(1)).astype(bool)
+    return np.where(neg, -mag, mag).astype(np.float16)
 
 
 def materialize(seed, num_feature_tiles, P, f0, nf, c0, nc, proj_type):
@@ -180,14 +212,11 @@ def materialize(seed, num_feature_tiles, P, f0, nf, c0, nc, proj_type):
         bitpos = np.where(slot % np.uint32(2) == 1, 31, 15).astype(np.uint32) - shift_index
         bit = (word >> bitpos) & np.uint32(1)
         return np.where(bit == 1, np.float32(1.0), np.float32(-1.0)).astype(np.float32)
-    ctr[..., 0] = off // np.uint32(4)
+    ctr[..., 0] = off // np.uint32(8)
     w = philox4x32_10(ctr, key)
-    e = off % np.uint32(4)
-    wa = np.where(e < 2, w[..., 0], w[..., 2])
-    wb = np.where(e < 2, w[..., 1], w[..., 3])
-    z0, z1 = box_muller_unrounded(wa, wb)
-    z = np.where(e % np.uint32(2) == 1, z1, z0).astype(np.float32)
-    return z.astype(np.float16).astype(np.float32)  # numpy's float16 cast is round-to-nearest-even
+    e = off % np.uint32(8)
+    word = np.take_along_axis(w, (e // np.uint32(2))[..., None].astype(np.int64), axis=-1)[..., 0]
+    return normal_from_word(word, e % np.uint32(2) == 1).astype(np.float32)
 
 
 def project_fp64(G, seed, num_feature_tiles, proj_dim_cols, proj_type, chunk=4096):
@@ -237,8 +266,11 @@ class COracle:
         lib.jlo_tiling.restype = None
         lib.jlo_entry.argtypes = [u32, u32, u64, u64, u32, i32]
         lib.jlo_entry.restype = ctypes.c_float
-        lib.jlo_normal_unrounded.argtypes = [u32, u32, i32]
-        lib.jlo_normal_unrounded.restype = ctypes.c_float
+        lib.jlo_normal_from_word.argtypes = [u32, i32]
+        lib.jlo_normal_from_word.restype = ctypes.c_float
+        for name in ("jlo_radius_half", "jlo_cos_half", "jlo_sin_half"):
+            getattr(lib, name).argtypes = [u32]
+            getattr(lib, name).restype = ctypes.c_uint16
         lib.jlo_half_bits.argtypes = [ctypes.c_float]
         lib.jlo_half_bits.restype = ctypes.c_uint16
         lib.jlo_materialize.argtypes = [u32, u32, u64, u64, u64, u32, u32, i32, fp]
@@ -266,8 +298,17 @@ class COracle:
     def entry(self, seed, tiles, P, f, c, proj_type):
         return float(self.lib.jlo_entry(seed, tiles, P, f, c, proj_type))
 
-    def normal_unrounded(self, wa, wb, second):
-        return float(self.lib.jlo_normal_unrounded(wa, wb, int(second)))
+    def normal_from_word(self, w, sine):
+        return float(self.lib.jlo_normal_from_word(int(w), int(sine)))
+
+    def radius_half(self, x):
+        return int(self.lib.jlo_radius_half(int(x)))
+
+    def cos_half(self, a):
+        return int(self.lib.jlo_cos_half(int(a)))
+
+    def sin_half(self, a):
+        return int(self.lib.jlo_sin_half(int(a)))
 
     def half_bits(self, v):
         return int(self.lib.jlo_half_bits(ctypes.c_float(v)))

@@ -93,24 +93,85 @@ def test_project_matches_numpy_matmul(c_oracle):
         np.testing.assert_allclose(got2, want, rtol=1e-12, atol=1e-12)
 
 
-def test_box_muller_against_float64_math(c_oracle):
+def _ulp16(v):
+    """Spacing of fp16 numbers at |v| (subnormal spacing below 2^-14)."""
+    e = np.floor(np.log2(np.maximum(np.abs(v), 2.0**-14)))
+    return 2.0 ** (e - 10)
+
+
+def test_factor_tables_against_float64_math(c_oracle):
+    # The tables of the normal entries are fp16 roundings of binary32 evaluations of
+    # sqrt(-2 ln u), cos and sin.  A correctly rounded table computed with the float64 math
+    # library can differ only where the exact value sits within the binary32 error (a few 2^-24)
+    # of an fp16 rounding boundary: never by more than one fp16 step, and only rarely at all.
+    R, C, S = npo.normal_tables()
+    assert R.dtype == np.float16 and R.shape == (1 << 15,) and C.shape == S.shape == (1 << 13,)
+    x = np.arange(1 << 15, dtype=np.float64)
+    want_r = np.sqrt(-2.0 * np.log((x + 0.5) / 2.0**15))
+    theta = (np.arange(1 << 13, dtype=np.float64) + 0.5) * (np.pi / 2) / 2.0**13
+    for got, want in ((R, want_r), (C, np.cos(theta)), (S, np.sin(theta))):
+        got64 = got.astype(np.float64)
+        exact = want.astype(np.float16).astype(np.float64)
+        assert np.all(np.abs(got64 - want) <= 0.5 * _ulp16(want) * (1 + 2e-3))
+        assert np.mean(got64 == exact) > 0.998
+    # before the rounding the binary32 sequences are good to a few units in the last place
+    np.testing.assert_allclose(npo.radius_f32(np.arange(1 << 15)), want_r, rtol=4e-7)
+    c32, s32 = npo.cos_sin_f32(np.arange(1 << 13))
+    np.testing.assert_allclose(c32, np.cos(theta), rtol=3e-7)
+    np.testing.assert_allclose(s32, np.sin(theta), rtol=3e-7)
+    # extremes and symmetry: largest radius sqrt(2 * 16 ln 2), mirror image about pi/4
+    assert float(R[0]) == float(np.float16(np.sqrt(32 * np.log(2.0)))) and R[-1] > 0
+    assert np.all(np.diff(R.astype(np.float64)) <= 0)
+    assert np.array_equal(C, S[::-1])
+    # the C oracle holds the same tables
+    for i in list(range(0, 1 << 15, 509)) + [0, 1, (1 << 15) - 1]:
+        assert c_oracle.radius_half(i) == int(R[i].view(np.uint16))
+    for i in list(range(0, 1 << 13, 127)) + [0, 4095, 4096, 8191]:
+        assert c_oracle.cos_half(i) == int(C[i].view(np.uint16))
+        assert c_oracle.sin_half(i) == int(S[i].view(np.uint16))
+
+
+def test_normal_entry_is_box_muller_in_fp16(c_oracle):
+    # entry = +-fp16(R[x] * C[a] or S[a]); against Box-Muller in float64 with the same uniform
+    # u = (x + 1/2) / 2^15 and the same angle: each factor is off by at most 2^-11 of itself (half
+    # an fp16 step), the rounding of the product adds half a step
     rng = np.random.default_rng(7)
-    wa = rng.integers(0, 2**32, size=4000, dtype=np.uint64).astype(np.uint32)
-    wb = rng.integers(0, 2**32, size=4000, dtype=np.uint64).astype(np.uint32)
-    # include the extremes of the radius and all quadrant boundaries
-    wa[:4] = [0, 0xFFFFFFFF, 1 << 31, 0x1FF]
-    wb[:8] = [0, 1 << 30, 1 << 31, 3 << 30, 0xFFFFFFFF, (1 << 30) - 1, 0x3F, 1 << 29]
-    z0, z1 = npo.box_muller_unrounded(wa, wb)
-    u = (2.0 * (wa >> 9).astype(np.float64) + 1.0) / 2.0**24
-    r = np.sqrt(-2.0 * np.log(u))
-    theta = (wb >> 30).astype(np.float64) * (np.pi / 2) + (
-        ((wb >> 6) & 0xFFFFFF).astype(np.float64) - 2.0**23
-    ) * (np.pi / 2) / 2.0**24
-    np.testing.assert_allclose(z0, r * np.cos(theta), rtol=3e-6, atol=1e-6)
-    np.testing.assert_allclose(z1, r * np.sin(theta), rtol=3e-6, atol=1e-6)
-    for i in range(0, 4000, 97):
-        assert c_oracle.normal_unrounded(int(wa[i]), int(wb[i]), 0) == float(z0[i])
-        assert c_oracle.normal_unrounded(int(wa[i]), int(wb[i]), 1) == float(z1[i])
+    w = rng.integers(0, 2**32, size=20_000, dtype=np.uint64).astype(np.uint32)
+    w[:6] = [0, 0xFFFFFFFF, 0x7FFF0000, 0x00007FFC, 0x80008000, 0x7FFF7FFC]
+    x = ((w >> 16) & 0x7FFF).astype(np.float64)
+    a = ((w >> 2) & 0x1FFF).astype(np.float64)
+    r = np.sqrt(-2.0 * np.log((x + 0.5) / 2.0**15))
+    theta = (a + 0.5) * (np.pi / 2) / 2.0**13
+    R, C, S = npo.normal_tables()
+    for sine, trig, sign_bit, tab in ((False, np.cos(theta), 15, C), (True, np.sin(theta), 31, S)):
+        z = npo.normal_from_word(w, np.full(w.shape, sine))
+        assert z.dtype == np.float16
+        sign = np.where((w >> sign_bit) & 1, -1.0, 1.0)
+        want = sign * r * trig
+        err = np.abs(z.astype(np.float64) - want)
+        assert np.all(err <= (2.0**-10 * np.abs(want) + 0.5 * _ulp16(want)) * (1 + 1e-3))
+        assert np.median(err / _ulp16(want)) < 0.5
+        # the definition itself, restated with exact rational arithmetic on a sample
+        from fractions import Fraction
+        for i in range(0, 20_000, 401):
+            p = Fraction(float(R[int(x[i])])) * Fraction(float(tab[int(a[i])]))
+            lo = np.float16(float(p))  # float(p) is exact (22 significant bits)
+            assert float(z[i]) == float(sign[i]) * float(lo)
+            assert c_oracle.normal_from_word(int(w[i]), sine) == float(z[i])
+
+
+def test_normal_block_uses_every_word_for_one_pair(c_oracle):
+    # one tile of 8 features = one Philox block: entries (2i, 2i + 1) come from word i
+    seed, col = 5, 9
+    words = c_oracle.philox([0, 0, 0, 0], [c_oracle.stream_seed(seed, col, 0), 0])
+    colv = c_oracle.materialize(seed, 1, 8, 0, 8, col, 1, G)[:, 0]
+    for e in range(8):
+        assert colv[e] == c_oracle.normal_from_word(words[e // 2], e % 2)
+    # and the second block of the stream serves features 8..15
+    words1 = c_oracle.philox([1, 0, 0, 0], [c_oracle.stream_seed(seed, col, 0), 0])
+    colv = c_oracle.materialize(seed, 1, 16, 8, 8, col, 1, G)[:, 0]
+    for e in range(8):
+        assert colv[e] == c_oracle.normal_from_word(words1[e // 2], e % 2)
 
 
 def test_half_rounding_matches_numpy_float16(c_oracle):
@@ -137,5 +198,10 @@ def test_normal_entries_are_fp16_standard_normals(c_oracle):
 
     assert stats.kstest(S.ravel()[:50_000], "norm").pvalue > 1e-3
     # the cos and sin branches of one pair are uncorrelated, so are neighbouring columns
-    assert abs(np.corrcoef(S[0::4].ravel(), S[1::4].ravel())[0, 1]) < 5 / math.sqrt(n / 4)
+    assert abs(np.corrcoef(S[0::2].ravel(), S[1::2].ravel())[0, 1]) < 5 / math.sqrt(n / 2)
+    # and their squares add up to the squared radius: chi-square with two degrees of freedom
+    r2 = S[0::2].ravel() ** 2 + S[1::2].ravel() ** 2
+    assert stats.kstest(r2[:50_000], "chi2", args=(2,)).pvalue > 1e-3
+    # tails: the radius grid ends at sqrt(32 ln 2) = 4.71
+    assert np.abs(S).max() <= 4.72 and np.abs(S).max() > 3.5
     assert abs(np.corrcoef(S[:, 0], S[:, 1])[0, 1]) < 5 / math.sqrt(S.shape[0])

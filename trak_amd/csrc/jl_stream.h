@@ -12,7 +12,7 @@
 //     (fast_jl/random.cuh:15-17);
 //   * entries are consumed in feature order inside a tile; a Rademacher entry
 //     costs one random bit, bit set -> +1 (fast_jl/random.cuh:33-37); a normal
-//     entry is a Box-Muller normal rounded to fp16 (fast_jl/random.cuh:50-60).
+//     entry is a Box-Muller normal in fp16 (fast_jl/random.cuh:50-60).
 //
 // What is new: the generator is Philox4x32-10 (the reference uses cuRAND XORWOW,
 // whose draws cannot be reproduced off an NVIDIA toolchain).  The stream of
@@ -26,12 +26,17 @@
 //   32x32x16 MFMA in bit 15 / bit 31 of (word << q), which is where the sign
 //   bits of a packed pair of 16-bit floats live.
 //
-// Normal: feature offset o uses block n = o / 4; words (0,1) give entries
-//   o%4 == 0 (cos branch) and 1 (sin branch), words (2,3) give 2 and 3.  The
-//   Box-Muller transform is spelled out below in IEEE binary32 operations
-//   (add, mul, fma, int<->float conversions of exactly representable values)
-//   so that any IEEE machine reproduces it bit for bit; the result is rounded
-//   to fp16 (round to nearest even).
+// Normal: feature offset o uses block n = o / 8; word (o % 8) / 2 of the block makes the
+//   Box-Muller pair of entries o % 8 = 2i (cosine) and 2i + 1 (sine):
+//       entry = +-fp16( R[x] * C[a] )   resp.   +-fp16( R[x] * S[a] )
+//   with a 15-bit radius index x, a 13-bit angle index a and two sign bits taken from the word,
+//       R[x] = fp16( sqrt(-2 ln((x + 1/2) / 2^15)) ),
+//       C[a], S[a] = fp16( cos, sin of (a + 1/2) * (pi/2) / 2^13 ),
+//   i.e. a uniform angle on a grid of 2^15 directions around the circle (quadrant by the two
+//   signs).  R, C and S are spelled out below in IEEE binary32 operations (add, mul, fma,
+//   int<->float conversions of exactly representable values) and rounded to fp16 (nearest even),
+//   so any IEEE machine reproduces them bit for bit; the product of the two fp16 factors is
+//   exact in binary32 and is rounded once.  The kernel keeps R and (C, S) as tables in LDS.
 #pragma once
 #include <stdint.h>
 
@@ -139,10 +144,10 @@ JL_HD float jl_add_(float a, float b) {
 #define JL_ADD(a, b) jl::jl_add_((a), (b))
 #endif
 
-// Radius r = sqrt(-2 ln u), u = (2*(w >> 9) + 1) / 2^24 in (0, 1).
-JL_HD float bm_radius(uint32_t w) {
-    const uint32_t x = ((w >> 9) << 1) | 1u;  // odd, < 2^24: exact as float
-    const uint32_t xb = f2u((float)x);
+// Radius table entry: r = sqrt(-2 ln u), u = (2x + 1) / 2^16 in (0, 1), for a 15-bit index x.
+JL_HD float bm_radius(uint32_t x) {
+    const uint32_t odd = (x << 1) | 1u;  // < 2^16: exact as float
+    const uint32_t xb = f2u((float)odd);
     int e = (int)(xb >> 23) - 127;
     float m = u2f((xb & 0x007FFFFFu) | 0x3F800000u);  // [1, 2)
     if (m > 1.41421354f) {
@@ -163,7 +168,7 @@ JL_HD float bm_radius(uint32_t w) {
     float y = JL_MUL(t, JL_MUL(z, p));
     y = JL_FMA(-0.5f, z, y);
     const float lnm = JL_ADD(t, y);
-    const float lnu = JL_FMA((float)(e - 24), 0.693147182f, lnm);
+    const float lnu = JL_FMA((float)(e - 16), 0.693147182f, lnm);
     const float s = JL_MUL(-2.0f, lnu);
     // sqrt(s) by three Newton steps on 1/sqrt(s) from an integer seed
     float g = u2f(0x5f3759dfu - (f2u(s) >> 1));
@@ -177,11 +182,13 @@ JL_HD float bm_radius(uint32_t w) {
     return JL_MUL(s, g);
 }
 
-// cos and sin of the angle  (w >> 30) * pi/2 + (((w >> 6) & 0xFFFFFF) - 2^23) * (pi/2) / 2^24.
-JL_HD void bm_cossin(uint32_t w, float* c_out, float* s_out) {
-    const uint32_t qd = w >> 30;
-    const float fi = (float)((w >> 6) & 0x00FFFFFFu);
-    const float yv = JL_MUL(JL_ADD(fi, -8388608.0f), 9.36266447e-8f);  // (pi/2) * 2^-24
+// Angle table entry: cos and sin of theta = (a + 1/2) * (pi/2) / 2^13 in (0, pi/2) for a 13-bit
+// index a.  The upper half of the range is the mirror image of the lower one (cos <-> sin), so
+// the polynomials only see (0, pi/4).
+JL_HD void bm_cossin(uint32_t a, float* c_out, float* s_out) {
+    const bool mirror = a >= 4096u;
+    const uint32_t am = mirror ? 8191u - a : a;
+    const float yv = JL_MUL(JL_ADD((float)am, 0.5f), 1.91747604e-4f);  // pi / 2^14
     const float y2 = JL_MUL(yv, yv);
     float ps = JL_FMA(-1.9515295891e-4f, y2, 8.3321608736e-3f);
     ps = JL_FMA(ps, y2, -1.6666654611e-1f);
@@ -189,21 +196,8 @@ JL_HD void bm_cossin(uint32_t w, float* c_out, float* s_out) {
     float pc = JL_FMA(2.443315711809948e-5f, y2, -1.388731625493765e-3f);
     pc = JL_FMA(pc, y2, 4.166664568298827e-2f);
     const float cs = JL_FMA(JL_MUL(pc, y2), y2, JL_FMA(-0.5f, y2, 1.0f));
-    const float c0 = (qd & 1u) ? sn : cs;
-    const float s0 = (qd & 1u) ? cs : sn;
-    const uint32_t negc = (((qd + 1u) >> 1) & 1u) << 31;
-    const uint32_t negs = (qd >> 1) << 31;
-    *c_out = u2f(f2u(c0) ^ negc);
-    *s_out = u2f(f2u(s0) ^ negs);
-}
-
-// The two binary32 normals of one word pair (before the rounding to fp16).
-JL_HD void bm_pair(uint32_t wa, uint32_t wb, float* z0, float* z1) {
-    const float r = bm_radius(wa);
-    float c, s;
-    bm_cossin(wb, &c, &s);
-    *z0 = JL_MUL(r, c);
-    *z1 = JL_MUL(r, s);
+    *c_out = mirror ? sn : cs;
+    *s_out = mirror ? cs : sn;
 }
 
 // binary32 -> binary16 bit pattern, round to nearest even (|v| < 65504 here, no NaN).  On the
@@ -263,15 +257,32 @@ JL_HD float entry_rademacher(uint32_t sseed, uint32_t o) {
     return rademacher_bit(b, o & 127u) ? 1.0f : -1.0f;
 }
 
+// The fields of one random word: it makes one Box-Muller pair.
+//   bits 16..30  radius index x          bit 31  sign of the sine entry
+//   bits  2..14  angle index a           bit 15  sign of the cosine entry      (bits 0, 1 unused)
+JL_HD uint32_t normal_radius_index(uint32_t w) { return (w >> 16) & 0x7FFFu; }
+JL_HD uint32_t normal_angle_index(uint32_t w) { return (w >> 2) & 0x1FFFu; }
+
+// fp16 product of two fp16 values, round to nearest even (the product is exact in binary32).
+JL_HD uint16_t f16_mul_rne(uint16_t a, uint16_t b) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    const _Float16 p = __builtin_bit_cast(_Float16, a) * __builtin_bit_cast(_Float16, b);
+    return __builtin_bit_cast(uint16_t, p);
+#else
+    return f32_to_f16_rne(JL_MUL(f16_bits_to_f32(a), f16_bits_to_f32(b)));
+#endif
+}
+
 JL_HD uint16_t entry_normal_f16bits(uint32_t sseed, uint32_t o) {
-    const u32x4 b = stream_block(sseed, o >> 2);
-    const uint32_t e = o & 3u;
-    float z0, z1;
-    if (e < 2u)
-        bm_pair(b.x, b.y, &z0, &z1);
-    else
-        bm_pair(b.z, b.w, &z0, &z1);
-    return f32_to_f16_rne((e & 1u) ? z1 : z0);
+    const u32x4 b = stream_block(sseed, o >> 3);
+    const uint32_t e = o & 7u;
+    const uint32_t w = word_of(b, e >> 1);
+    const uint16_t r = f32_to_f16_rne(bm_radius(normal_radius_index(w)));
+    float c, s;
+    bm_cossin(normal_angle_index(w), &c, &s);
+    const uint16_t t = f32_to_f16_rne((e & 1u) ? s : c);
+    const uint16_t sign = (uint16_t)(((e & 1u) ? (w >> 31) : (w >> 15)) << 15);
+    return (uint16_t)(f16_mul_rne(r, t) ^ sign);
 }
 
 JL_HD float entry_normal(uint32_t sseed, uint32_t o) {

@@ -368,39 +368,6 @@ __device__ __forceinline__ uint32_t sign_pair(uint32_t m, uint32_t one) {
     return __builtin_amdgcn_bitop3_b32(m, one, one | 0x80008000u, 0xCA);
 }
 
-__device__ __forceinline__ uint32_t pack_f16(float a, float b) {
-    return (uint32_t)jl::f32_to_f16_rne(a) | ((uint32_t)jl::f32_to_f16_rne(b) << 16);
-}
-
-// The 8 normal entries of offsets o0..o0+7 (o0 multiple of 8) as packed fp16.
-__device__ __forceinline__ uint4 normal_oct_f16(uint32_t sseed, uint32_t o0) {
-    const jl::u32x4 b0 = jl::stream_block(sseed, (o0 >> 2));
-    const jl::u32x4 b1 = jl::stream_block(sseed, (o0 >> 2) + 1u);
-    float z[8];
-    jl::bm_pair(b0.x, b0.y, &z[0], &z[1]);
-    jl::bm_pair(b0.z, b0.w, &z[2], &z[3]);
-    jl::bm_pair(b1.x, b1.y, &z[4], &z[5]);
-    jl::bm_pair(b1.z, b1.w, &z[6], &z[7]);
-    uint4 r;
-    r.x = pack_f16(z[0], z[1]);
-    r.y = pack_f16(z[2], z[3]);
-    r.z = pack_f16(z[4], z[5]);
-    r.w = pack_f16(z[6], z[7]);
-    return r;
-}
-
-// Split packed fp16 pairs into bf16 high and low terms (s = hi + lo exactly).
-__device__ __forceinline__ void f16pair_to_bf16_terms(uint32_t hp, uint32_t& hi, uint32_t& lo) {
-    const float a = jl::f16_bits_to_f32((uint16_t)(hp & 0xFFFFu));
-    const float b = jl::f16_bits_to_f32((uint16_t)(hp >> 16));
-    const uint32_t ah = __float_as_uint(a) & 0xFFFF0000u;
-    const uint32_t bh = __float_as_uint(b) & 0xFFFF0000u;
-    const float al = a - __uint_as_float(ah);
-    const float bl = b - __uint_as_float(bh);
-    hi = (ah >> 16) | bh;
-    lo = (__float_as_uint(al) >> 16) | (__float_as_uint(bl) & 0xFFFF0000u);
-}
-
 // Workgroup id -> (column block, tile).  Workgroups are handed to the 8 XCDs round-robin
 // by linear id; this puts the column blocks of one feature tile on the same XCD, next to
 // each other in time, so the tile is fetched from HBM once and then served by that XCD's L2.
@@ -440,7 +407,7 @@ __device__ __forceinline__ uint4 signs_of(uint64_t m01, uint64_t m23, uint32_t o
 
 // GATHER: g_in is a device array of trakhip_segment and ld their number; otherwise g_in is the
 // dense [rows, P] matrix with row pitch ld.
-template <int IN, int PT, bool GATHER, int W>
+template <int IN, bool GATHER, int W>
 __global__ __launch_bounds__(64 * W, 2) void jl_project_kernel(
     const void* __restrict__ g_in, uint64_t ld, uint32_t rows, uint64_t P, uint32_t k,
     uint32_t seed, uint32_t tiles, uint64_t tile_size, uint32_t chunks_per_tile,
@@ -524,72 +491,43 @@ __global__ __launch_bounds__(64 * W, 2) void jl_project_kernel(
                         tid);
             const uint16_t* a_base = lds + cur * kBufElems + a_off;
 
-            if (PT == TRAKHIP_RADEMACHER) {
-                uint64_t w01[kGroups], w23[kGroups];
+            uint64_t w01[kGroups], w23[kGroups];
+#pragma unroll
+            for (int j = 0; j < kGroups; ++j) {
+                const jl::u32x4 w = jl::stream_block(sseed[j], 2u * s + h);
+                w01[j] = ((uint64_t)w.y << 32) | w.x;
+                w23[j] = ((uint64_t)w.w << 32) | w.z;
+            }
+            // 64 steps (q, j).  Issue order per step: shifts of the NEXT operand, MFMA of this
+            // step, sign expansion of the next operand.  The MFMA then never directly follows
+            // the VALU instructions that wrote its operand (no wait states to pad).
+            uint64_t m01, m23;
+            shifted_pairs(w01[0], w23[0], 0, m01, m23);
+            uint4 b = signs_of(m01, m23, one);
+            uint4 a[2][kPlanes];  // A operands of this q and of the next one (read one q ahead)
+#pragma unroll
+            for (int pl = 0; pl < kPlanes; ++pl)
+                a[0][pl] = *reinterpret_cast<const uint4*>(a_base + pl * kPlaneElems);
+#pragma unroll
+            for (int q = 0; q < 16; ++q) {
 #pragma unroll
                 for (int j = 0; j < kGroups; ++j) {
-                    const jl::u32x4 w = jl::stream_block(sseed[j], 2u * s + h);
-                    w01[j] = ((uint64_t)w.y << 32) | w.x;
-                    w23[j] = ((uint64_t)w.w << 32) | w.z;
-                }
-                // 64 steps (q, j).  Issue order per step: shifts of the NEXT operand, MFMA of this
-                // step, sign expansion of the next operand.  The MFMA then never directly follows
-                // the VALU instructions that wrote its operand (no wait states to pad).
-                uint64_t m01, m23;
-                shifted_pairs(w01[0], w23[0], 0, m01, m23);
-                uint4 b = signs_of(m01, m23, one);
-                uint4 a[2][kPlanes];  // A operands of this q and of the next one (read one q ahead)
+                    const int step = q * kGroups + j;
+                    const bool last = step + 1 == 16 * kGroups;
+                    if (!last) shifted_pairs(w01[(step + 1) % kGroups], w23[(step + 1) % kGroups],
+                                             (step + 1) / kGroups, m01, m23);
+                    if (j == 0 && q + 1 < 16) {
 #pragma unroll
-                for (int pl = 0; pl < kPlanes; ++pl)
-                    a[0][pl] = *reinterpret_cast<const uint4*>(a_base + pl * kPlaneElems);
-#pragma unroll
-                for (int q = 0; q < 16; ++q) {
-#pragma unroll
-                    for (int j = 0; j < kGroups; ++j) {
-                        const int step = q * kGroups + j;
-                        const bool last = step + 1 == 16 * kGroups;
-                        if (!last) shifted_pairs(w01[(step + 1) % kGroups], w23[(step + 1) % kGroups],
-                                                 (step + 1) / kGroups, m01, m23);
-                        if (j == 0 && q + 1 < 16) {
-#pragma unroll
-                            for (int pl = 0; pl < kPlanes; ++pl)
-                                a[(q + 1) & 1][pl] =
-                                    *reinterpret_cast<const uint4*>(a_base + pl * kPlaneElems + 8 * (q + 1));
-                        }
-                        __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-                        for (int pl = 0; pl < kPlanes; ++pl) acc[j] = mfma16(a[q & 1][pl], b, acc[j], kBf);
-                        __builtin_amdgcn_sched_barrier(0);
-                        if (!last) b = signs_of(m01, m23, one);
-                        __builtin_amdgcn_sched_barrier(0);
+                        for (int pl = 0; pl < kPlanes; ++pl)
+                            a[(q + 1) & 1][pl] =
+                                *reinterpret_cast<const uint4*>(a_base + pl * kPlaneElems + 8 * (q + 1));
                     }
-                }
-            } else {
-                const uint32_t o_chunk = s * (uint32_t)kChunk + 128u * h;
-#pragma unroll 1
-                for (int q = 0; q < 16; ++q) {
-                    uint4 a[kPlanes];
+                    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-                    for (int pl = 0; pl < kPlanes; ++pl)
-                        a[pl] = *reinterpret_cast<const uint4*>(a_base + pl * kPlaneElems + 8 * q);
-#pragma unroll
-                    for (int j = 0; j < kGroups; ++j) {
-                        const uint4 bh = normal_oct_f16(sseed[j], o_chunk + 8u * q);
-                        if (!kBf) {
-                            acc[j] = mfma16(a[0], bh, acc[j], false);
-                        } else {
-                            uint4 hi, lo;
-                            f16pair_to_bf16_terms(bh.x, hi.x, lo.x);
-                            f16pair_to_bf16_terms(bh.y, hi.y, lo.y);
-                            f16pair_to_bf16_terms(bh.z, hi.z, lo.z);
-                            f16pair_to_bf16_terms(bh.w, hi.w, lo.w);
-#pragma unroll
-                            for (int pl = 0; pl < kPlanes; ++pl) {
-                                acc[j] = mfma16(a[pl], hi, acc[j], true);
-                                acc[j] = mfma16(a[pl], lo, acc[j], true);
-                            }
-                        }
-                    }
+                    for (int pl = 0; pl < kPlanes; ++pl) acc[j] = mfma16(a[q & 1][pl], b, acc[j], kBf);
+                    __builtin_amdgcn_sched_barrier(0);
+                    if (!last) b = signs_of(m01, m23, one);
+                    __builtin_amdgcn_sched_barrier(0);
                 }
             }
 
@@ -611,6 +549,321 @@ __global__ __launch_bounds__(64 * W, 2) void jl_project_kernel(
         for (int r = 0; r < 16; ++r) {
             const uint32_t m = 8u * (r >> 2) + 4u * h + (r & 3);
             if (m < rows) out[(uint64_t)m * k + col0 + 32u * j] = acc[j][r];
+        }
+    }
+}
+
+// ---- normal (Gaussian) projection ------------------------------------------------------------
+//
+// Same decomposition as the Rademacher kernel (8 waves, 32-column groups, 256-feature chunks,
+// lane half h owns features [128h, 128h + 128) of a chunk), but the cost sits elsewhere: a matrix
+// entry is used for 32 multiply-adds only, and making one costs about ten vector instructions
+// (Philox4x32-10: one block per eight entries) against 1.5 for a sign, so the kernel is bound by
+// the vector ALU, not by the matrix pipe.  What keeps the count that low:
+//   * one random word makes a whole Box-Muller pair: the radius R[x] and the pair (C[a], S[a])
+//     come out of two LDS tables (64 KB + 32 KB, filled at kernel start from the binary32
+//     sequences of jl_stream.h), one v_pk_mul_f16 multiplies and rounds both entries, one
+//     v_bitop3_b32 applies the two sign bits;
+//   * the matrix entries are fp16 whatever the gradient type is, so the gradients are brought to
+//     fp16 once per chunk at staging time instead of splitting every entry into bf16 terms in the
+//     hot loop: bf16 and fp32 chunks are multiplied row by row by the power of two that puts the
+//     row's largest magnitude into [2^14, 2^15) (bf16: one exact fp16 plane for everything within
+//     2^-31 of it; fp32: two planes h1 + h2, 22 significant bits), the accumulators follow the
+//     row's factor from chunk to chunk (v_ldexp_f32, exact) and the factor is taken out again
+//     before the partial sums are written.
+
+typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+typedef unsigned short ushort2_t __attribute__((ext_vector_type(2)));
+
+constexpr int kRadiusEntries = 1 << 15;
+constexpr int kAngleEntries = 1 << 13;
+#ifndef JL_NORMAL_UNROLL
+#define JL_NORMAL_UNROLL 1
+#endif
+constexpr int kNormalUnroll = JL_NORMAL_UNROLL;  // MFMA steps of the hot loop unrolled together
+
+template <int IN>
+struct NormalTraits;
+template <>
+struct NormalTraits<TRAKHIP_F16> {
+    static constexpr int planes = 1, buffers = 2;
+    static constexpr bool scaled = false;
+};
+template <>
+struct NormalTraits<TRAKHIP_BF16> {
+    static constexpr int planes = 1, buffers = 2;
+    static constexpr bool scaled = true;
+};
+template <>
+struct NormalTraits<TRAKHIP_F32> {
+    static constexpr int planes = 2, buffers = 1;  // x * 2^sh = h1 + h2 (+ at most 2^-22 of it)
+    static constexpr bool scaled = true;
+};
+
+// Power of two that brings a row whose largest binary32 exponent field is emax into [2^14, 2^15);
+// an all-zero (or all-subnormal) row keeps its scale.
+__device__ __forceinline__ int row_shift(uint32_t emax) { return emax ? 141 - (int)emax : 0; }
+
+// Slot of row m in the per-chunk exponent lists: lane half h reads its sixteen accumulator rows
+// m = 8*(r/4) + 4*h + r%4 (r = 0..15) as sixteen consecutive ints.
+__device__ __forceinline__ int row_slot(uint32_t row) { return ((row >> 2) & 1) * 16 + (row >> 3) * 4 + (row & 3); }
+
+__device__ __forceinline__ uint32_t pack_f16_rne(float a, float b) {
+    const half2_t v = {(_Float16)a, (_Float16)b};
+    return __builtin_bit_cast(uint32_t, v);
+}
+
+// bf16 chunk -> one scaled fp16 plane.  The 32 threads that share tid / 32 hold one row (two rows
+// per thread, 16 apart); sh_prev[] is the row's exponent in the previous chunk.
+__device__ __forceinline__ void store_scaled_bf16(const uint4 (&v)[2], uint16_t* lds, int (*sh)[32], int tid,
+                                                  int (&sh_prev)[2]) {
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        const uint32_t row = (tid >> 5) + 16 * i, sg = tid & 31;
+        const uint32_t w[4] = {v[i].x, v[i].y, v[i].z, v[i].w};
+        ushort2_t m = __builtin_bit_cast(ushort2_t, w[0] & 0x7F807F80u);
+#pragma unroll
+        for (int t = 1; t < 4; ++t) m = __builtin_elementwise_max(m, __builtin_bit_cast(ushort2_t, w[t] & 0x7F807F80u));
+        uint32_t e = m[0] > m[1] ? m[0] : m[1];
+#pragma unroll
+        for (int d = 1; d < 32; d <<= 1) {
+            const uint32_t o = (uint32_t)__shfl_xor((int)e, d, 64);
+            e = o > e ? o : e;
+        }
+        const int shift = row_shift(e >> 7);
+        uint32_t h[4];
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+            h[t] = pack_f16_rne(ldexpf(__uint_as_float(w[t] << 16), shift),
+                                ldexpf(__uint_as_float(w[t] & 0xFFFF0000u), shift));
+        *reinterpret_cast<uint4*>(lds + row * kLdsRow + 8 * sg) = uint4{h[0], h[1], h[2], h[3]};
+        if (sg == 0) {
+            sh[0][row_slot(row)] = shift - sh_prev[i];
+            sh[1][row_slot(row)] = shift;
+        }
+        sh_prev[i] = shift;
+    }
+}
+
+// fp32 chunk -> two scaled fp16 planes.  The 64 threads of a wave hold one row (four rows per
+// thread, 8 apart).
+__device__ __forceinline__ void store_scaled_f32(const uint4 (&v)[4], uint16_t* lds, int (*sh)[32], int tid,
+                                                 int (&sh_prev)[4]) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const uint32_t row = (tid >> 6) + 8 * i, sg = tid & 63;
+        const uint32_t w[4] = {v[i].x, v[i].y, v[i].z, v[i].w};
+        uint32_t e = 0;
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            const uint32_t x = (w[t] >> 23) & 0xFFu;
+            e = x > e ? x : e;
+        }
+#pragma unroll
+        for (int d = 1; d < 64; d <<= 1) {
+            const uint32_t o = (uint32_t)__shfl_xor((int)e, d, 64);
+            e = o > e ? o : e;
+        }
+        const int shift = row_shift(e);
+        float g[4], r[4];
+        _Float16 h1[4];
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            g[t] = ldexpf(__uint_as_float(w[t]), shift);
+            h1[t] = (_Float16)g[t];
+            r[t] = g[t] - (float)h1[t];  // exact
+        }
+        const half2_t a0 = {h1[0], h1[1]}, a1 = {h1[2], h1[3]};
+        *reinterpret_cast<uint2*>(lds + row * kLdsRow + 4 * sg) =
+            uint2{__builtin_bit_cast(uint32_t, a0), __builtin_bit_cast(uint32_t, a1)};
+        *reinterpret_cast<uint2*>(lds + kPlaneElems + row * kLdsRow + 4 * sg) =
+            uint2{pack_f16_rne(r[0], r[1]), pack_f16_rne(r[2], r[3])};
+        if (sg == 0) {
+            sh[0][row_slot(row)] = shift - sh_prev[i];
+            sh[1][row_slot(row)] = shift;
+        }
+        sh_prev[i] = shift;
+    }
+}
+
+// The Box-Muller pair of one random word as packed fp16 (cosine entry low, sine entry high):
+// fields of the word as in jl_stream.h (radius index bits 16..30, angle index bits 2..14, signs
+// bits 15 and 31).  r_tab holds fp16 R[x], cs_tab the packed fp16 pairs (C[a], S[a]).
+__device__ __forceinline__ uint32_t normal_pair(uint32_t w, const char* r_tab, const char* cs_tab) {
+    const _Float16 r = *reinterpret_cast<const _Float16*>(r_tab + ((w >> 15) & 0xFFFEu));
+    const uint32_t cs = *reinterpret_cast<const uint32_t*>(cs_tab + (w & 0x7FFCu));
+    const half2_t rr = {r, r};
+    const half2_t z = rr * __builtin_bit_cast(half2_t, cs);  // v_pk_mul_f16: exact products, rounded once
+    // z ^ (w & 0x80008000): truth table of a ^ (b & c)
+    return __builtin_amdgcn_bitop3_b32(__builtin_bit_cast(uint32_t, z), w, 0x80008000u, 0x78);
+}
+
+// GPW = 32-column groups per wave: 4 (workgroup = 1024 columns) or 2 (512 columns, for projection
+// dimensions that are an odd multiple of 512).  Always 8 waves; arguments as jl_project_kernel.
+template <int IN, bool GATHER, int GPW>
+__global__ __launch_bounds__(512, 2) void jl_project_normal_kernel(
+    const void* __restrict__ g_in, uint64_t ld, uint32_t rows, uint64_t P, uint32_t k, uint32_t seed,
+    uint32_t tiles, uint64_t tile_size, uint32_t chunks_per_tile, uint32_t chunks_per_group,
+    float* __restrict__ partial) {
+    constexpr int W = 8;
+    typedef NormalTraits<IN> Tr;
+    typedef typename StageOf<IN, GATHER, W>::type Stage;
+    typedef typename StageOf<IN, GATHER, W>::elem Elem;
+    constexpr int kColsPerWG = W * GPW * 32;
+    constexpr int kPlanes = Tr::planes;
+    constexpr int kBuffers = Tr::buffers;
+    constexpr int kBufElems = kPlanes * kPlaneElems;
+    constexpr bool kScaled = Tr::scaled;
+
+    __shared__ __attribute__((aligned(16))) uint16_t lds[kBuffers * kBufElems];
+    __shared__ __attribute__((aligned(16))) uint16_t r_tab[kRadiusEntries];
+    __shared__ __attribute__((aligned(16))) uint32_t cs_tab[kAngleEntries];
+    __shared__ __attribute__((aligned(16))) int sh_lds[kBuffers][2][32];  // per row: change of exponent, exponent
+
+    const uint32_t col_blocks = k / kColsPerWG;
+    uint32_t cb, group;
+    map_workgroup(blockIdx.x, col_blocks, cb, group);
+    const uint64_t total_chunks = (uint64_t)tiles * chunks_per_tile;
+    const uint64_t c_begin = (uint64_t)group * chunks_per_group;
+    if (c_begin >= total_chunks) return;  // padding of the group count to a multiple of 8
+    const uint64_t c_end = c_begin + chunks_per_group < total_chunks ? c_begin + chunks_per_group : total_chunks;
+    const uint32_t t0 = (uint32_t)(c_begin / chunks_per_tile), s0 = (uint32_t)(c_begin % chunks_per_tile);
+    const uint32_t t_last = (uint32_t)((c_end - 1) / chunks_per_tile);
+    const uint32_t s_last_end = (uint32_t)((c_end - 1) % chunks_per_tile) + 1;
+
+    const int tid = threadIdx.x;
+    const int wave = tid >> 6, lane = tid & 63;
+    const uint32_t n = lane & 31, h = lane >> 5;
+    const uint32_t col0 = cb * kColsPerWG + wave * (GPW * 32) + n;
+
+    // the two tables; the first barrier below publishes them
+    for (int i = tid; i < kRadiusEntries; i += 64 * W) r_tab[i] = jl::f32_to_f16_rne(jl::bm_radius((uint32_t)i));
+    for (int i = tid; i < kAngleEntries; i += 64 * W) {
+        float c, sn;
+        jl::bm_cossin((uint32_t)i, &c, &sn);
+        cs_tab[i] = (uint32_t)jl::f32_to_f16_rne(c) | ((uint32_t)jl::f32_to_f16_rne(sn) << 16);
+    }
+    const char* rt = reinterpret_cast<const char*>(r_tab);
+    const char* ct = reinterpret_cast<const char*>(cs_tab);
+
+    floatx16 acc[GPW];
+#pragma unroll
+    for (int j = 0; j < GPW; ++j)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[j][r] = 0.0f;
+
+    const Elem* g = reinterpret_cast<const Elem*>(g_in);
+    const uint32_t a_off = n * kLdsRow + 128 * h;
+
+    Stage st;
+    int sh_prev[Stage::N];
+#pragma unroll
+    for (int i = 0; i < Stage::N; ++i) sh_prev[i] = 0;
+    auto stage_store = [&](int buf) {
+        if constexpr (IN == TRAKHIP_F16)
+            st.store(lds + buf * kBufElems, tid);
+        else if constexpr (IN == TRAKHIP_BF16)
+            store_scaled_bf16(st.v, lds + buf * kBufElems, sh_lds[buf], tid, sh_prev);
+        else
+            store_scaled_f32(st.v, lds + buf * kBufElems, sh_lds[buf], tid, sh_prev);
+    };
+    {
+        const uint64_t lo = (uint64_t)t0 * tile_size;
+        const uint64_t hi = (lo + tile_size < P) ? lo + tile_size : P;
+        if constexpr (GATHER) st.init(g, (uint32_t)ld, lo + (uint64_t)s0 * kChunk, P, tid);
+        st.load(g, ld, rows, lo + (uint64_t)s0 * kChunk, hi, tid);
+    }
+    int cur = 0, last = 0;
+    if (kBuffers == 2) {
+        stage_store(0);
+        __syncthreads();
+    }
+
+    for (uint32_t tile = t0; tile <= t_last; ++tile) {
+        const uint64_t f_lo = (uint64_t)tile * tile_size;
+        const uint64_t f_hi = (f_lo + tile_size < P) ? f_lo + tile_size : P;
+        const uint32_t s_begin = tile == t0 ? s0 : 0u;
+        const uint32_t chunks = tile == t_last ? s_last_end : chunks_per_tile;
+        const uint64_t nf_lo = f_lo + tile_size;
+        const uint64_t nf_hi = (nf_lo + tile_size < P) ? nf_lo + tile_size : P;
+
+        uint32_t sseed[GPW];
+#pragma unroll
+        for (int j = 0; j < GPW; ++j) sseed[j] = jl::stream_seed(seed, col0 + 32u * j, tile);
+
+        for (uint32_t s = s_begin; s < chunks; ++s) {
+            const bool more_here = s + 1 < chunks;
+            const bool more = more_here || tile < t_last;
+            if (kBuffers == 1) {
+                __syncthreads();  // everyone is done reading the previous chunk
+                stage_store(0);
+                __syncthreads();
+            }
+            if (more)
+                st.load(g, ld, rows, more_here ? f_lo + (uint64_t)(s + 1) * kChunk : nf_lo, more_here ? f_hi : nf_hi,
+                        tid);
+            const uint16_t* a_base = lds + cur * kBufElems + a_off;
+
+            if (kScaled) {
+                // the rows of this chunk carry other powers of two than those of the last one
+                const int4* dp = reinterpret_cast<const int4*>(&sh_lds[cur][0][16 * h]);
+                int d[16];
+#pragma unroll
+                for (int t = 0; t < 4; ++t) {
+                    const int4 x = dp[t];
+                    d[4 * t] = x.x, d[4 * t + 1] = x.y, d[4 * t + 2] = x.z, d[4 * t + 3] = x.w;
+                }
+#pragma unroll
+                for (int j = 0; j < GPW; ++j)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) acc[j][r] = ldexpf(acc[j][r], d[r]);
+            }
+
+            // Philox block of (column, offset o): o / 8 with o = 256 s + 128 h + 8 q
+            const uint32_t n0 = 32u * s + 16u * h;
+#pragma unroll kNormalUnroll
+            for (int q = 0; q < 16; ++q) {
+                uint4 a[kPlanes];
+#pragma unroll
+                for (int pl = 0; pl < kPlanes; ++pl)
+                    a[pl] = *reinterpret_cast<const uint4*>(a_base + pl * kPlaneElems + 8 * q);
+#pragma unroll
+                for (int j = 0; j < GPW; ++j) {
+                    const jl::u32x4 blk = jl::stream_block(sseed[j], n0 + (uint32_t)q);
+                    const uint4 b = {normal_pair(blk.x, rt, ct), normal_pair(blk.y, rt, ct),
+                                     normal_pair(blk.z, rt, ct), normal_pair(blk.w, rt, ct)};
+#pragma unroll
+                    for (int pl = 0; pl < kPlanes; ++pl) acc[j] = mfma16(a[pl], b, acc[j], false);
+                }
+            }
+
+            last = cur;
+            if (kBuffers == 2) {
+                if (more) stage_store(cur ^ 1);
+                __syncthreads();
+                cur ^= 1;
+            }
+        }
+    }
+
+    float* out = partial + (uint64_t)group * rows * k;
+    int ex[16];
+#pragma unroll
+    for (int r = 0; r < 16; ++r) ex[r] = 0;
+    if (kScaled) {
+        const int4* ep = reinterpret_cast<const int4*>(&sh_lds[last][1][16 * h]);
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            const int4 x = ep[t];
+            ex[4 * t] = x.x, ex[4 * t + 1] = x.y, ex[4 * t + 2] = x.z, ex[4 * t + 3] = x.w;
+        }
+    }
+#pragma unroll
+    for (int j = 0; j < GPW; ++j) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const uint32_t m = 8u * (r >> 2) + 4u * h + (r & 3);
+            if (m < rows) out[(uint64_t)m * k + col0 + 32u * j] = kScaled ? ldexpf(acc[j][r], -ex[r]) : acc[j][r];
         }
     }
 }
@@ -709,15 +962,27 @@ Plan make_plan(uint64_t P, uint32_t k, uint32_t num_feature_tiles) {
     return p;
 }
 
-template <int IN, int PT, bool GATHER, int W>
-hipError_t launch_one(const void* in, uint64_t ld, uint32_t rows, uint64_t P, uint32_t k,
-                      uint32_t seed, const Plan& pl, float* partial, hipStream_t s) {
+template <int IN, bool GATHER, int W>
+hipError_t launch_rademacher(const void* in, uint64_t ld, uint32_t rows, uint64_t P, uint32_t k, uint32_t seed,
+                             const Plan& pl, float* partial, hipStream_t s) {
     const uint32_t groups8 = (pl.groups + 7u) / 8u * 8u;
     const uint64_t wgs = (uint64_t)groups8 * pl.col_blocks;
     if (wgs > 0x7FFFFFFFull) return hipErrorInvalidValue;
-    hipLaunchKernelGGL((jl_project_kernel<IN, PT, GATHER, W>), dim3((uint32_t)wgs), dim3(64 * W), 0, s, in, ld,
-                       rows, P, k, seed, pl.tl.tiles, pl.tl.tile_size, pl.chunks_per_tile,
-                       pl.chunks_per_group, partial);
+    hipLaunchKernelGGL((jl_project_kernel<IN, GATHER, W>), dim3((uint32_t)wgs), dim3(64 * W), 0, s, in, ld, rows, P,
+                       k, seed, pl.tl.tiles, pl.tl.tile_size, pl.chunks_per_tile, pl.chunks_per_group, partial);
+    return hipGetLastError();
+}
+
+// W (the plan's waves per 128 columns) selects the column groups per wave; the kernel has 8 waves
+template <int IN, bool GATHER, int W>
+hipError_t launch_normal(const void* in, uint64_t ld, uint32_t rows, uint64_t P, uint32_t k, uint32_t seed,
+                         const Plan& pl, float* partial, hipStream_t s) {
+    const uint32_t groups8 = (pl.groups + 7u) / 8u * 8u;
+    const uint64_t wgs = (uint64_t)groups8 * pl.col_blocks;
+    if (wgs > 0x7FFFFFFFull) return hipErrorInvalidValue;
+    hipLaunchKernelGGL((jl_project_normal_kernel<IN, GATHER, W / 2>), dim3((uint32_t)wgs), dim3(512), 0, s, in, ld,
+                       rows, P, k, seed, pl.tl.tiles, pl.tl.tile_size, pl.chunks_per_tile, pl.chunks_per_group,
+                       partial);
     return hipGetLastError();
 }
 
@@ -727,12 +992,12 @@ typedef hipError_t (*LaunchFn)(const void*, uint64_t, uint32_t, uint64_t, uint32
 template <int W>
 LaunchFn pick_w(int dtype, int proj_type, bool gather) {
     static const LaunchFn table[2][3][2] = {
-        {{launch_one<TRAKHIP_F16, TRAKHIP_RADEMACHER, false, W>, launch_one<TRAKHIP_F16, TRAKHIP_NORMAL, false, W>},
-         {launch_one<TRAKHIP_BF16, TRAKHIP_RADEMACHER, false, W>, launch_one<TRAKHIP_BF16, TRAKHIP_NORMAL, false, W>},
-         {launch_one<TRAKHIP_F32, TRAKHIP_RADEMACHER, false, W>, launch_one<TRAKHIP_F32, TRAKHIP_NORMAL, false, W>}},
-        {{launch_one<TRAKHIP_F16, TRAKHIP_RADEMACHER, true, W>, launch_one<TRAKHIP_F16, TRAKHIP_NORMAL, true, W>},
-         {launch_one<TRAKHIP_BF16, TRAKHIP_RADEMACHER, true, W>, launch_one<TRAKHIP_BF16, TRAKHIP_NORMAL, true, W>},
-         {launch_one<TRAKHIP_F32, TRAKHIP_RADEMACHER, true, W>, launch_one<TRAKHIP_F32, TRAKHIP_NORMAL, true, W>}},
+        {{launch_rademacher<TRAKHIP_F16, false, W>, launch_normal<TRAKHIP_F16, false, W>},
+         {launch_rademacher<TRAKHIP_BF16, false, W>, launch_normal<TRAKHIP_BF16, false, W>},
+         {launch_rademacher<TRAKHIP_F32, false, W>, launch_normal<TRAKHIP_F32, false, W>}},
+        {{launch_rademacher<TRAKHIP_F16, true, W>, launch_normal<TRAKHIP_F16, true, W>},
+         {launch_rademacher<TRAKHIP_BF16, true, W>, launch_normal<TRAKHIP_BF16, true, W>},
+         {launch_rademacher<TRAKHIP_F32, true, W>, launch_normal<TRAKHIP_F32, true, W>}},
     };
     return table[gather ? 1 : 0][dtype][proj_type];
 }
