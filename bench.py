@@ -200,51 +200,69 @@ def bench_batch_scaling(torch, dev):
     return res
 
 
+def _config_calls(torch, dev, name):
+    """(call, flop per call, description) for one named projection configuration: the synthetic
+    inputs of the benchmark configurations other than the headline one, resident on the device."""
+    import numpy as np
+
+    from trak_amd import ChunkedCudaProjector, CudaProjector, ProjectionType
+
+    gen = torch.Generator(device=dev).manual_seed(20_001)
+    if name == "c1":
+        g = torch.randn(16, 1_048_576, generator=gen, device=dev) * 1e-3
+        p = CudaProjector(1_048_576, 512, 42, ProjectionType.rademacher, dev, 32)
+        return (lambda: p.project(g, 0)), 2.0 * 16 * 1_048_576 * 512, "fp32 rademacher [16,1048576] -> 512"
+    if name == "c2":
+        g = (torch.randn(32, 4_825_610, generator=gen, device=dev) * 5e-4).half()
+        g[torch.rand(32, 4_825_610, generator=gen, device=dev) < 0.01] = 0
+        p = CudaProjector(4_825_610, 2048, 0, ProjectionType.rademacher, dev, 32)
+        return (lambda: p.project(g, 0)), 2.0 * 32 * 4_825_610 * 2048, "fp16 rademacher [32,4825610] -> 2048"
+    if name == "c3_dict":
+        shapes = resnet18_param_shapes()
+        P = sum(math.prod(sh) for sh in shapes)
+        grads = {i: (torch.randn(32, *sh, generator=gen, device=dev) * 1e-3).half() for i, sh in enumerate(shapes)}
+        p = CudaProjector(P, 4096, 7, ProjectionType.rademacher, dev, 32)
+        return (lambda: p.project(grads, 0)), 2.0 * 32 * P * 4096, "fp16 rademacher ResNet-18 gradient dict (62 tensors) -> 4096"
+    if name in ("c4", "c4_rademacher"):
+        chunk = 27_370_560
+        seeds = np.random.default_rng(123).integers(0, 500, size=4)
+        pt = ProjectionType.normal if name == "c4" else ProjectionType.rademacher
+        # Student-t (nu = 3) scaled by 1e-4: normal / sqrt(chi2_3 / 3)
+        grads = {}
+        for i in range(4):
+            z = torch.randn(32, chunk, generator=gen, device=dev)
+            c = torch.randn(3, 32, chunk, generator=gen, device=dev, dtype=torch.float16).float().square_().sum(0)
+            grads[i] = (z * torch.rsqrt(c / 3.0) * 1e-4).bfloat16()
+            del z, c
+        per = [CudaProjector(chunk, 4096, int(seeds[i]), pt, dev, 32) for i in range(4)]
+        p = ChunkedCudaProjector(per, chunk, [chunk] * 4, 32, dev, torch.bfloat16)
+        return (lambda: p.project(grads, 0)), 2.0 * 32 * 4 * chunk * 4096, \
+            f"bf16 {pt.value} chunked (4 x 27370560) [32,109482240] -> 4096"
+    raise ValueError(f"unknown configuration {name}")
+
+
+def bench_config(torch, dev, name, reps):
+    call, flop, what = _config_calls(torch, dev, name)
+    call()
+    torch.cuda.synchronize()
+    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    a.record()
+    for _ in range(reps):
+        call()
+    b.record()
+    torch.cuda.synchronize()
+    ms = a.elapsed_time(b) / reps
+    return {"what": what, "ms": ms, "tflops": flop / ms / 1e9}
+
+
 def bench_other_configs(torch, dev):
     """Throughput of the other projection configurations (the CPU-runnable fp32 case, the
     ResNet-9-sized case and the BERT-sized chunked normal case); not part of the default line,
     `--all-configs` prints them to stderr."""
-    from trak_amd import ChunkedCudaProjector, CudaProjector, ProjectionType
-
     res = {}
-
-    def timed(fn, reps):
-        fn()
-        torch.cuda.synchronize()
-        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        a.record()
-        for _ in range(reps):
-            fn()
-        b.record()
-        torch.cuda.synchronize()
-        return a.elapsed_time(b) / reps
-
-    gen = torch.Generator(device=dev).manual_seed(20_001)
-    g1 = torch.randn(16, 1_048_576, generator=gen, device=dev) * 1e-3
-    p1 = CudaProjector(1_048_576, 512, 42, ProjectionType.rademacher, dev, 32)
-    ms = timed(lambda: p1.project(g1, 0), 50)
-    res["c1_fp32_rademacher_[16,1048576]_k512"] = {"ms": ms, "tflops": 2.0 * 16 * 1_048_576 * 512 / ms / 1e9}
-
-    g2 = (torch.randn(32, 4_825_610, generator=gen, device=dev) * 5e-4).half()
-    g2[torch.rand(32, 4_825_610, generator=gen, device=dev) < 0.01] = 0
-    p2 = CudaProjector(4_825_610, 2048, 0, ProjectionType.rademacher, dev, 32)
-    ms = timed(lambda: p2.project(g2, 0), 30)
-    res["c2_fp16_rademacher_[32,4825610]_k2048"] = {"ms": ms, "tflops": 2.0 * 32 * 4_825_610 * 2048 / ms / 1e9}
-    del g1, g2
-
-    import numpy as np
-
-    chunk = 27_370_560
-    seeds = np.random.default_rng(123).integers(0, 500, size=4)
-    grads = {i: (torch.randn(32, chunk, generator=gen, device=dev) * 1e-4).bfloat16() for i in range(4)}
-    per = [CudaProjector(chunk, 4096, int(seeds[i]), ProjectionType.normal, dev, 32) for i in range(4)]
-    p4 = ChunkedCudaProjector(per, chunk, [chunk] * 4, 32, dev, torch.bfloat16)
-    ms = timed(lambda: p4.project(grads, 0), 2)
-    res["c4_bf16_normal_chunked_[32,109482240]_k4096"] = {"ms": ms, "tflops": 2.0 * 32 * 4 * chunk * 4096 / ms / 1e9}
-    per_r = [CudaProjector(chunk, 4096, int(seeds[i]), ProjectionType.rademacher, dev, 32) for i in range(4)]
-    p4r = ChunkedCudaProjector(per_r, chunk, [chunk] * 4, 32, dev, torch.bfloat16)
-    ms = timed(lambda: p4r.project(grads, 0), 5)
-    res["c4_shape_bf16_rademacher_chunked"] = {"ms": ms, "tflops": 2.0 * 32 * 4 * chunk * 4096 / ms / 1e9}
+    for name, reps in (("c1", 50), ("c2", 30), ("c4", 3), ("c4_rademacher", 5)):
+        res[name] = bench_config(torch, dev, name, reps)
+        torch.cuda.empty_cache()
     return res
 
 
@@ -460,6 +478,9 @@ def main():
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--all-configs", action="store_true",
                     help="also time the other projection configurations and print them to stderr")
+    ap.add_argument("--only", default=None, metavar="NAME",
+                    help="run just one workload for --steps calls and print its timing (for profiler runs): "
+                         "c1 | c2 | c3_dict | c4 | c4_rademacher | scoring")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run one 1 GiB device-to-device copy (reference point for rocprofv3 byte counters)")
     args = ap.parse_args()
@@ -480,6 +501,12 @@ def main():
         dst.copy_(src)
         torch.cuda.synchronize()
         del src, dst
+    if args.only:
+        if args.only == "scoring":
+            print(json.dumps({"only": "scoring", **bench_scoring(torch, dev, reps=max(1, min(args.steps, 3)))}))
+        else:
+            print(json.dumps({"only": args.only, **bench_config(torch, dev, args.only, args.steps)}))
+        return
     proj = bench_projection(torch, dev, args.steps, args.warmup, args.batches)
     torch.cuda.empty_cache()
     if args.all_configs:

@@ -715,10 +715,16 @@ __global__ __launch_bounds__(512, 2) void jl_project_normal_kernel(
     constexpr int kBufElems = kPlanes * kPlaneElems;
     constexpr bool kScaled = Tr::scaled;
 
-    __shared__ __attribute__((aligned(16))) uint16_t lds[kBuffers * kBufElems];
-    __shared__ __attribute__((aligned(16))) uint16_t r_tab[kRadiusEntries];
-    __shared__ __attribute__((aligned(16))) uint32_t cs_tab[kAngleEntries];
-    __shared__ __attribute__((aligned(16))) int sh_lds[kBuffers][2][32];  // per row: change of exponent, exponent
+    // One LDS block, tables first: a DS instruction adds a 16-bit immediate to the address register,
+    // so a table that starts below 64 KB is indexed without an extra addition per lookup.
+    constexpr int kCsBytes = kAngleEntries * 4, kRBytes = kRadiusEntries * 2;
+    constexpr int kStageBytes = kBuffers * kBufElems * 2;
+    __shared__ __attribute__((aligned(16))) char smem[kCsBytes + kRBytes + kStageBytes + kBuffers * 2 * 32 * 4];
+    uint32_t* cs_tab = reinterpret_cast<uint32_t*>(smem);
+    uint16_t* r_tab = reinterpret_cast<uint16_t*>(smem + kCsBytes);
+    uint16_t* lds = reinterpret_cast<uint16_t*>(smem + kCsBytes + kRBytes);
+    // per buffer and row: change of the row's exponent against the previous chunk, and the exponent
+    int (*sh_lds)[2][32] = reinterpret_cast<int (*)[2][32]>(smem + kCsBytes + kRBytes + kStageBytes);
 
     const uint32_t col_blocks = k / kColsPerWG;
     uint32_t cb, group;
