@@ -507,24 +507,48 @@ __global__ __launch_bounds__(64 * kWaves, 2) void gemm_nt16_kernel(
     __syncthreads();
 
     const int a_row = (wm * 64 + x) * 8, b_row = (BM + wn * (32 * JT) + x) * 8;  // first piece of the lane's rows
+    // A step is four sub-steps of eight MFMAs (two A fragments x four B fragments).  The six fragments of
+    // sub-step u + 1 are requested before the MFMAs of sub-step u are issued, so an LDS read has eight MFMAs
+    // (256 cycles) to arrive instead of stalling the wave; the per-step barrier sits in front of the last
+    // sub-step, whose MFMAs then cover the first reads from the other buffer.  Two register sets, alternating.
+    piece fa[2][2], fb[2][JT];
+    auto fetch = [&](int buf, int u, int set) {
+        const piece* l = lds[buf] + ((2 * u + h) ^ ((x >> 1) & 7));
+#pragma unroll
+        for (int i = 0; i < 2; ++i) fa[set][i] = l[a_row + 256 * i];
+#pragma unroll
+        for (int j = 0; j < JT; ++j) fb[set][j] = l[b_row + 256 * j];
+    };
+    fetch(0, 0, 0);
     for (uint64_t s = 0; s < steps; ++s) {
         const int cur = (int)(s & 1);
         if (s + 1 < steps) dma(s + 1, lds[cur ^ 1]);
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
-            const piece* l = lds[cur] + ((2 * u + h) ^ ((x >> 1) & 7));
-            piece fa[2];
-#pragma unroll
-            for (int i = 0; i < 2; ++i) fa[i] = l[a_row + 256 * i];
-#pragma unroll
-            for (int j = 0; j < JT; ++j) {
-                const piece fb = l[b_row + 256 * j];
-#pragma unroll
-                for (int i = 0; i < 2; ++i) acc[i][j] = mfma16<F16>(fa[i], fb, acc[i][j]);
+            const int set = u & 1;
+            // Wait for this sub-step's fragments HERE, while they are the only LDS reads in flight: the
+            // compiler waits for all outstanding LDS reads at once (it cannot order them against the
+            // LDS-direct loads), so the next reads are issued after this point and stay in flight under
+            // the MFMAs.
+            asm volatile("" ::"v"(fa[set][0]), "v"(fa[set][1]), "v"(fb[set][0]), "v"(fb[set][1]), "v"(fb[set][2]),
+                         "v"(fb[set][3]));
+            __builtin_amdgcn_sched_barrier(0);
+            if (u < 3) {
+                fetch(cur, u + 1, set ^ 1);
+            } else {
+                // every read of this buffer has completed; wait for this wave's part of the next buffer,
+                // meet the other waves, then start on the next buffer
+                asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+                __syncthreads();
+                if (s + 1 < steps) fetch(cur ^ 1, 0, 0);
             }
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int j = 0; j < JT; ++j)
+#pragma unroll
+                for (int i = 0; i < 2; ++i) acc[i][j] = mfma16<F16>(fa[set][i], fb[set][j], acc[i][j]);
+            __builtin_amdgcn_sched_barrier(0);
         }
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        __syncthreads();
     }
     store_c<ACCUM, JT>(acc, C, ldc, M, N, m0 + wm * 64, n0 + wn * (32 * JT) + x, h, alpha, beta, row_scale);
 }
