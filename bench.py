@@ -27,10 +27,24 @@ sys.path.insert(0, ROOT)
 
 PEAK_FP16_TFLOPS = 2500.0   # MI355X dense fp16/bf16 MFMA
 PEAK_FP32_TFLOPS = 157.3    # MI355X fp32 MFMA
-# HBM bytes of one projection-kernel launch at the benchmark shape, from rocprofv3 --pmc FETCH_SIZE and
-# WRITE_SIZE (profiles/jl_project_f16_rademacher_resnet18_hbm_counters.txt): 365528 KiB x 2.0 (the factor
-# a 1 GiB copy needs for the same counter) fetched + 32768 KiB x 1.0 written.
-PROJECT_KERNEL_HBM_BYTES = (365528 * 2.0 + 32768 * 1.0) * 1024
+# HBM bytes of one projection-kernel launch at the benchmark shape come from the tracked rocprofv3 summary
+# (FETCH_SIZE and WRITE_SIZE in KiB per dispatch, each times the factor a 1 GiB copy needs for the same counter).
+TRAFFIC_PROFILE = os.path.join("profiles", "jl_project_f16_rademacher_resnet18_hbm_counters.txt")
+
+
+def profiled_kernel_traffic():
+    """(bytes per launch, source file) read from the tracked HBM-counter summary, or (None, None)."""
+    import re
+
+    try:
+        text = open(os.path.join(ROOT, TRAFFIC_PROFILE)).read()
+        f = re.search(r"^\s*FETCH_SIZE\s+([\d.]+) KiB x ([\d.]+)", text, re.M)
+        w = re.search(r"^\s*WRITE_SIZE\s+([\d.]+) KiB x ([\d.]+)", text, re.M)
+        return (float(f.group(1)) * float(f.group(2)) + float(w.group(1)) * float(w.group(2))) * 1024, TRAFFIC_PROFILE
+    except (OSError, AttributeError, ValueError):
+        return None, None
+
+
 METRIC = "JL proj TFLOP/s & % MFMA peak at P=11.7M,k=4096,B=32; scoring TFLOP/s"
 
 
@@ -77,7 +91,7 @@ def make_batches(torch, dev, n_batches, B, P, seed):
     return out
 
 
-def bench_projection(torch, dev, steps, warmup, n_batches):
+def bench_projection(torch, dev, steps, warmup, n_batches, sustain_s=2.0):
     from trak_amd import _lib, fast_jl
 
     lib = _lib.load()
@@ -116,7 +130,33 @@ def bench_projection(torch, dev, steps, warmup, n_batches):
     kernel_ms = sorted(hip.elapsed_ms(a, b) for a, b in evs)
     kernel_avg = sum(kernel_ms) / len(kernel_ms)
     flop = 2.0 * B * P * k
+
+    # sustained: back-to-back calls over the resident batches for `sustain_s` seconds (the kernel's bound
+    # is power, so a figure over seconds belongs beside the one over the timed steps)
+    sustained = None
+    if sustain_s > 0:
+        n = max(steps, int(math.ceil(sustain_s * 1e3 / ms_per_step)))
+        evs = [(hip.event(), hip.event()) for _ in range(n)]
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for i in range(n):
+            g = batches[i % n_batches]
+            hip.record(evs[i][0], stream)
+            _lib.check(lib.trakhip_project_partials(vp(g.data_ptr()), _lib.F16, B, P, P, vp(ws.data_ptr()), ws.numel(),
+                                                    k, seed, tiles, _lib.RADEMACHER, vp(stream)))
+            hip.record(evs[i][1], stream)
+            _lib.check(lib.trakhip_project_reduce(vp(ws.data_ptr()), B, P, k, tiles, 1.0, vp(out.data_ptr()), vp(stream)))
+        torch.cuda.synchronize()
+        wall = time.perf_counter() - t0
+        km = sorted(hip.elapsed_ms(a, b) for a, b in evs)
+        sustained = {
+            "calls": n, "seconds": round(wall, 3), "tflops": round(flop * n / wall / 1e12, 1),
+            "kernel_ms_min": round(km[0], 4), "kernel_ms_median": round(km[n // 2], 4),
+            "kernel_ms_max": round(km[-1], 4),
+            "kernel_tflops_median": round(flop / km[n // 2] / 1e9, 1),
+        }
     return {
+        "sustained": sustained,
         "flop": flop,
         "ms_per_step": ms_per_step,
         "tflops": flop / (ms_per_step * 1e-3) / 1e12,
@@ -253,6 +293,45 @@ def bench_config(torch, dev, name, reps):
     torch.cuda.synchronize()
     ms = a.elapsed_time(b) / reps
     return {"what": what, "ms": ms, "tflops": flop / ms / 1e9}
+
+
+MFMA_RATE_CASES = [
+    # name, instruction (0 f16, 1 bf16, 2 f32), operand kind of A, of B (see trak_amd/csrc/mfma_rate.hip)
+    ("f16 A=0 B=0", 0, 0, 0),
+    ("f16 A=gradient-like B=+-1 (as the projection kernel)", 0, 1, 2),
+    ("f16 A=+-1 B=gradient-like (swapped)", 0, 2, 1),
+    ("f16 A=random B=random", 0, 3, 3),
+    ("bf16 A=random B=random (as the 16-bit GEMM kernels)", 1, 4, 4),
+    ("f32 A=random B=random (v_mfma_f32_32x32x2_f32)", 2, 3, 3),
+]
+
+
+def bench_mfma_rate(torch, dev, iters=300_000):
+    """What a loop of nothing but independent MFMAs sustains on this machine, by operand data (the
+    clock is power limited, so the rate depends on the data): the reference point for the projection
+    and GEMM kernels.  One dispatch per case, timed with events on the launch stream."""
+    path = os.path.join(ROOT, "trak_amd", "libtrakhip_diag.so")
+    if not os.path.exists(path):
+        raise ImportError(f"{path} is missing: build it with `python -m trak_amd.build`")
+    lib = ctypes.CDLL(path)
+    lib.trakhip_diag_mfma_rate_out_floats.restype = ctypes.c_size_t
+    lib.trakhip_diag_mfma_rate.restype = ctypes.c_double
+    lib.trakhip_diag_mfma_rate.argtypes = [ctypes.c_int] * 4 + [ctypes.c_void_p, ctypes.c_void_p]
+    out = torch.empty(lib.trakhip_diag_mfma_rate_out_floats(), dtype=torch.float32, device=dev)
+    stream = torch.cuda.current_stream(dev).cuda_stream
+    res = {}
+    for name, instr, ka, kb in MFMA_RATE_CASES:
+        lib.trakhip_diag_mfma_rate(instr, ka, kb, 20_000, out.data_ptr(), stream)
+        torch.cuda.synchronize()
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        flop = lib.trakhip_diag_mfma_rate(instr, ka, kb, iters, out.data_ptr(), stream)
+        b.record()
+        torch.cuda.synchronize()
+        assert flop > 0
+        ms = a.elapsed_time(b)
+        res[name] = {"ms": round(ms, 2), "tflops": round(flop / ms / 1e9, 1)}
+    return res
 
 
 def bench_other_configs(torch, dev):
@@ -428,7 +507,7 @@ def bench_scoring(torch, dev, reps=3):
     }
 
 
-def cpu_baseline(torch):
+def cpu_baseline(torch, cpu_c4=False):
     """trak's BasicProjector CPU path (restated in oracle/basic_projector.py) on its CPU-runnable
     configuration, all host cores; plus a bounded BasicScoreComputer sample."""
     from oracle.basic_projector import BasicProjectorCPU
@@ -448,6 +527,28 @@ def cpu_baseline(torch):
         "value": flop / dt / 1e12, "unit": "TFLOP/s", "cores": cores, "kind": "port",
         "sample": f"BasicProjector restatement, full config [16,1048576] fp32 -> 512 rademacher, {dt:.2f} s",
     }
+    # The larger projection configurations take minutes to hours on a CPU (every 100-column block regenerates
+    # a [P, 100] fp32 matrix): two full blocks are timed and the time is scaled by num_blocks / 2
+    # (trak/projectors.py:258-314 does the same work for every block).  fp32, as BasicProjector runs on a CPU.
+    def sample(B, P, k, seed, proj_type, scale, chunks=1):
+        g = torch.randn(B, P, generator=gen) * scale
+        pr = BasicProjectorCPU(grad_dim=P, proj_dim=k, seed=seed, proj_type=proj_type)
+        blocks = 2
+        t0 = time.perf_counter()
+        pr.project(g, model_id=0, max_blocks=blocks)
+        dt = time.perf_counter() - t0
+        full = dt * pr.num_blocks / blocks * chunks
+        return {"tflops": 2.0 * B * P * chunks * k / full / 1e12, "extrapolated": True, "blocks_timed": blocks,
+                "blocks_total": pr.num_blocks * chunks, "sample_s": round(dt, 2), "estimated_full_s": round(full, 1)}
+
+    res["other_configs"] = {
+        "c2_[32,4825610]_k2048_rademacher": sample(32, 4_825_610, 2048, 0, "rademacher", 5e-4),
+        "c3_[32,11689512]_k4096_rademacher": sample(32, 11_689_512, 4096, 7, "rademacher", 1e-3),
+    }
+    if cpu_c4:
+        # one of the four parameter chunks; the other three cost the same
+        res["other_configs"]["c4_[32,109482240]_k4096_normal_4_chunks"] = sample(32, 27_370_560, 4096, 123, "normal",
+                                                                                 1e-4, chunks=4)
     N, M, kk = 50_000, 10_000, 4096  # the scoring configuration in full
     X = torch.randn(N, kk, generator=gen) / 64
     Xt = torch.randn(M, kk, generator=gen) / 64
@@ -474,13 +575,17 @@ def main():
     ap.add_argument("--steps", type=int, default=30)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--batches", type=int, default=16, help="distinct resident batches cycled through")
+    ap.add_argument("--sustain", type=float, default=2.0,
+                    help="seconds of back-to-back calls for the `sustained` figure (0 = skip)")
+    ap.add_argument("--cpu-c4", action="store_true",
+                    help="also time the BERT-sized normal configuration's BasicProjector sample on the CPU (about a minute)")
     ap.add_argument("--no-scoring", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--all-configs", action="store_true",
                     help="also time the other projection configurations and print them to stderr")
     ap.add_argument("--only", default=None, metavar="NAME",
                     help="run just one workload for --steps calls and print its timing (for profiler runs): "
-                         "c1 | c2 | c3_dict | c4 | c4_rademacher | scoring")
+                         "c1 | c2 | c3_dict | c4 | c4_rademacher | scoring | mfma_rate")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run one 1 GiB device-to-device copy (reference point for rocprofv3 byte counters)")
     args = ap.parse_args()
@@ -502,12 +607,14 @@ def main():
         torch.cuda.synchronize()
         del src, dst
     if args.only:
-        if args.only == "scoring":
+        if args.only == "mfma_rate":
+            print(json.dumps({"only": "mfma_rate", **bench_mfma_rate(torch, dev)}))
+        elif args.only == "scoring":
             print(json.dumps({"only": "scoring", **bench_scoring(torch, dev, reps=max(1, min(args.steps, 3)))}))
         else:
             print(json.dumps({"only": args.only, **bench_config(torch, dev, args.only, args.steps)}))
         return
-    proj = bench_projection(torch, dev, args.steps, args.warmup, args.batches)
+    proj = bench_projection(torch, dev, args.steps, args.warmup, args.batches, args.sustain)
     torch.cuda.empty_cache()
     if args.all_configs:
         print(json.dumps(bench_other_configs(torch, dev), indent=1), file=sys.stderr)
@@ -518,8 +625,9 @@ def main():
         torch.cuda.empty_cache()
     scoring = None if args.no_scoring else bench_scoring(torch, dev)
     torch.cuda.empty_cache()
-    cpu = None if args.no_cpu else cpu_baseline(torch)
+    cpu = None if args.no_cpu else cpu_baseline(torch, args.cpu_c4)
 
+    traffic, traffic_source = profiled_kernel_traffic()
     line = {
         "metric": METRIC,
         "value": round(proj["tflops"], 3),
@@ -546,12 +654,14 @@ def main():
             "peak": PEAK_FP16_TFLOPS,
             "unit": "TFLOP/s",
             "frac": round(proj["kernel_tflops"] / PEAK_FP16_TFLOPS, 4),
-            "traffic": PROJECT_KERNEL_HBM_BYTES,
+            "traffic": traffic,
             "traffic_unit": "bytes per launch (algorithmic input+output: %d)" % (32 * 11_689_512 * 2 + 32 * 4096 * 4),
+            "traffic_source": traffic_source,
             "kernel": "jl_project_kernel<f16, rademacher>",
             "kernel_ms_avg": round(proj["kernel_ms_avg"], 4),
             "kernel_ms_min": round(proj["kernel_ms_min"], 4),
         },
+        "sustained": proj["sustained"],
         "cpu_baseline": cpu,
         "scoring": scoring,
     }

@@ -2,7 +2,7 @@
 """Writes tests/golden/reference_vectors.npz: small input/output vectors of the reference's own
 CPU-runnable code for the functions of the hot path that no closed form pins by value:
 BasicProjector (its matrix comes from torch's CPU generator), vectorize,
-get_parameter_chunk_sizes and BasicScoreComputer.
+get_parameter_chunk_sizes, BasicScoreComputer (fp32 and fp16) and ChunkedCudaProjector's accumulation.
 
 Run once, in the container that has the reference checked out at /root/reference:
     python tests/golden/make_reference_vectors.py
@@ -63,6 +63,36 @@ acc = torch.zeros(130, 11)
 sc.get_scores(feats, Xt, acc)
 out["sc_X"], out["sc_Xt"] = X.numpy(), Xt.numpy()
 out["sc_xtx"], out["sc_features"], out["sc_scores"] = xtx.numpy(), feats.numpy(), acc.numpy()
+# ChunkedCudaProjector: the reference's class, driven with CPU BasicProjectors in place of
+# CudaProjectors (both return fp32 parts for the packed chunk), with a 16-bit `dtype`: pins how the
+# chunk projections are accumulated (in `dtype`, rounded after every chunk: trak/projectors.py:472-495)
+from trak.projectors import ChunkedCudaProjector  # noqa: E402
+
+cg = {
+    "a": torch.randn(3, 40, 10, generator=gen) * 0.7,
+    "b": torch.randn(3, 300, generator=gen) * 0.7,
+    "c": torch.randn(3, generator=gen),
+    "d": torch.randn(3, 25, 12, generator=gen) * 0.7,
+}
+sizes = [400 + 300 + 1, 300]          # "d" does not fit next to the first three under a limit of 750
+for k_, v in cg.items():
+    out[f"chunk_in_{k_}"] = v.numpy()
+for tag, dt in (("fp16", torch.float16), ("bf16", torch.bfloat16)):
+    per = [BasicProjector(grad_dim=sz, proj_dim=128, seed=3 + i, proj_type=ProjectionType.rademacher,
+                          device="cpu", dtype=torch.float32) for i, sz in enumerate(sizes)]
+    cp = ChunkedCudaProjector(per, 750, sizes, 4, "cpu", dt)
+    res = cp.project({k_: v.to(dt) for k_, v in cg.items()}, model_id=0)
+    assert res.dtype == dt and res.shape == (3, 128)
+    out[f"chunk_out_{tag}"] = res.float().numpy()
+
+# BasicScoreComputer with a 16-bit dtype and three row blocks: pins the per-block rounding of X^T X,
+# lambda added in the 16-bit type and the type of the returned features (trak/score_computers.py:145-177)
+Xh = (torch.randn(130, 16, generator=gen) / 2).half()
+sch = BasicScoreComputer(dtype=torch.float16, device="cpu", CUDA_MAX_DIM_SIZE=50, lambda_reg=1e-2)
+xtx_h = sch.get_xtx(Xh)
+feats_h = sch.get_x_xtx_inv(Xh, xtx_h)
+assert xtx_h.dtype == torch.float16 and feats_h.dtype == torch.float16
+out["sch_X"], out["sch_xtx"], out["sch_features"] = Xh.float().numpy(), xtx_h.float().numpy(), feats_h.float().numpy()
 out["torch_version"] = np.array(torch.__version__)
 
 path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "reference_vectors.npz")

@@ -71,3 +71,61 @@ def test_gpu_score_computer_matches_reference_vectors(gpu):
     assert rel(xtx.cpu().numpy(), GOLD["sc_xtx"]) < 1e-5
     assert rel(feats.cpu().numpy(), GOLD["sc_features"]) < 1e-4
     assert rel(acc.numpy(), GOLD["sc_scores"]) < 1e-4
+
+
+@pytest.mark.parametrize("tag,dt", [("fp16", torch.float16), ("bf16", torch.bfloat16)])
+def test_chunked_accumulation_in_dtype_matches_reference_vectors(tag, dt):
+    # The reference's ChunkedCudaProjector adds the fp32 chunk projections into an accumulator of its
+    # `dtype`, rounding after every chunk (trak/projectors.py:472-495).  accumulate_in_dtype=True must
+    # give its bits; the default (fp32 sum, one rounding) must be the correctly rounded sum instead.
+    from trak_amd import ChunkedCudaProjector
+
+    grads = {k: torch.from_numpy(GOLD[f"chunk_in_{k}"]).to(dt) for k in ("a", "b", "c", "d")}
+    sizes = [701, 300]
+    per = [BasicProjectorCPU(grad_dim=sz, proj_dim=128, seed=3 + i, proj_type="rademacher") for i, sz in enumerate(sizes)]
+    exact = ChunkedCudaProjector(per, 750, sizes, 4, "cpu", dt, accumulate_in_dtype=True).project(grads, model_id=0)
+    assert exact.dtype == dt and exact.shape == (3, 128)
+    assert np.array_equal(exact.float().numpy(), GOLD[f"chunk_out_{tag}"])
+    default = ChunkedCudaProjector(per, 750, sizes, 4, "cpu", dt).project(grads, model_id=0)
+    flat = vectorize(grads, device="cpu")
+    parts = [per[0].project(flat[:, :701], model_id=0), per[1].project(flat[:, 701:], model_id=0)]
+    assert torch.equal(default, (parts[0] + parts[1]).to(dt))
+    # the two differ by the extra rounding of the first chunk's part: at most one step of dt at its size
+    step = torch.finfo(dt).eps * torch.maximum(parts[0].abs(), default.float().abs())
+    assert ((exact.float() - default.float()).abs() <= step).all()
+    assert not torch.equal(exact, default)
+    # a batch larger than feat_bs is refused (the reference fails on its packing copy)
+    big = {k: torch.cat([v, v]) for k, v in grads.items()}
+    with pytest.raises(RuntimeError, match="feat_bs"):
+        ChunkedCudaProjector(per, 750, sizes, 4, "cpu", dt).project(big, model_id=0)
+
+
+@pytest.mark.gpu
+def test_gpu_score_computer_fp16_in_dtype_matches_reference_vectors(gpu):
+    # fp16 `dtype`, three row blocks: the reference rounds every block product and the running sum to
+    # fp16 and adds lambda in fp16 (trak/score_computers.py:147-162).  Its CPU matmul and this GPU one
+    # add the 50 products of a block in different orders, so single entries may land on the other side
+    # of an fp16 rounding boundary: at most one fp16 step apart, and nearly all identical.
+    from trak_amd import BasicScoreComputer
+
+    X = torch.from_numpy(GOLD["sch_X"]).half()
+    want_xtx, want_f = GOLD["sch_xtx"], GOLD["sch_features"]
+    sc = BasicScoreComputer(dtype=torch.float16, device="cuda:0", CUDA_MAX_DIM_SIZE=50, lambda_reg=1e-2,
+                            accumulate_in_dtype=True)
+    xtx = sc.get_xtx(X)
+    assert xtx.dtype == torch.float16
+    got = xtx.float().cpu().numpy()
+    step = np.maximum(np.abs(want_xtx), 2.0**-14) * 2.0**-10
+    assert np.all(np.abs(got - want_xtx) <= step)
+    assert np.mean(got == want_xtx) > 0.9
+    feats = sc.get_x_xtx_inv(X, xtx)
+    assert feats.dtype == torch.float16
+    rel = np.abs(feats.float().cpu().numpy() - want_f).max() / np.abs(want_f).max()
+    assert rel < 5e-3
+    # the default (fp32 sums, one rounding) is the more accurate of the two against float64
+    sc32 = BasicScoreComputer(dtype=torch.float16, device="cuda:0", CUDA_MAX_DIM_SIZE=50, lambda_reg=1e-2)
+    x64 = GOLD["sch_X"].astype(np.float64)
+    truth = x64.T @ x64
+    err_default = np.abs(sc32.get_xtx(X).float().cpu().numpy() - truth).max()
+    err_exact = np.abs(got - truth).max()
+    assert err_default <= err_exact + 1e-12

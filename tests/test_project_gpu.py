@@ -305,6 +305,38 @@ def test_full_size_resnet18_shape(gpu, c_oracle):
         assert np.linalg.norm(got - want) / np.linalg.norm(want) < 1e-3
 
 
+def test_full_size_resnet18_gradient_dict_through_the_projector(gpu, c_oracle):
+    # what TRAKer.featurize hands to the projector at this shape: the dict of the 62 ResNet-18
+    # parameter gradients (trak/gradient_computers.py:145-160), here with one log-uniform scale per
+    # parameter.  CudaProjector.project(dict) reads it in place; the result must be the bits of
+    # flatten-then-project and agree with the float64 contraction.
+    import bench
+    from trak_amd import vectorize
+
+    shapes = bench.resnet18_param_shapes()
+    B, k, seed = 32, 4096, 7
+    P = sum(math.prod(sh) for sh in shapes)
+    assert P == 11_689_512 and len(shapes) == 62
+    gen = torch.Generator(device=gpu).manual_seed(20_003)
+    scale = 10 ** (torch.rand(len(shapes), generator=gen, device=gpu) * 3 - 5)
+    grads = {f"p{i}": (torch.randn(B, *sh, generator=gen, device=gpu) * scale[i]).half() for i, sh in enumerate(shapes)}
+    proj = _projector(P, k, seed, ProjectionType.rademacher, torch.float16)
+    out = proj.project(grads, model_id=0)
+    flat = vectorize(grads, device=gpu)
+    assert flat.shape == (B, P)
+    dense = fast_jl.project_rademacher_32(flat, k, seed, proj.num_sms)
+    assert torch.equal(out, dense)
+    g32 = to_f32_numpy(flat)
+    for c in (0, 1023, 1024, 3333, 4095):   # columns of all four column blocks, both ends
+        want = c_oracle.project(g32, seed, proj.num_sms, c, 1, R)[:, 0]
+        got = out[:, c].cpu().numpy().astype(np.float64)
+        assert np.linalg.norm(got - want) / np.linalg.norm(want) < 1e-3, c
+    # a second checkpoint (model_id) uses another matrix: seed + 10^4 * model_id (trak/projectors.py:409)
+    out1 = proj.project(grads, model_id=1)
+    assert torch.equal(out1, fast_jl.project_rademacher_32(flat, k, seed + 10_000, proj.num_sms))
+    assert not torch.equal(out1, out)
+
+
 def test_full_size_cpu_runnable_shape(gpu, c_oracle):
     # gradients [16, 1 048 576] fp32 iid N(0, 1e-3^2), k = 512, seed 42: every column against the
     # float64 contraction, to the fp32 bar
@@ -492,7 +524,7 @@ def test_many_rows(gpu, c_oracle, proj_type, dtype, B):
             assert np.array_equal(got[r], c_oracle.materialize(seed, tiles, P, feats[r], 1, 0, k, proj_type)[0]), r
     # a batch and its first 32 rows agree
     head = fn(proj_type)(g[:32].contiguous(), k, seed, tiles)
-    assert torch.allclose(out[:32], head, rtol=1e-4, atol=1e-5)
+    assert torch.equal(out[:32], head)   # same launch shape, same matrix, same order of additions
 
 
 def test_many_rows_gather(gpu):

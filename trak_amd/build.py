@@ -9,6 +9,8 @@ import sys
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libtrakhip.so")
+DIAG_LIB = os.path.join(HERE, "libtrakhip_diag.so")  # measurement aid for bench.py, not the product ABI
+DIAG_SOURCES = ["mfma_rate.hip"]
 SOURCES = ["capi.hip", "project.hip", "gemm.hip", "spd.hip", "store.hip", "gemm_split.hip"]
 FLAGS = [
     "--offload-arch=gfx950",
@@ -44,6 +46,15 @@ def build(verbose=True, jobs=4):
     if verbose:
         print(" ".join(cmd), flush=True)
     subprocess.check_call(cmd)
+    cmd = [hipcc, *FLAGS, "-shared", "-o", DIAG_LIB, *[os.path.join(CSRC, s) for s in DIAG_SOURCES]]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    out = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT)
+    text = "\n".join(l for l in out.stdout.decode(errors="replace").splitlines() if "packed-fp32-ops" not in l)
+    if text.strip():
+        print(text)
+    if out.returncode != 0:
+        raise RuntimeError("hipcc failed on the measurement aid")
     return LIB
 
 

@@ -176,7 +176,13 @@ class ChunkedCudaProjector:
         feat_bs: int,
         device: torch.device,
         dtype: torch.dtype,
+        accumulate_in_dtype: bool = False,
     ):
+        # accumulate_in_dtype=True reproduces the reference's arithmetic to the bit: the running sum of
+        # the chunk projections is kept in `dtype` and rounded after every addition
+        # (trak/projectors.py:472-474, :490-495, :509-514).  The default keeps the sum in fp32 and rounds
+        # once at the end, which is at least as accurate and what the kernels produce anyway.
+        self.accumulate_in_dtype = accumulate_in_dtype
         self.projector_per_chunk = projector_per_chunk
         self.proj_dim = self.projector_per_chunk[0].proj_dim
         self.proj_type = self.projector_per_chunk[0].proj_type
@@ -189,77 +195,66 @@ class ChunkedCudaProjector:
         self.input_allocated = False
 
     def allocate_input(self):
-        if self.input_allocated:
-            return
-        # the widest chunk that will actually be packed (the reference allocates max_chunk_size
-        # columns, i.e. always close to 2^32 / feat_bs elements per row)
-        width = int(max(self.params_per_chunk))
-        self.ch_input = ch.zeros(size=(self.feat_bs, width), device=self.device, dtype=self.dtype)
+        """Kept for interface compatibility (trak/projectors.py:452-462 allocates a
+        [feat_bs, max_chunk_size] packing buffer here): nothing is packed in this implementation, the
+        chunks are projected where the gradients are."""
         self.input_allocated = True
 
     def free_memory(self):
-        if not self.input_allocated:
-            return
-        del self.ch_input
         self.input_allocated = False
 
-    def _project_in_place(self, grads, model_id):
-        """Same grouping rule as the packing path below, but every chunk is handed to its projector
-        as a dict, which projects the parameter tensors where they are."""
-        groups, current, pointer = [], {}, 0
-        for name, p in grads.items():
+    def _chunk_sizes(self, grads):
+        """Greedy grouping of the dict's parameters into chunks of at most max_chunk_size features,
+        in dict order - the rule of trak/projectors.py:479-503 and of get_parameter_chunk_sizes
+        (trak/utils.py:297-331).  Returns [(first parameter index, end index, features)]."""
+        groups, begin, width = [], 0, 0
+        for i, p in enumerate(grads.values()):
             param_size = 1 if len(p.shape) < 2 else p[0].numel()
-            if pointer + param_size > self.max_chunk_size:
-                groups.append((current, pointer))
-                current, pointer = {}, 0
-            current[name] = p
-            pointer += param_size
-        groups.append((current, pointer))
-        actual_bs = min(self.feat_bs, next(iter(grads.values())).shape[0])
+            if width + param_size > self.max_chunk_size:
+                groups.append((begin, i, width))
+                begin, width = i, 0
+            width += param_size
+        groups.append((begin, len(grads), width))
+        got = [g[2] for g in groups]
+        assert got == [int(x) for x in self.params_per_chunk], (got, list(self.params_per_chunk))
+        return groups
+
+    def _accumulate(self, parts, rows):
+        """Sum of the chunk projections (fp32 each, as fast_jl returns them), returned in `dtype`."""
+        if self.accumulate_in_dtype:
+            acc = ch.zeros(size=(rows, self.proj_dim), device=self.device, dtype=self.dtype)
+            for part in parts:
+                acc.add_(part)  # fp32 + dtype -> rounded to dtype after every chunk, as the reference does
+            return acc
         acc = None
-        for index, (group, size) in enumerate(groups):
-            assert size == self.params_per_chunk[index]
-            if actual_bs != next(iter(group.values())).shape[0]:
-                group = {k: v[:actual_bs] for k, v in group.items()}
-            part = self.projector_per_chunk[index].project(group, model_id=model_id)
-            acc = part if acc is None else acc.add_(part)
+        for part in parts:
+            acc = part.to(ch.float32) if acc is None else acc.add_(part)
         return acc.to(self.dtype)
 
     def project(self, grads, model_id):
+        names = list(grads.keys())
         tensors = list(grads.values())
+        rows = tensors[0].shape[0]
+        if rows > self.feat_bs:
+            # the reference's packing buffer has feat_bs rows: a larger batch fails on its copy_
+            # (trak/projectors.py:500-502)
+            raise RuntimeError(f"batch of {rows} rows exceeds feat_bs = {self.feat_bs}")
+        groups = self._chunk_sizes(grads)
         if fast_jl.gather_supported(tensors) and tensors[0].dtype == self.dtype:
-            return self._project_in_place(grads, model_id)
-        self.allocate_input()
-        acc = ch.zeros(size=(self.feat_bs, self.proj_dim), device=self.device, dtype=ch.float32)
-        pointer = 0
-        projector_index = 0
-        actual_bs = 0
-        for p in grads.values():
-            if len(p.shape) < 2:
-                p_flat = p.data.unsqueeze(-1)
-            else:
-                p_flat = p.data.flatten(start_dim=1)
-
-            param_size = p_flat.size(1)
-            if pointer + param_size > self.max_chunk_size:
-                assert pointer == self.params_per_chunk[projector_index]
-                # the kernel takes the row pitch, so the packed prefix is projected in place
-                acc[:actual_bs].add_(
-                    self.projector_per_chunk[projector_index].project(
-                        self.ch_input[:actual_bs, :pointer], model_id=model_id
-                    )
-                )
-                pointer = 0
-                projector_index += 1
-
-            actual_bs = min(self.ch_input.size(0), p_flat.size(0))
-            self.ch_input[:actual_bs, pointer : pointer + param_size].copy_(p_flat)
-            pointer += param_size
-
-        assert pointer == self.params_per_chunk[projector_index]
-        acc[:actual_bs].add_(
-            self.projector_per_chunk[projector_index].project(
-                self.ch_input[:actual_bs, :pointer], model_id=model_id
+            # every chunk goes to its projector as a dict, which projects the tensors where they are
+            parts = (
+                self.projector_per_chunk[i].project({n: grads[n] for n in names[b:e]}, model_id=model_id)
+                for i, (b, e, _) in enumerate(groups)
             )
+            return self._accumulate(parts, rows)
+        # mixed dtypes or host tensors: one flat [rows, P] copy in `dtype` (what the reference's packing
+        # buffer holds after its copy_), projected chunk by chunk through column slices
+        flat = vectorize({n: t.to(self.dtype) for n, t in grads.items()}, device=self.device)
+        edges = [0]
+        for _, _, width in groups:
+            edges.append(edges[-1] + width)
+        parts = (
+            self.projector_per_chunk[i].project(flat[:, edges[i]:edges[i + 1]], model_id=model_id)
+            for i in range(len(groups))
         )
-        return acc[:actual_bs].to(self.dtype)
+        return self._accumulate(parts, rows)

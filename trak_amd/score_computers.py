@@ -66,6 +66,20 @@ class BasicScoreComputer(AbstractScoreComputer):
     power of two, two fp16 planes, three MFMAs per k step: entries keep 22 significand bits relative
     to their row's largest magnitude instead of all 24; 1.75 times the speed of "split").  fp16 / bf16
     operands are multiplied as they are (exact products) under "split" and "split2".
+
+    Differences from the reference that a caller can meet:
+      * the device must be a GPU (the reference also runs on "cpu");
+      * `X^T X + lambda I` is inverted by a Cholesky factorization.  When that fails - the matrix is
+        symmetric but not positive definite, which happens to a Gram matrix that was rounded to fp16
+        (TRAKer's default) or has deficient rank (fewer training points than proj_dim with
+        lambda_reg = 0) - it falls back to LU through torch.linalg.inv on the device, the call the
+        reference itself makes (trak/score_computers.py:163), and logs a warning; only an exactly
+        singular matrix or a non-finite inverse raises torch.linalg.LinAlgError;
+      * sums are kept in fp32 and rounded to `dtype` once.  accumulate_in_dtype=True reproduces the
+        reference's arithmetic instead: `X^T X` is the sum over blocks of CUDA_MAX_DIM_SIZE rows of
+        block products each rounded to `dtype`, the running sum rounded to `dtype` after every
+        block (trak/score_computers.py:147-153), and lambda is added in the dtype of `xtx`
+        (:160-162).  It costs one pass per block and only matters for fp16 / bf16 `dtype`.
     """
 
     def __init__(
@@ -76,8 +90,10 @@ class BasicScoreComputer(AbstractScoreComputer):
         logging_level=logging.INFO,
         lambda_reg: float = 0.0,
         gemm: str = "split",
+        accumulate_in_dtype: bool = False,
     ) -> None:
         super().__init__(dtype, device)
+        self.accumulate_in_dtype = accumulate_in_dtype
         if gemm not in ("split", "split2", "fp32"):
             raise ValueError('gemm must be "split", "split2" or "fp32"')
         self.gemm = gemm
@@ -95,22 +111,39 @@ class BasicScoreComputer(AbstractScoreComputer):
             return [grads]  # resident: one pass, the kernel walks all rows
         return ch.split(grads, split_size_or_sections=self.CUDA_MAX_DIM_SIZE, dim=0)
 
+    def _gram(self, block, out, beta):
+        if self.gemm != "fp32":
+            # the operand is block^T, read in place; lower-triangle tiles + mirror image
+            gram_split(self._split(block, transposed=True), out=out, alpha=1.0, beta=beta)
+        else:
+            gemm_tn(block, block, out=out, alpha=1.0, beta=beta)
+
     def get_xtx(self, grads: Tensor) -> Tensor:
         self.proj_dim = grads.shape[1]
+        if self.accumulate_in_dtype:
+            # trak/score_computers.py:147-153 to the letter: `result += block.T @ block` with both sides
+            # in `dtype`, blocks of CUDA_MAX_DIM_SIZE rows wherever the gradients live
+            result = ch.zeros(self.proj_dim, self.proj_dim, dtype=self.dtype, device=self._dev)
+            product = ch.empty(self.proj_dim, self.proj_dim, dtype=ch.float32, device=self._dev)
+            for block in ch.split(grads, split_size_or_sections=self.CUDA_MAX_DIM_SIZE, dim=0):
+                self._gram(block.to(self._dev), product, 0.0)
+                result += product.to(block.dtype)  # the block product in the gradients' type, as `block.T @ block` returns it
+            return result
         result = ch.zeros(self.proj_dim, self.proj_dim, dtype=ch.float32, device=self._dev)
         for block in self._blocks(grads):
-            block = block.to(self._dev)
-            if self.gemm != "fp32":
-                # the operand is block^T, read in place; lower-triangle tiles + mirror image
-                gram_split(self._split(block, transposed=True), out=result, alpha=1.0, beta=1.0)
-            else:
-                gemm_tn(block, block, out=result, alpha=1.0, beta=1.0)
+            self._gram(block.to(self._dev), result, 1.0)
         return result.to(self.dtype)
 
     def get_x_xtx_inv(self, grads: Tensor, xtx: Tensor) -> Tensor:
         # (xtx + lambda I)^-1 in fp32, divided by the mean absolute entry
         # (trak/score_computers.py:160-166)
-        xtx_inv, _ = spd_inverse(xtx.to(self._dev), lambda_reg=self.lambda_reg, normalize=True)
+        xtx = xtx.to(self._dev)
+        if self.accumulate_in_dtype:
+            # lambda is added in the dtype of xtx (trak/score_computers.py:160-162), then fp32
+            xtx_reg = xtx + self.lambda_reg * ch.eye(xtx.size(dim=0), device=xtx.device, dtype=xtx.dtype)
+            xtx_inv, _ = spd_inverse(xtx_reg, lambda_reg=0.0, normalize=True, general_fallback=True)
+        else:
+            xtx_inv, _ = spd_inverse(xtx, lambda_reg=self.lambda_reg, normalize=True, general_fallback=True)
         xtx_inv = xtx_inv.to(self.dtype)
 
         result = ch.empty(grads.shape[0], xtx_inv.shape[1], dtype=ch.float32, device=self._dev)

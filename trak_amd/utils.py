@@ -4,6 +4,7 @@ Mirrors the hot-path part of the reference's trak/utils.py: `vectorize` (:80-110
 `get_parameter_chunk_sizes` (:297-331) and `get_matrix_mult` (:248-294).
 """
 import ctypes
+import logging
 
 import numpy as np
 import torch
@@ -356,10 +357,16 @@ def gram_split(a, out=None, alpha=1.0, beta=0.0):
     return out
 
 
-def spd_inverse(a, lambda_reg=0.0, normalize=False):
+def spd_inverse(a, lambda_reg=0.0, normalize=False, general_fallback=False):
     """(a + lambda*I)^-1 for a symmetric positive definite fp32 matrix on the GPU; with
     normalize=True the result is divided by mean(|inverse|) (trak/score_computers.py:160-166).
-    Returns (inverse, mean_abs tensor of 1 element)."""
+    Returns (inverse, mean_abs tensor of 1 element).
+
+    A matrix that is not positive definite raises torch.linalg.LinAlgError, unless
+    general_fallback=True: then it is inverted by LU with torch.linalg.inv on the device - the very
+    call the reference makes at trak/score_computers.py:163 - which returns something for every
+    matrix that is not exactly singular (a Gram matrix rounded to fp16, or one of deficient rank,
+    is symmetric but need not be positive definite)."""
     if a.dim() != 2 or a.shape[0] != a.shape[1]:
         raise RuntimeError("spd_inverse needs a square matrix")
     a = _as_f32_rows(a, "a")
@@ -391,9 +398,20 @@ def spd_inverse(a, lambda_reg=0.0, normalize=False):
         _lib.check(code)
         bad = int(status.item())  # also orders the workspace's lifetime after the kernels
     if bad != 0:
-        raise torch.linalg.LinAlgError(
-            f"spd_inverse: the matrix is not positive definite (pivot {bad - 1} is not positive)"
+        if not general_fallback:
+            raise torch.linalg.LinAlgError(
+                f"spd_inverse: the matrix is not positive definite (pivot {bad - 1} is not positive)"
+            )
+        logging.getLogger("ScoreComputer").warning(
+            "X^T X + lambda I is not positive definite (pivot %d): inverting it by LU, as the reference does", bad - 1
         )
+        reg = a + float(lambda_reg) * torch.eye(n, device=a.device, dtype=torch.float32)
+        inv = torch.linalg.inv(reg)  # raises LinAlgError for an exactly singular matrix, like the reference
+        if not bool(torch.isfinite(inv).all()):
+            raise torch.linalg.LinAlgError("spd_inverse: the inverse has non-finite entries")
+        mean_abs = inv.abs().mean().reshape(1)
+        if normalize:
+            inv = inv / mean_abs
     return inv, mean_abs
 
 
