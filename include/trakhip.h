@@ -43,6 +43,7 @@ extern "C" {
 #define TRAKHIP_ERR_NO_DEVICE -10
 #define TRAKHIP_ERR_POINTER -11  /* destination is neither device memory nor page-locked host memory */
 #define TRAKHIP_ERR_STATIC_LIMIT -12 /* trakhip_project_static: shape needs more than its static scratch */
+#define TRAKHIP_ERR_HOST_MEMORY -13  /* host-side bookkeeping of a call could not be allocated */
 
 const char* trakhip_strerror(int code);
 

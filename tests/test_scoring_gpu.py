@@ -138,6 +138,60 @@ def test_spd_inverse_closed_forms_and_failure(gpu):
         spd_inverse(bad.to(gpu))
 
 
+def test_gram_matrices_that_are_not_positive_definite(gpu):
+    # The reference inverts with LU (trak/score_computers.py:163), which returns something for every
+    # matrix that is not exactly singular; the Cholesky path needs a positive definite matrix.
+    from trak_amd import BasicScoreComputer
+
+    gen = torch.Generator().manual_seed(3)
+    # (1) fewer training points than proj_dim, ridge > 0: rank-deficient Gram + lambda I is positive
+    #     definite, and the inverse must match float64
+    N, k, lam = 60, 256, 1e-2
+    X = torch.randn(N, k, generator=gen) / 8
+    sc = BasicScoreComputer(dtype=torch.float32, device=gpu, lambda_reg=lam)
+    xtx = sc.get_xtx(X.to(gpu))
+    feats = sc.get_x_xtx_inv(X.to(gpu), xtx).cpu().numpy().astype(np.float64)
+    x64 = X.numpy().astype(np.float64)
+    inv64 = np.linalg.inv(x64.T @ x64 + lam * np.eye(k))
+    want = x64 @ (inv64 / np.abs(inv64).mean())
+    # X lies in the span where the inverse is small (1/9 .. 1) while the inverse itself is dominated by
+    # 1/lambda = 100 on the complement: X @ inv cancels two orders of magnitude, so fp32 arithmetic
+    # (this library's or torch.linalg.inv's alike) gives these features to about 1e-4, not 1e-6
+    err = np.abs(feats - want).max() / np.abs(want).max()
+    ref = torch.linalg.inv(xtx.double().cpu().float() + lam * torch.eye(k))
+    ref_err = np.abs((X @ (ref / ref.abs().mean())).numpy() - want).max() / np.abs(want).max()
+    assert err < max(1e-3, 3 * ref_err)
+    # (2) the same with lambda_reg = 0 (TRAKer's default): the Gram matrix is singular up to rounding.
+    #     The Cholesky path fails and the LU fallback answers with finite values, as the reference does,
+    #     or raises LinAlgError when LU itself finds the matrix singular - never anything else
+    sc0 = BasicScoreComputer(dtype=torch.float32, device=gpu, lambda_reg=0.0)
+    #     (the inverse of a numerically singular matrix is rounding noise, so there are no values to compare)
+    try:
+        f0 = sc0.get_x_xtx_inv(X.to(gpu), xtx)
+        assert f0.shape == (N, k) and torch.isfinite(f0).all()
+    except torch.linalg.LinAlgError:
+        pass
+    # (3) an ill-conditioned Gram matrix rounded to fp16 (TRAKer's use_half_precision default hands the
+    #     inverse exactly this): the rounding makes it indefinite.  The result must be the inverse of the
+    #     matrix that was handed over, as the reference's LU gives it
+    k = 192
+    q, _ = torch.linalg.qr(torch.randn(k, k, generator=gen, dtype=torch.float64))
+    spectrum = 1000.0 / torch.arange(1, k + 1, dtype=torch.float64) ** 2.5      # condition number 5e5
+    gram = ((q * spectrum) @ q.T).half()
+    g64 = gram.double().numpy()
+    assert np.linalg.eigvalsh((g64 + g64.T) / 2).min() < 0                       # indefinite after the rounding
+    with pytest.raises(torch.linalg.LinAlgError):
+        spd_inverse(gram.float().to(gpu))
+    inv, mean_abs = spd_inverse(gram.float().to(gpu), normalize=True, general_fallback=True)
+    ref = torch.linalg.inv(gram.float().to(gpu))          # the reference's call on the same matrix
+    assert torch.allclose(mean_abs, ref.abs().mean().reshape(1), rtol=1e-5)
+    assert torch.allclose(inv * mean_abs, ref, rtol=1e-4, atol=1e-4 * float(ref.abs().max()))
+    sch = BasicScoreComputer(dtype=torch.float16, device=gpu, lambda_reg=0.0)
+    Xh = (torch.randn(500, k, generator=gen) / 8).half().to(gpu)
+    out = sch.get_x_xtx_inv(Xh, gram.to(gpu))
+    assert out.dtype == torch.float16 and torch.isfinite(out).all()
+
+
 def split_planes_to_numpy(op):
     """[planes, padded rows, padded K] float32 view of a SplitOperand (layout: plane, k-octet, row,
     8 values of 16 bits: bf16 for an fp32 or bf16 source, fp16 for an fp16 source)."""

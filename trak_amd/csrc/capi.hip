@@ -21,6 +21,7 @@ const char* trakhip_strerror(int code) {
             return "destination is neither device memory nor page-locked host memory";
         case TRAKHIP_ERR_STATIC_LIMIT:
             return "shape needs more scratch than the static array of trakhip_project_static holds";
+        case TRAKHIP_ERR_HOST_MEMORY: return "out of host memory while planning the call";
         default: return "unknown trakhip error";
     }
 }

@@ -405,7 +405,7 @@ void collect_nodes(uint64_t lo, uint64_t hi, size_t depth, std::vector<std::vect
     collect_nodes(mid, hi, depth + 1, levels);
 }
 
-int tri_inverse(Ctx& c, uint64_t nblk) {
+int tri_inverse_impl(Ctx& c, uint64_t nblk) {
     std::vector<std::vector<Node>> levels;
     collect_nodes(0, nblk, 0, levels);
     const uint64_t np = c.np;
@@ -437,6 +437,15 @@ int tri_inverse(Ctx& c, uint64_t nblk) {
         }
     }
     return TRAKHIP_OK;
+}
+
+// The node lists live in host containers; nothing they throw (std::bad_alloc) may cross the C ABI.
+int tri_inverse(Ctx& c, uint64_t nblk) {
+    try {
+        return tri_inverse_impl(c, nblk);
+    } catch (...) {
+        return TRAKHIP_ERR_HOST_MEMORY;
+    }
 }
 
 }  // namespace

@@ -12,20 +12,22 @@ import torch
 from . import _lib
 
 _DTYPES = {torch.float16: _lib.F16, torch.bfloat16: _lib.BF16, torch.float32: _lib.F32}
-_workspaces = {}
-_segment_tables = {}  # (device, rows) -> device table; the key holds every pointer, so a hit is exact
+_workspaces = {}      # (device, stream) -> scratch buffer
+_segment_tables = {}  # (device, stream, rows) -> device table; the key holds every pointer, so a hit is exact
 _SEGMENT_TABLE_CACHE = 16
 
 
 def _workspace(device, nbytes):
-    """One growing scratch buffer per device (stands in for the per-call torch::zeros of
-    fast_jl/fast_jl.cu:48-49).  Calls on one device must not overlap on different streams."""
-    buf = _workspaces.get(device)
+    """One growing scratch buffer per device and stream (stands in for the per-call torch::zeros of
+    fast_jl/fast_jl.cu:48-49): calls on different streams never share scratch, calls on one stream
+    are ordered by the stream."""
+    key = (device, torch.cuda.current_stream(device).cuda_stream)
+    buf = _workspaces.get(key)
     if buf is None or buf.numel() < nbytes:
         buf = None
-        _workspaces.pop(device, None)
+        _workspaces.pop(key, None)
         buf = torch.empty(max(nbytes, 1), dtype=torch.uint8, device=device)
-        _workspaces[device] = buf
+        _workspaces[key] = buf
     return buf
 
 
@@ -37,8 +39,9 @@ def free_workspaces():
 def _segment_table(device, rows):
     """Device array of trakhip_segment {ptr, first, numel, ld} for these rows.  Gradient buffers
     come back at the same addresses batch after batch (caching allocator), so the upload is
-    usually skipped."""
-    key = (device, rows)
+    usually skipped.  The cache is per stream: the upload is enqueued on the stream that later
+    reads the table, so a hit never races with it."""
+    key = (device, torch.cuda.current_stream(device).cuda_stream, rows)
     table = _segment_tables.get(key)
     if table is None:
         if len(_segment_tables) >= _SEGMENT_TABLE_CACHE:
