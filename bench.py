@@ -9,10 +9,15 @@ step      = one `trakhip_project` call on one resident batch [32, 11_689_512] fp
 value     = 2*B*P*k flop per step / time per step, in TFLOP/s.
 roofline  = the projection kernel alone (phase 1 of the call), timed with HIP events recorded
             on the launch stream around every launch, against the dense fp16 MFMA peak.
-cpu_baseline = the CPU restatement of trak's BasicProjector (oracle/basic_projector.py) on the
-            CPU-runnable configuration ([16, 1_048_576] fp32 -> 512), timed on this host.
+cpu_baseline = the CPU restatement of trak's BasicProjector (oracle/basic_projector.py) timed on this host:
+            the CPU-runnable configuration ([16, 1_048_576] fp32 -> 512) in full, the ResNet-9- and
+            ResNet-18-sized configurations as two full 100-column blocks each, scaled by num_blocks / 2
+            and flagged "extrapolated" (the BERT-sized one only with --cpu-c4).
+sustained = the same calls back to back for --sustain seconds (default 2).
 `scoring` = BasicScoreComputer at N=50_000, M=10_000, k=4096 fp32: GEMM TFLOP/s against the fp32
             MFMA peak, the SPD inverse separately, and a CPU sample beside it.
+`--only NAME` runs one workload alone (for profiler runs): c1 | c2 | c3_dict | c4 | c4_rademacher |
+            scoring | mfma_rate.
 """
 import argparse
 import ctypes
