@@ -111,6 +111,44 @@ def test_tiny_values_and_exact_zeros(gpu, c_oracle, dtype):
     assert rel_l2_rows(out[:, :64].cpu().numpy(), want).max() < TOL[dtype]
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("k", [512, 1024])
+def test_normal_projection_follows_the_rows_scale_from_chunk_to_chunk(gpu, c_oracle, dtype, k):
+    # The normal kernel brings every 256-feature chunk of a row to fp16 with the row's own power of two
+    # and carries the accumulators from one chunk's factor to the next.  Blocks of features whose sizes
+    # differ by up to 2^±80 (far outside fp16), rows of different magnitude, all-zero stretches and
+    # rows that are zero throughout must all come out as the float64 contraction says.
+    B, P, tiles, seed = 23, 9_000, 7, 31
+    gen = torch.Generator(device="cpu").manual_seed(12)
+    expo = torch.randint(-80, 81, (P // 300,), generator=gen).double()
+    expo[::7] = 0
+    scale = (2.0 ** expo).repeat_interleave(300)[None, :]
+    g = (torch.randn(B, P, generator=gen).double() * scale)
+    g *= (2.0 ** torch.randint(-20, 21, (B, 1), generator=gen).double())   # every row its own size
+    g[:, 1200:2100] = 0.0           # an all-zero stretch longer than three chunks
+    g[5] = 0.0                      # a row of zeros
+    g[7, :] = 0.0
+    g[7, 4321] = 3.0                # a one-hot row
+    g = g.to(dtype)
+    assert torch.isfinite(g).all()
+    out = fn(G)(g.to(gpu), k, seed, tiles)
+    assert torch.isfinite(out).all()
+    want = c_oracle.project(to_f32_numpy(g), seed, tiles, k - 40, 40, G)
+    got = out[:, k - 40 :].cpu().numpy().astype(np.float64)
+    live = np.linalg.norm(want, axis=1) > 0
+    assert not live[5] and not got[5].any()
+    assert rel_l2_rows(got[live], want[live]).max() < TOL[dtype]
+    # the one-hot row reads the matrix row back exactly (3 * entry is exact in fp32)
+    s_row = c_oracle.materialize(seed, tiles, P, 4321, 1, 0, k, G)[0]
+    assert np.array_equal(out[7].cpu().numpy(), 3.0 * s_row)
+    # scaling a row by a power of two scales its projection exactly
+    g2 = g.clone()
+    g2[3] *= 2.0 ** 9
+    out2 = fn(G)(g2.to(gpu), k, seed, tiles)
+    assert torch.equal(out2[3], out[3] * 2.0 ** 9)
+    assert torch.equal(out2[4], out[4])
+
+
 def test_row_pitch_and_unaligned_rows(gpu, c_oracle):
     # a column slice of a wider buffer (pitch > P) whose rows start at odd element offsets
     B, P, k, tiles, seed = 16, 3001, 512, 256, 3
