@@ -129,6 +129,12 @@ def test_normal_projection_follows_the_rows_scale_from_chunk_to_chunk(gpu, c_ora
     g[5] = 0.0                      # a row of zeros
     g[7, :] = 0.0
     g[7, 4321] = 3.0                # a one-hot row
+    # one huge chunk followed by tiny ones, and the reverse: sums carried from a chunk of magnitude 2^90 must
+    # not be blown up when chunks of magnitude 2^-90 follow, nor swamp a huge chunk that comes last
+    g[9] = torch.randn(P, generator=gen).double() * 2.0 ** -90
+    g[9, :256] = torch.randn(256, generator=gen).double() * 2.0 ** 90
+    g[10] = torch.randn(P, generator=gen).double() * 2.0 ** -90
+    g[10, P - 256 :] = torch.randn(256, generator=gen).double() * 2.0 ** 90
     g = g.to(dtype)
     assert torch.isfinite(g).all()
     out = fn(G)(g.to(gpu), k, seed, tiles)

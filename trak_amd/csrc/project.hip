@@ -567,10 +567,10 @@ __global__ __launch_bounds__(64 * W, 2) void jl_project_kernel(
 //   * the matrix entries are fp16 whatever the gradient type is, so the gradients are brought to
 //     fp16 once per chunk at staging time instead of splitting every entry into bf16 terms in the
 //     hot loop: bf16 and fp32 chunks are multiplied row by row by the power of two that puts the
-//     row's largest magnitude into [2^14, 2^15) (bf16: one exact fp16 plane for everything within
-//     2^-31 of it; fp32: two planes h1 + h2, 22 significant bits), the accumulators follow the
-//     row's factor from chunk to chunk (v_ldexp_f32, exact) and the factor is taken out again
-//     before the partial sums are written.
+//     largest magnitude the row has shown so far into [2^14, 2^15) (bf16: one exact fp16 plane for
+//     everything within 2^-31 of it; fp32: two planes h1 + h2, 22 significant bits), the
+//     accumulators are scaled down when that maximum grows (v_ldexp_f32, exact) and the factor is
+//     taken out again before the partial sums are written.
 
 typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
 typedef unsigned short ushort2_t __attribute__((ext_vector_type(2)));
@@ -600,9 +600,26 @@ struct NormalTraits<TRAKHIP_F32> {
     static constexpr bool scaled = true;
 };
 
-// Power of two that brings a row whose largest binary32 exponent field is emax into [2^14, 2^15);
-// an all-zero (or all-subnormal) row keeps its scale.
-__device__ __forceinline__ int row_shift(uint32_t emax) { return emax ? 141 - (int)emax : 0; }
+// Power of two that brings a row whose largest binary32 exponent field is emax into [2^14, 2^15).
+// A row keeps ONE reference exponent that only ever moves towards larger magnitudes: the smallest
+// such power over the chunks seen so far (kNoScale until the first chunk that is not all zero).  A
+// chunk is converted with the reference, so whatever it holds below 2^-38 of the row's running
+// maximum rounds away (it could not change the row's result beyond 2^-38 of its size), and the
+// accumulators are only ever scaled down when the reference moves - they cannot overflow.
+constexpr int kNoScale = 1 << 20;
+struct RowScale {
+    int use;    // exponent applied to this chunk
+    int delta;  // change against the exponent the accumulators carry (<= 0)
+};
+__device__ __forceinline__ RowScale next_row_scale(uint32_t emax, int& ref) {
+    const int want = emax ? 141 - (int)emax : kNoScale;
+    const int prev = ref;
+    ref = want < ref ? want : ref;
+    RowScale r;
+    r.use = ref == kNoScale ? 0 : ref;
+    r.delta = prev == kNoScale ? 0 : r.use - prev;
+    return r;
+}
 
 // Slot of row m in the per-chunk exponent lists: lane half h reads its sixteen accumulator rows
 // m = 8*(r/4) + 4*h + r%4 (r = 0..15) as sixteen consecutive ints.
@@ -614,9 +631,9 @@ __device__ __forceinline__ uint32_t pack_f16_rne(float a, float b) {
 }
 
 // bf16 chunk -> one scaled fp16 plane.  The 32 threads that share tid / 32 hold one row (two rows
-// per thread, 16 apart); sh_prev[] is the row's exponent in the previous chunk.
+// per thread, 16 apart); sh_ref[] is the row's reference exponent so far.
 __device__ __forceinline__ void store_scaled_bf16(const uint4 (&v)[2], uint16_t* lds, int (*sh)[32], int tid,
-                                                  int (&sh_prev)[2]) {
+                                                  int (&sh_ref)[2]) {
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
         const uint32_t row = (tid >> 5) + 16 * i, sg = tid & 31;
@@ -630,25 +647,24 @@ __device__ __forceinline__ void store_scaled_bf16(const uint4 (&v)[2], uint16_t*
             const uint32_t o = (uint32_t)__shfl_xor((int)e, d, 64);
             e = o > e ? o : e;
         }
-        const int shift = row_shift(e >> 7);
+        const RowScale rs = next_row_scale(e >> 7, sh_ref[i]);
         uint32_t h[4];
 #pragma unroll
         for (int t = 0; t < 4; ++t)
-            h[t] = pack_f16_rne(ldexpf(__uint_as_float(w[t] << 16), shift),
-                                ldexpf(__uint_as_float(w[t] & 0xFFFF0000u), shift));
+            h[t] = pack_f16_rne(ldexpf(__uint_as_float(w[t] << 16), rs.use),
+                                ldexpf(__uint_as_float(w[t] & 0xFFFF0000u), rs.use));
         *reinterpret_cast<uint4*>(lds + row * kLdsRow + 8 * sg) = uint4{h[0], h[1], h[2], h[3]};
         if (sg == 0) {
-            sh[0][row_slot(row)] = shift - sh_prev[i];
-            sh[1][row_slot(row)] = shift;
+            sh[0][row_slot(row)] = rs.delta;
+            sh[1][row_slot(row)] = rs.use;
         }
-        sh_prev[i] = shift;
     }
 }
 
 // fp32 chunk -> two scaled fp16 planes.  The 64 threads of a wave hold one row (four rows per
 // thread, 8 apart).
 __device__ __forceinline__ void store_scaled_f32(const uint4 (&v)[4], uint16_t* lds, int (*sh)[32], int tid,
-                                                 int (&sh_prev)[4]) {
+                                                 int (&sh_ref)[4]) {
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
         const uint32_t row = (tid >> 6) + 8 * i, sg = tid & 63;
@@ -664,12 +680,12 @@ __device__ __forceinline__ void store_scaled_f32(const uint4 (&v)[4], uint16_t* 
             const uint32_t o = (uint32_t)__shfl_xor((int)e, d, 64);
             e = o > e ? o : e;
         }
-        const int shift = row_shift(e);
+        const RowScale rs = next_row_scale(e, sh_ref[i]);
         float g[4], r[4];
         _Float16 h1[4];
 #pragma unroll
         for (int t = 0; t < 4; ++t) {
-            g[t] = ldexpf(__uint_as_float(w[t]), shift);
+            g[t] = ldexpf(__uint_as_float(w[t]), rs.use);
             h1[t] = (_Float16)g[t];
             r[t] = g[t] - (float)h1[t];  // exact
         }
@@ -679,10 +695,9 @@ __device__ __forceinline__ void store_scaled_f32(const uint4 (&v)[4], uint16_t* 
         *reinterpret_cast<uint2*>(lds + kPlaneElems + row * kLdsRow + 4 * sg) =
             uint2{pack_f16_rne(r[0], r[1]), pack_f16_rne(r[2], r[3])};
         if (sg == 0) {
-            sh[0][row_slot(row)] = shift - sh_prev[i];
-            sh[1][row_slot(row)] = shift;
+            sh[0][row_slot(row)] = rs.delta;
+            sh[1][row_slot(row)] = rs.use;
         }
-        sh_prev[i] = shift;
     }
 }
 
@@ -762,16 +777,16 @@ __global__ __launch_bounds__(512, 2) void jl_project_normal_kernel(
     const uint32_t a_off = n * kLdsRow + 128 * h;
 
     Stage st;
-    int sh_prev[Stage::N];
+    int sh_ref[Stage::N];
 #pragma unroll
-    for (int i = 0; i < Stage::N; ++i) sh_prev[i] = 0;
+    for (int i = 0; i < Stage::N; ++i) sh_ref[i] = kNoScale;
     auto stage_store = [&](int buf) {
         if constexpr (IN == TRAKHIP_F16)
             st.store(lds + buf * kBufElems, tid);
         else if constexpr (IN == TRAKHIP_BF16)
-            store_scaled_bf16(st.v, lds + buf * kBufElems, sh_lds[buf], tid, sh_prev);
+            store_scaled_bf16(st.v, lds + buf * kBufElems, sh_lds[buf], tid, sh_ref);
         else
-            store_scaled_f32(st.v, lds + buf * kBufElems, sh_lds[buf], tid, sh_prev);
+            store_scaled_f32(st.v, lds + buf * kBufElems, sh_lds[buf], tid, sh_ref);
     };
     {
         const uint64_t lo = (uint64_t)t0 * tile_size;
@@ -811,7 +826,7 @@ __global__ __launch_bounds__(512, 2) void jl_project_normal_kernel(
             const uint16_t* a_base = lds + cur * kBufElems + a_off;
 
             if (kScaled) {
-                // the rows of this chunk carry other powers of two than those of the last one
+                // rows whose reference exponent moved with this chunk: bring their sums along (down only)
                 const int4* dp = reinterpret_cast<const int4*>(&sh_lds[cur][0][16 * h]);
                 int d[16];
 #pragma unroll
