@@ -10,8 +10,12 @@
  *                         reference's own generator is cuRAND XORWOW (fast_jl/random.cuh:19),
  *                         which is replaced by Philox in this build.
  *                         PINNED by Random123's kat_vectors (tests/test_oracle_philox.py).
- *   jlo_stream_seed       fast_jl/random.cuh:15-17  (closed form, uint32 wrap).  PINNED by
- *                         hand-computed values.
+ *   jlo_stream_name       fast_jl/random.cuh:15-17  (closed form, uint32 wrap): the 32-bit value
+ *                         that names the stream of (column, tile); the reference seeds the
+ *                         pair's generator with it.  PINNED by hand-computed values.
+ *   jlo_stream_block      block number n of the stream named s: Philox with counter
+ *                         (n, s, 0, 0) and key (seed, 0) - a definition of this build.
+ *                         PINNED by Random123's kat_vectors through jlo_philox4x32_10.
  *   jlo_tiling            fast_jl/fast_jl.cu:42 (T = min(F, tiles)) and
  *                         fast_jl/fast_jl_kernel.cuh:124 (fts = ceil(F / T)).  PINNED by the
  *                         iteration counts of the reference's shapes.
@@ -62,9 +66,15 @@ void jlo_philox4x32_10(const uint32_t ctr[4], const uint32_t key[2], uint32_t ou
     out[3] = c3;
 }
 
-uint32_t jlo_stream_seed(uint32_t seed, uint32_t column, uint32_t tile) {
+uint32_t jlo_stream_name(uint32_t seed, uint32_t column, uint32_t tile) {
     uint64_t v = (uint64_t)seed + (uint64_t)658105236u * column + (uint64_t)359124577u * tile;
     return (uint32_t)(v & 0xFFFFFFFFu);
+}
+
+void jlo_stream_block(uint32_t seed, uint32_t name, uint32_t block, uint32_t out[4]) {
+    uint32_t ctr[4] = {block, name, 0u, 0u};
+    uint32_t key[2] = {seed, 0u};
+    jlo_philox4x32_10(ctr, key, out);
 }
 
 void jlo_tiling(uint64_t P, uint32_t num_feature_tiles, uint32_t* tiles, uint64_t* tile_size) {
@@ -235,21 +245,16 @@ float jlo_entry(uint32_t seed, uint32_t num_feature_tiles, uint64_t P, uint64_t 
     jlo_tiling(P, num_feature_tiles, &tiles, &tile_size);
     uint32_t tile = (uint32_t)(f / tile_size);
     uint32_t offset = (uint32_t)(f - (uint64_t)tile * tile_size);
-    uint32_t key[2] = {jlo_stream_seed(seed, c, tile), 0u};
     uint32_t out[4];
     if (proj_type == JLO_RADEMACHER) {
-        uint32_t ctr[4] = {offset / 128u, 0u, 0u, 0u};
-        jlo_philox4x32_10(ctr, key, out);
-        uint32_t j = offset % 128u;
-        uint32_t mfma_index = j / 8u;       /* which of the 16 shifts */
-        uint32_t slot = j % 8u;             /* which of the lane's 8 operand elements */
-        uint32_t word = out[slot / 2u];
-        uint32_t bitpos = (slot % 2u ? 31u : 15u) - mfma_index;
-        return ((word >> bitpos) & 1u) ? 1.0f : -1.0f;
+        /* 128 entries per block: entry number i is bit i of the block, words in order, least
+         * significant bit first */
+        jlo_stream_block(seed, jlo_stream_name(seed, c, tile), offset / 128u, out);
+        uint32_t bit = offset % 128u;
+        return ((out[bit / 32u] >> (bit % 32u)) & 1u) ? 1.0f : -1.0f;
     } else {
         /* eight entries per block; word i of the block makes entries 2i (cosine) and 2i+1 (sine) */
-        uint32_t ctr[4] = {offset / 8u, 0u, 0u, 0u};
-        jlo_philox4x32_10(ctr, key, out);
+        jlo_stream_block(seed, jlo_stream_name(seed, c, tile), offset / 8u, out);
         uint32_t e = offset % 8u;
         return jlo_normal_from_word(out[e / 2u], (int)(e % 2u));
     }
@@ -282,19 +287,14 @@ void jlo_project(const float* G, uint64_t B, uint64_t P, uint64_t ld, uint32_t s
             uint64_t lo = (uint64_t)t * tile_size;
             uint64_t hi = lo + tile_size < P ? lo + tile_size : P;
             if (lo >= hi) continue;
-            uint32_t key[2] = {jlo_stream_seed(seed, c, t), 0u};
             for (uint64_t base = lo; base < hi; base += 128) {
                 uint64_t cnt = hi - base < 128 ? hi - base : 128;
                 uint32_t off0 = (uint32_t)(base - lo);
                 if (proj_type == JLO_RADEMACHER) {
-                    uint32_t ctr[4] = {off0 / 128u, 0u, 0u, 0u};
                     uint32_t w[4];
-                    jlo_philox4x32_10(ctr, key, w);
-                    for (uint32_t jj = 0; jj < cnt; ++jj) {
-                        uint32_t word = w[(jj % 8u) / 2u];
-                        uint32_t bitpos = ((jj % 8u) % 2u ? 31u : 15u) - jj / 8u;
-                        col[jj] = ((word >> bitpos) & 1u) ? 1.0f : -1.0f;
-                    }
+                    jlo_stream_block(seed, jlo_stream_name(seed, c, t), off0 / 128u, w);
+                    for (uint32_t jj = 0; jj < cnt; ++jj)
+                        col[jj] = ((w[jj / 32u] >> (jj % 32u)) & 1u) ? 1.0f : -1.0f;
                 } else {
                     for (uint32_t jj = 0; jj < cnt; ++jj)
                         col[jj] = jlo_entry(seed, num_feature_tiles, P, base + jj, c, proj_type);

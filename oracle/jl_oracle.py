@@ -6,7 +6,9 @@ from the specification, not from the C oracle or the library's header).  Only te
 __graft_entry__.smoke() and the cpu_baseline leg of bench.py may import it.
 
 Restated reference behaviour (MadryLab/trak):
-  * stream_seed   -- fast_jl/random.cuh:15-17
+  * stream_name   -- fast_jl/random.cuh:15-17: the 32-bit value that names the random stream of
+    a (JL column, feature tile) pair (the reference seeds the pair's generator with it); block n
+    of the stream named s is Philox(counter = (n, s, 0, 0), key = (seed, 0))
   * tiling        -- fast_jl/fast_jl.cu:42, fast_jl/fast_jl_kernel.cuh:124
   * Rademacher: one random bit per entry, bit set -> +1 -- fast_jl/random.cuh:33-37
   * Normal: Box-Muller normal in fp16 (fp16 radius times fp16 cos/sin, rounded once)
@@ -52,13 +54,22 @@ def philox4x32_10(ctr, key):
     return np.stack(c, axis=-1).astype(np.uint32)
 
 
-def stream_seed(seed, column, tile):
+def stream_name(seed, column, tile):
     v = (
         np.uint64(seed)
         + np.uint64(658105236) * np.asarray(column, dtype=np.uint64)
         + np.uint64(359124577) * np.asarray(tile, dtype=np.uint64)
     )
     return (v & _MASK).astype(np.uint32)
+
+
+def stream_blocks(seed, name, block):
+    """Blocks of the streams named `name`, broadcast over the arguments -> (..., 4) uint32."""
+    name, block = np.broadcast_arrays(np.asarray(name, dtype=np.uint32), np.asarray(block, dtype=np.uint32))
+    ctr = np.stack([block, name, np.zeros_like(block), np.zeros_like(block)], axis=-1)
+    key = np.zeros(block.shape + (2,), dtype=np.uint32)
+    key[..., 0] = np.uint32(seed & 0xFFFFFFFF)
+    return philox4x32_10(ctr, key)
 
 
 def tiling(P, num_feature_tiles):
@@ -199,21 +210,15 @@ def materialize(seed, num_feature_tiles, P, f0, nf, c0, nc, proj_type):
     tile = f // np.uint64(tile_size)
     off = (f - tile * np.uint64(tile_size)).astype(np.uint32)
     off = np.broadcast_to(off, (nf, nc))
-    key = np.zeros((nf, nc, 2), dtype=np.uint32)
-    key[..., 0] = stream_seed(seed, np.broadcast_to(c, (nf, nc)), np.broadcast_to(tile, (nf, nc)))
-    ctr = np.zeros((nf, nc, 4), dtype=np.uint32)
+    name = stream_name(seed, np.broadcast_to(c, (nf, nc)), np.broadcast_to(tile, (nf, nc)))
     if proj_type == RADEMACHER:
-        ctr[..., 0] = off // np.uint32(128)
-        w = philox4x32_10(ctr, key)
-        j = off % np.uint32(128)
-        shift_index = j // np.uint32(8)
-        slot = j % np.uint32(8)
-        word = np.take_along_axis(w, (slot // np.uint32(2))[..., None].astype(np.int64), axis=-1)[..., 0]
-        bitpos = np.where(slot % np.uint32(2) == 1, 31, 15).astype(np.uint32) - shift_index
-        bit = (word >> bitpos) & np.uint32(1)
+        # entry i of a 128-entry block is bit i of the block: word i // 32, bit i % 32
+        w = stream_blocks(seed, name, off // np.uint32(128))
+        i = off % np.uint32(128)
+        word = np.take_along_axis(w, (i // np.uint32(32))[..., None].astype(np.int64), axis=-1)[..., 0]
+        bit = (word >> (i % np.uint32(32))) & np.uint32(1)
         return np.where(bit == 1, np.float32(1.0), np.float32(-1.0)).astype(np.float32)
-    ctr[..., 0] = off // np.uint32(8)
-    w = philox4x32_10(ctr, key)
+    w = stream_blocks(seed, name, off // np.uint32(8))
     e = off % np.uint32(8)
     word = np.take_along_axis(w, (e // np.uint32(2))[..., None].astype(np.int64), axis=-1)[..., 0]
     return normal_from_word(word, e % np.uint32(2) == 1).astype(np.float32)
@@ -260,8 +265,10 @@ class COracle:
         up = ctypes.POINTER(u32)
         lib.jlo_philox4x32_10.argtypes = [up, up, up]
         lib.jlo_philox4x32_10.restype = None
-        lib.jlo_stream_seed.argtypes = [u32, u32, u32]
-        lib.jlo_stream_seed.restype = u32
+        lib.jlo_stream_name.argtypes = [u32, u32, u32]
+        lib.jlo_stream_name.restype = u32
+        lib.jlo_stream_block.argtypes = [u32, u32, u32, up]
+        lib.jlo_stream_block.restype = None
         lib.jlo_tiling.argtypes = [u64, u32, up, ctypes.POINTER(u64)]
         lib.jlo_tiling.restype = None
         lib.jlo_entry.argtypes = [u32, u32, u64, u64, u32, i32]
@@ -286,8 +293,13 @@ class COracle:
         self.lib.jlo_philox4x32_10(c, k, o)
         return [int(x) for x in o]
 
-    def stream_seed(self, seed, column, tile):
-        return int(self.lib.jlo_stream_seed(seed, column, tile))
+    def stream_name(self, seed, column, tile):
+        return int(self.lib.jlo_stream_name(seed, column, tile))
+
+    def stream_block(self, seed, name, block):
+        o = (ctypes.c_uint32 * 4)()
+        self.lib.jlo_stream_block(seed, name, block, o)
+        return [int(x) for x in o]
 
     def tiling(self, P, num_feature_tiles):
         t = ctypes.c_uint32()

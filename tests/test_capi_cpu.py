@@ -80,7 +80,7 @@ def test_workspace_size():
     assert lib.trakhip_project_workspace(32, 11_689_512, 4096, 256) == 64 * 32 * 4096 * 4
     assert lib.trakhip_project_workspace(48, 1000, 512, 256) == 256 * 32 * 512 * 4      # 256 tiles x 1 chunk
     assert lib.trakhip_project_workspace(8, 25, 1024, 256) == 25 * 8 * 1024 * 4
-    assert lib.trakhip_project_workspace(16, 1_048_576, 512, 256) == 512 * 16 * 512 * 4  # runs shorter than a tile
+    assert lib.trakhip_project_workspace(16, 1_048_576, 512, 256) == 256 * 16 * 512 * 4  # one 512-column block
     assert lib.trakhip_project_workspace(0, 25, 1024, 256) == 0
     assert lib.trakhip_spd_inverse_workspace(4096) >= 3 * 4096 * 4096 * 4
     assert lib.trakhip_spd_inverse_workspace(100) >= 3 * 128 * 128 * 4

@@ -33,18 +33,17 @@ def test_rademacher_uses_every_bit_of_a_block_once(c_oracle):
     # one tile of 128 features: entry j must be a distinct bit of the block's 128 bits
     seed, col = 99, 17
     P = 128
-    words = c_oracle.philox([0, 0, 0, 0], [c_oracle.stream_seed(seed, col, 0), 0])
+    words = c_oracle.philox([0, c_oracle.stream_name(seed, col, 0), 0, 0], [seed, 0])
     col_vals = c_oracle.materialize(seed, 1, P, 0, P, col, 1, R)[:, 0]
-    bits = [(words[w] >> b) & 1 for w in range(4) for b in range(32)]
-    assert sorted((col_vals > 0).astype(int).tolist()) == sorted(bits)
-    # flipping the mapping check: reconstruct each entry from its documented position
+    # entry j is bit j of the block read as one 128-bit little-endian number
+    block = sum(w << (32 * i) for i, w in enumerate(words))
     for j in range(128):
-        q, i = divmod(j, 8)
-        bit = (words[i // 2] >> (15 - q + 16 * (i % 2))) & 1
-        assert col_vals[j] == (1.0 if bit else -1.0)
-    # and the positions are all different
-    pos = {(i // 2, 15 - q + 16 * (i % 2)) for q in range(16) for i in range(8)}
-    assert len(pos) == 128
+        assert col_vals[j] == (1.0 if (block >> j) & 1 else -1.0)
+    # the second block of the stream serves features 128..255
+    words1 = c_oracle.philox([1, c_oracle.stream_name(seed, col, 0), 0, 0], [seed, 0])
+    block1 = sum(w << (32 * i) for i, w in enumerate(words1))
+    col_vals = c_oracle.materialize(seed, 1, 256, 128, 128, col, 1, R)[:, 0]
+    assert [v > 0 for v in col_vals] == [bool((block1 >> j) & 1) for j in range(128)]
 
 
 def test_rademacher_values_and_balance(c_oracle):
@@ -67,9 +66,11 @@ def test_streams_differ_across_tiles_columns_and_seeds(c_oracle):
     assert not np.array_equal(a, b) and not np.array_equal(a, c)
     assert not np.array_equal(a[:, 0], a[:, 1])
     # seed enters additively with the column and tile strides (fast_jl/random.cuh:15-17):
-    # seed + 658105236 at column 0 is the stream of (seed, column 1)
+    # seed + 658105236 at column 0 has the stream name of (seed, column 1), but the seed is also
+    # the generator's key: another projector seed never replays a stream of this one
     d = c_oracle.materialize((1 + 658105236) % 2**32, 256, 1 << 16, 0, 256, 0, 1, R)
-    assert np.array_equal(d[:, 0], a[:, 1])
+    assert c_oracle.stream_name((1 + 658105236) % 2**32, 0, 0) == c_oracle.stream_name(1, 1, 0)
+    assert not np.array_equal(d[:, 0], a[:, 1])
 
 
 @pytest.mark.parametrize("P,expect_odd", [(10_240, False), (10_241, True)])
@@ -163,12 +164,12 @@ def test_normal_entry_is_box_muller_in_fp16(c_oracle):
 def test_normal_block_uses_every_word_for_one_pair(c_oracle):
     # one tile of 8 features = one Philox block: entries (2i, 2i + 1) come from word i
     seed, col = 5, 9
-    words = c_oracle.philox([0, 0, 0, 0], [c_oracle.stream_seed(seed, col, 0), 0])
+    words = c_oracle.philox([0, c_oracle.stream_name(seed, col, 0), 0, 0], [seed, 0])
     colv = c_oracle.materialize(seed, 1, 8, 0, 8, col, 1, G)[:, 0]
     for e in range(8):
         assert colv[e] == c_oracle.normal_from_word(words[e // 2], e % 2)
     # and the second block of the stream serves features 8..15
-    words1 = c_oracle.philox([1, 0, 0, 0], [c_oracle.stream_seed(seed, col, 0), 0])
+    words1 = c_oracle.philox([1, c_oracle.stream_name(seed, col, 0), 0, 0], [seed, 0])
     colv = c_oracle.materialize(seed, 1, 16, 8, 8, col, 1, G)[:, 0]
     for e in range(8):
         assert colv[e] == c_oracle.normal_from_word(words1[e // 2], e % 2)

@@ -45,18 +45,29 @@ def test_philox_is_a_bijection_of_the_counter_low_word(c_oracle):
     assert len({tuple(r) for r in out.tolist()}) == 4096
 
 
-def test_stream_seed_closed_form(c_oracle):
+def test_stream_name_closed_form(c_oracle):
     # fast_jl/random.cuh:15-17: seed + 658105236*column + 359124577*tile, uint32 wrap
     cases = [(0, 0, 0), (42, 1, 0), (42, 0, 1), (7, 4095, 255), (0xFFFFFFFF, 15359, 255), (10**8, 513, 107)]
     for seed, col, tile in cases:
         expect = (seed + 658105236 * col + 359124577 * tile) % 2**32
-        assert c_oracle.stream_seed(seed, col, tile) == expect
-        assert int(npo.stream_seed(seed, col, tile)) == expect
+        assert c_oracle.stream_name(seed, col, tile) == expect
+        assert int(npo.stream_name(seed, col, tile)) == expect
     # hand-computed: 42 + 658105236 = 658105278 ; 42 + 359124577 = 359124619
-    assert c_oracle.stream_seed(42, 1, 0) == 658105278
-    assert c_oracle.stream_seed(42, 0, 1) == 359124619
+    assert c_oracle.stream_name(42, 1, 0) == 658105278
+    assert c_oracle.stream_name(42, 0, 1) == 359124619
     # wrap: 658105236 * 7 = 4606736652 -> mod 2^32 = 311769356
-    assert c_oracle.stream_seed(0, 7, 0) == 311769356
+    assert c_oracle.stream_name(0, 7, 0) == 311769356
+
+
+def test_stream_block_is_philox_with_the_name_in_the_counter(c_oracle):
+    # block n of the stream named s under a projector seed: counter (n, s, 0, 0), key (seed, 0)
+    for seed, name, n in [(0, 0, 0), (42, 658105278, 3), (0xFFFFFFFF, 0x12345678, 0xFFFFFFFF)]:
+        want = c_oracle.philox([n, name, 0, 0], [seed, 0])
+        assert c_oracle.stream_block(seed, name, n) == want
+        assert npo.stream_blocks(seed, name, n).tolist() == want
+    # Random123's known-answer vector with zero counter and key, read as block 0 of stream 0 of
+    # seed 0 (the other published vectors have counter and key words this entry point keeps zero)
+    assert c_oracle.stream_block(0, 0, 0) == [0x6627E8D5, 0xE169C58D, 0xBC57AC4C, 0x9B00DBD8]
 
 
 def test_tiling_matches_reference_iteration_counts(c_oracle):

@@ -7,24 +7,24 @@
 // What is kept from the reference kernel (fast_jl):
 //   * the feature axis is cut into T = min(P, num_feature_tiles) tiles of
 //     fts = ceil(P / T) features (fast_jl/fast_jl.cu:42, fast_jl/fast_jl_kernel.cuh:124);
-//   * every (JL column c, feature tile t) pair owns one random stream whose
-//     32-bit seed is  seed + 658105236*c + 359124577*t  with uint32 wrap-around
-//     (fast_jl/random.cuh:15-17);
+//   * every (JL column c, feature tile t) pair owns one random stream, named by the 32-bit
+//     value  seed + 658105236*c + 359124577*t  with uint32 wrap-around
+//     (fast_jl/random.cuh:15-17, where it seeds the pair's generator);
 //   * entries are consumed in feature order inside a tile; a Rademacher entry
 //     costs one random bit, bit set -> +1 (fast_jl/random.cuh:33-37); a normal
 //     entry is a Box-Muller normal in fp16 (fast_jl/random.cuh:50-60).
 //
 // What is new: the generator is Philox4x32-10 (the reference uses cuRAND XORWOW,
-// whose draws cannot be reproduced off an NVIDIA toolchain).  The stream of
-// (c, t) is the block sequence
-//       block(n) = Philox4x32-10(counter = (n, 0, 0, 0), key = (stream_seed, 0))
-// i.e. what curand_init(stream_seed, 0, 0) would address with a Philox state.
+// whose draws cannot be reproduced off an NVIDIA toolchain).  The stream named s of a
+// projector with seed `seed` is the block sequence
+//       block(n) = Philox4x32-10(counter = (n, s, 0, 0), key = (seed, 0)).
+// The stream's name sits in the counter and not in the key so that the ten round keys are the
+// same for every lane of a kernel (scalar operands, no per-lane key schedule).
 //
-// Rademacher: feature offset o inside the tile uses block n = o / 128.  With
-//   j = o % 128, q = j / 8, i = j % 8  the entry is bit (15 - q + 16*(i & 1)) of
-//   word (i >> 1) of that block.  This places the 8 entries a lane feeds to one
-//   32x32x16 MFMA in bit 15 / bit 31 of (word << q), which is where the sign
-//   bits of a packed pair of 16-bit floats live.
+// Rademacher: feature offset o inside the tile uses block n = o / 128, and the entry is bit
+//   o % 128 of the block read as a 128-bit little-endian number (bit j % 32 of word j / 32).
+//   The 8 entries a lane feeds to one 32x32x16 MFMA (offsets 8q .. 8q + 7) are byte q of the
+//   block: the kernel looks the eight signs up in a 256-entry table.
 //
 // Normal: feature offset o uses block n = o / 8; word (o % 8) / 2 of the block makes the
 //   Box-Muller pair of entries o % 8 = 2i (cosine) and 2i + 1 (sine):
@@ -60,7 +60,8 @@ struct u32x4 {
     uint32_t x, y, z, w;
 };
 
-JL_HD uint32_t stream_seed(uint32_t seed, uint32_t column, uint32_t tile) {
+// Name of the stream of (column, tile).
+JL_HD uint32_t stream_name(uint32_t seed, uint32_t column, uint32_t tile) {
     return seed + kColumnStride * column + kTileStride * tile;
 }
 
@@ -91,10 +92,10 @@ JL_HD u32x4 philox4x32_10(u32x4 c, uint32_t k0, uint32_t k1) {
     return c;
 }
 
-// Block n of the stream with seed s: counter (n, 0, 0, 0), key (s, 0).
-JL_HD u32x4 stream_block(uint32_t s, uint32_t n) {
-    u32x4 c = {n, 0u, 0u, 0u};
-    return philox4x32_10(c, s, 0u);
+// Block n of the stream named s: counter (n, s, 0, 0), key (seed, 0).
+JL_HD u32x4 stream_block(uint32_t seed, uint32_t s, uint32_t n) {
+    u32x4 c = {n, s, 0u, 0u};
+    return philox4x32_10(c, seed, 0u);
 }
 
 JL_HD uint32_t word_of(const u32x4& b, uint32_t i) {
@@ -103,8 +104,7 @@ JL_HD uint32_t word_of(const u32x4& b, uint32_t i) {
 
 // Rademacher entry for offset j (0..127) inside a 128-entry block: 1 -> +1, 0 -> -1.
 JL_HD uint32_t rademacher_bit(const u32x4& b, uint32_t j) {
-    const uint32_t q = j >> 3, i = j & 7u;
-    return (word_of(b, i >> 1) >> (15u - q + 16u * (i & 1u))) & 1u;
+    return (word_of(b, j >> 5) >> (j & 31u)) & 1u;
 }
 
 // ---- Box-Muller in explicit binary32 arithmetic -------------------------------------------
@@ -252,8 +252,8 @@ JL_HD float f16_bits_to_f32(uint16_t hbits) {
 
 // o = feature offset inside the tile.  Returns the value as binary32 (always exactly
 // representable in fp16).
-JL_HD float entry_rademacher(uint32_t sseed, uint32_t o) {
-    const u32x4 b = stream_block(sseed, o >> 7);
+JL_HD float entry_rademacher(uint32_t seed, uint32_t column, uint32_t tile, uint32_t o) {
+    const u32x4 b = stream_block(seed, stream_name(seed, column, tile), o >> 7);
     return rademacher_bit(b, o & 127u) ? 1.0f : -1.0f;
 }
 
@@ -273,8 +273,8 @@ JL_HD uint16_t f16_mul_rne(uint16_t a, uint16_t b) {
 #endif
 }
 
-JL_HD uint16_t entry_normal_f16bits(uint32_t sseed, uint32_t o) {
-    const u32x4 b = stream_block(sseed, o >> 3);
+JL_HD uint16_t entry_normal_f16bits(uint32_t seed, uint32_t column, uint32_t tile, uint32_t o) {
+    const u32x4 b = stream_block(seed, stream_name(seed, column, tile), o >> 3);
     const uint32_t e = o & 7u;
     const uint32_t w = word_of(b, e >> 1);
     const uint16_t r = f32_to_f16_rne(bm_radius(normal_radius_index(w)));
@@ -285,8 +285,8 @@ JL_HD uint16_t entry_normal_f16bits(uint32_t sseed, uint32_t o) {
     return (uint16_t)(f16_mul_rne(r, t) ^ sign);
 }
 
-JL_HD float entry_normal(uint32_t sseed, uint32_t o) {
-    return f16_bits_to_f32(entry_normal_f16bits(sseed, o));
+JL_HD float entry_normal(uint32_t seed, uint32_t column, uint32_t tile, uint32_t o) {
+    return f16_bits_to_f32(entry_normal_f16bits(seed, column, tile, o));
 }
 
 // Tiling of the feature axis (fast_jl/fast_jl.cu:42, fast_jl/fast_jl_kernel.cuh:124).

@@ -8,18 +8,18 @@
 // the workgroup staged in LDS.
 //
 // Work decomposition
-//   workgroup = 8 waves = 1024 JL columns (4 waves = 512 columns when the
-//               projection dimension is an odd multiple of 512) x a run of
-//               consecutive 256-feature chunks of the reference's feature
-//               tiles (fts = ceil(P / T) consecutive features each);
-//   wave      = 4 groups of 32 columns (four 32x32 fp32 accumulators);
+//   workgroup = 8 waves = 1024 JL columns (512 columns when the projection
+//               dimension is an odd multiple of 512) x a run of consecutive
+//               256-feature chunks of the reference's feature tiles
+//               (fts = ceil(P / T) consecutive features each);
+//   wave      = 4 (or 2) groups of 32 columns, one 32x32 fp32 accumulator each;
 //   lane      = (n = lane % 32, h = lane / 32): column n of each group, and the
 //               k-slots 8h..8h+7 of every MFMA.
 // The tile is walked in chunks of 256 features.  Lane half h owns features
 // [128h, 128h+128) of a chunk: MFMA number q (0..15) of the chunk contracts
-// features 128h + 8q + i (i = 0..7), so the 8 sign bits a lane needs for it sit
-// in bits 15/31 of (word_v << q), v = 0..3, of ONE Philox block per column per
-// chunk, and the A operand is 16 contiguous bytes of a gradient row.
+// features 128h + 8q + i (i = 0..7), so the 8 Rademacher signs a lane needs for it
+// are byte q of ONE Philox block per column per chunk, and the A operand is 16
+// contiguous bytes of a gradient row.
 //
 // A workgroup walks a run of consecutive chunks (across tile boundaries, adding the
 // products up in its accumulators) and writes one partial [B, 1024] block; a second
@@ -41,11 +41,8 @@ typedef _Float16 half8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 
-// A workgroup has W = 4 or 8 waves and covers 128 W columns: eight waves (one workgroup per CU) stage
-// every gradient chunk once per 1024 columns instead of once per 512, which halves the L2 -> LDS
-// traffic (3.6 % faster at the benchmark shape); four waves serve projection dimensions that are
-// an odd multiple of 512.
-constexpr int kGroups = 4;                            // 32-column groups per wave
+// A workgroup has 8 waves (one workgroup per CU, two waves per SIMD) and stages every gradient
+// chunk once for all its columns.
 constexpr int kColsMultiple = 512;                    // proj dim granularity (fast_jl_kernel.cuh:113)
 constexpr int kPieces = 32 * 32;                      // 16-byte pieces of a [32 x 256] chunk of 16-bit values
 constexpr int kChunk = 256;                           // features per staged chunk
@@ -359,14 +356,7 @@ struct StageOf<TRAKHIP_F32, true, W> {
     typedef trakhip_segment elem;
 };
 
-// ---- B operand generation --------------------------------------------------------------------
-
-// Packed pair of +-1 from bits 15 and 31 of m (bit set -> +1), every other bit of m ignored:
-// (m & one) | (~m & (one | 0x80008000)) as ONE v_bitop3_b32 (truth table 0xCA = a ? b : c).
-// one = 0x3C003C00 (fp16) or 0x3F803F80 (bf16).
-__device__ __forceinline__ uint32_t sign_pair(uint32_t m, uint32_t one) {
-    return __builtin_amdgcn_bitop3_b32(m, one, one | 0x80008000u, 0xCA);
-}
+// ---- Rademacher projection -------------------------------------------------------------------
 
 // Workgroup id -> (column block, tile).  Workgroups are handed to the 8 XCDs round-robin
 // by linear id; this puts the column blocks of one feature tile on the same XCD, next to
@@ -379,51 +369,82 @@ __device__ __forceinline__ void map_workgroup(uint32_t linear, uint32_t col_bloc
     tile = (idx / col_blocks) * 8u + xcd;
 }
 
-// Rademacher B operand of MFMA number q of the chunk for one column group, in two halves so the
-// caller can put the MFMA of the previous step between them:
-//   shifted_pairs: both word pairs shifted left by q, one full-rate v_lshlrev_b64 each (for a
-//     constant count the compiler would emit two 32-bit instructions per pair); bits crossing into
-//     the high word stay below bit 15, which sign_pair ignores;
-//   signs_of: one v_bitop3 per operand register.
-__device__ __forceinline__ void shifted_pairs(uint64_t w01, uint64_t w23, int q, uint64_t& m01, uint64_t& m23) {
-    m01 = w01;
-    m23 = w23;
-    if (q) {
-        // a shift count the compiler cannot see through keeps the 64-bit shift one instruction
-        int qq = q;
-        asm("" : "+s"(qq));
-        m01 = w01 << qq;
-        m23 = w23 << qq;
-    }
+// The B operand of one MFMA is eight signs = one byte of a Philox block, looked up in LDS:
+// entry e of the table holds the packed 16-bit values (bit i of e set -> +1, clear -> -1) for
+// i = 0..7.  There are sixteen copies of every entry, (e * 16 + copy) * 16 bytes from the start
+// of LDS, and a lane reads copy lane % 16: the sixteen lanes that the LDS serves in one cycle of a
+// 16-byte read then hit all 64 banks whatever their bytes are.
+constexpr int kSignCopies = 16;
+constexpr int kSignTableBytes = 256 * kSignCopies * 16;  // 64 KB
+
+// Address of the table entry for byte q % 4 of `word`: one v_perm_b32 puts the byte into bits
+// 8..15 over lane_base = (lane % 16) * 16.
+__device__ __forceinline__ uint32_t sign_entry_address(uint32_t word, int q, uint32_t lane_base) {
+    const uint32_t sel = 0x0C0C0000u | ((4u + (uint32_t)(q & 3)) << 8);  // {0, 0, word.byte[q % 4], lane_base.byte[0]}
+    return __builtin_amdgcn_perm(word, lane_base, sel);
 }
-__device__ __forceinline__ uint4 signs_of(uint64_t m01, uint64_t m23, uint32_t one) {
-    uint4 b;
-    b.x = sign_pair((uint32_t)m01, one);
-    b.y = sign_pair((uint32_t)(m01 >> 32), one);
-    b.z = sign_pair((uint32_t)m23, one);
-    b.w = sign_pair((uint32_t)(m23 >> 32), one);
-    return b;
+
+// Half of a Philox round on one column group's state: half 0 is the multiply of c.x (gives z, w
+// of the next state), half 1 the multiply of c.z (gives x, y).  The empty asm statements tie the
+// instructions to the place in the instruction stream where the call stands: without them the
+// compiler moves all the generator arithmetic of a chunk in front of its first MFMA.
+__device__ __forceinline__ void philox_half(const jl::u32x4& c, jl::u32x4& next, int half, uint32_t k0, uint32_t k1) {
+    if (half == 0) {
+        uint32_t x = c.x, w = c.w;
+        asm volatile("" : "+v"(x), "+v"(w));
+        const uint64_t p0 = (uint64_t)jl::kPhiloxM0 * x;
+        next.z = jl::xor3((uint32_t)(p0 >> 32), w, k1);
+        next.w = (uint32_t)p0;
+        asm volatile("" : "+v"(next.z), "+v"(next.w));
+    } else {
+        uint32_t z = c.z, y = c.y;
+        asm volatile("" : "+v"(z), "+v"(y));
+        const uint64_t p1 = (uint64_t)jl::kPhiloxM1 * z;
+        next.x = jl::xor3((uint32_t)(p1 >> 32), y, k0);
+        next.y = (uint32_t)p1;
+        asm volatile("" : "+v"(next.x), "+v"(next.y));
+    }
 }
 
 // GATHER: g_in is a device array of trakhip_segment and ld their number; otherwise g_in is the
-// dense [rows, P] matrix with row pitch ld.
-template <int IN, bool GATHER, int W>
-__global__ __launch_bounds__(64 * W, 2) void jl_project_kernel(
+// dense [rows, P] matrix with row pitch ld.  GPW = 32-column groups per wave: 4 (workgroup = 1024
+// columns) or 2 (512 columns, for projection dimensions that are an odd multiple of 512).
+//
+// The main loop is written out step by step.  A chunk is 16 * GPW steps (q, j): one table lookup
+// and one MFMA (three for fp32 gradients) for column group j and features 8q..8q+7 of the lane's
+// half of the chunk.  Under them runs the generator for the NEXT chunk, one half round or two per
+// step (nine rounds x GPW groups x two halves spread over the steps; the first round has scalar
+// operands and is done at the top of the chunk), and the operand reads run kAhead steps ahead of
+// the MFMA that uses them.  The matrix pipe stays busy only if the vector instructions between two
+// MFMAs of a wave fit into the time of one MFMA of each of the two waves of the SIMD (8 issue
+// slots of 4 cycles each, two of them for a 64-bit multiply), which is why the generator is cut
+// that fine.
+template <int IN, bool GATHER, int GPW>
+__global__ __launch_bounds__(512) void jl_project_kernel(
     const void* __restrict__ g_in, uint64_t ld, uint32_t rows, uint64_t P, uint32_t k,
     uint32_t seed, uint32_t tiles, uint64_t tile_size, uint32_t chunks_per_tile,
     uint32_t chunks_per_group, float* __restrict__ partial) {
+    constexpr int W = 8;
     typedef InTraits<IN> Tr;
     typedef typename StageOf<IN, GATHER, W>::type Stage;
     typedef typename StageOf<IN, GATHER, W>::elem Elem;
-    constexpr int kColsPerWG = W * kGroups * 32;
+    constexpr int kColsPerWG = W * GPW * 32;
     constexpr bool kBf = Tr::bf16;
     constexpr int kPlanes = Tr::planes;
     // 16-bit inputs: two LDS buffers, one barrier per chunk.  fp32 inputs (three planes) keep one
-    // buffer and two barriers so that two workgroups still fit on a CU.
+    // buffer and two barriers: two buffers of three planes do not fit next to the table.
     constexpr int kBuffers = kPlanes == 1 ? 2 : 1;
     constexpr int kBufElems = kPlanes * kPlaneElems;
+    constexpr int kSteps = 16 * GPW;
+    constexpr int kAhead = 3;                       // operand reads in flight
+    constexpr int kHalfRounds = 9 * GPW * 2;        // rounds 1..9 of the next chunk's blocks
+    static_assert(kSteps % (kAhead + 1) == 0, "the operand ring must close over a chunk");
+    static_assert(kHalfRounds >= kSteps && kHalfRounds <= 2 * kSteps, "one or two half rounds per step");
 
-    __shared__ __attribute__((aligned(16))) uint16_t lds[kBuffers * kBufElems];
+    // the table comes first: a DS instruction adds a 16-bit immediate to the address register, and
+    // a table entry's address is built without adding a base
+    __shared__ __attribute__((aligned(256))) char smem[kSignTableBytes + kBuffers * kBufElems * 2];
+    uint16_t* lds = reinterpret_cast<uint16_t*>(smem + kSignTableBytes);
 
     const uint32_t col_blocks = k / kColsPerWG;
     uint32_t cb, group;
@@ -441,17 +462,29 @@ __global__ __launch_bounds__(64 * W, 2) void jl_project_kernel(
     const int tid = threadIdx.x;
     const int wave = tid >> 6, lane = tid & 63;
     const uint32_t n = lane & 31, h = lane >> 5;
-    const uint32_t col0 = cb * kColsPerWG + wave * (kGroups * 32) + n;
+    const uint32_t col0 = cb * kColsPerWG + wave * (GPW * 32) + n;
 
-    floatx16 acc[kGroups];
+    {
+        const uint32_t plus = kBf ? 0x3F80u : 0x3C00u;
+        for (int idx = tid; idx < 256 * kSignCopies; idx += 64 * W) {
+            const uint32_t e = (uint32_t)idx / kSignCopies;
+            uint32_t v[8];
 #pragma unroll
-    for (int j = 0; j < kGroups; ++j)
+            for (int i = 0; i < 8; ++i) v[i] = plus | (((e >> i) & 1u) ? 0u : 0x8000u);
+            *reinterpret_cast<uint4*>(smem + idx * 16) =
+                uint4{v[0] | (v[1] << 16), v[2] | (v[3] << 16), v[4] | (v[5] << 16), v[6] | (v[7] << 16)};
+        }
+    }
+
+    floatx16 acc[GPW];
+#pragma unroll
+    for (int j = 0; j < GPW; ++j)
 #pragma unroll
         for (int r = 0; r < 16; ++r) acc[j][r] = 0.0f;
 
     const Elem* g = reinterpret_cast<const Elem*>(g_in);
-    const uint32_t one = kBf ? 0x3F803F80u : 0x3C003C00u;
     const uint32_t a_off = n * kLdsRow + 128 * h;
+    const uint32_t lane_base = (uint32_t)(lane & 15) << 4;
 
     Stage st;
     {
@@ -461,9 +494,15 @@ __global__ __launch_bounds__(64 * W, 2) void jl_project_kernel(
         st.load(g, ld, rows, lo + (uint64_t)s0 * kChunk, hi, tid);
     }
     int cur = 0;
-    if (kBuffers == 2) {
-        st.store(lds, tid);
-        __syncthreads();
+    if (kBuffers == 2) st.store(lds, tid);
+    __syncthreads();  // publishes the table (and the first chunk)
+
+    // the first two words of a block are bytes 0..7 = MFMA steps q = 0..7, the other two q = 8..15
+    uint32_t wd[GPW][4];
+#pragma unroll
+    for (int j = 0; j < GPW; ++j) {
+        const jl::u32x4 w = jl::stream_block(seed, jl::stream_name(seed, col0 + 32u * j, t0), 2u * s0 + h);
+        wd[j][0] = w.x, wd[j][1] = w.y, wd[j][2] = w.z, wd[j][3] = w.w;
     }
 
     for (uint32_t tile = t0; tile <= t_last; ++tile) {
@@ -473,10 +512,6 @@ __global__ __launch_bounds__(64 * W, 2) void jl_project_kernel(
         const uint32_t chunks = tile == t_last ? s_last_end : chunks_per_tile;
         const uint64_t nf_lo = f_lo + tile_size;                               // next tile
         const uint64_t nf_hi = (nf_lo + tile_size < P) ? nf_lo + tile_size : P;
-
-        uint32_t sseed[kGroups];
-#pragma unroll
-        for (int j = 0; j < kGroups; ++j) sseed[j] = jl::stream_seed(seed, col0 + 32u * j, tile);
 
         for (uint32_t s = s_begin; s < chunks; ++s) {
             const bool more_here = s + 1 < chunks;
@@ -491,19 +526,31 @@ __global__ __launch_bounds__(64 * W, 2) void jl_project_kernel(
                         tid);
             const uint16_t* a_base = lds + cur * kBufElems + a_off;
 
-            uint64_t w01[kGroups], w23[kGroups];
+            // The next chunk's blocks (of the next tile when this one ends here): first round now -
+            // its counter is (block, stream name, 0, 0) and the block number is the same for the
+            // GPW groups, so it is one multiply for all of them and one xor per group - the other
+            // nine under the MFMAs below.
+            jl::u32x4 pc[GPW], pn[GPW];
+            {
+                const uint32_t nblk = more_here ? 2u * (s + 1) + h : h;
+                const uint32_t ntile = more_here ? tile : tile + 1u;
+                const uint64_t p0 = (uint64_t)jl::kPhiloxM0 * nblk;
 #pragma unroll
-            for (int j = 0; j < kGroups; ++j) {
-                const jl::u32x4 w = jl::stream_block(sseed[j], 2u * s + h);
-                w01[j] = ((uint64_t)w.y << 32) | w.x;
-                w23[j] = ((uint64_t)w.w << 32) | w.z;
+                for (int j = 0; j < GPW; ++j) {
+                    pc[j].x = jl::stream_name(seed, col0 + 32u * j, ntile) ^ seed;
+                    pc[j].y = 0u;
+                    pc[j].z = (uint32_t)(p0 >> 32);
+                    pc[j].w = (uint32_t)p0;
+                }
             }
-            // 64 steps (q, j).  Issue order per step: shifts of the NEXT operand, MFMA of this
-            // step, sign expansion of the next operand.  The MFMA then never directly follows
-            // the VALU instructions that wrote its operand (no wait states to pad).
-            uint64_t m01, m23;
-            shifted_pairs(w01[0], w23[0], 0, m01, m23);
-            uint4 b = signs_of(m01, m23, one);
+
+            auto operand = [&](int step) -> uint4 {
+                const int q = step / GPW, j = step % GPW;
+                return *reinterpret_cast<const uint4*>(smem + sign_entry_address(wd[j][q >> 2], q, lane_base));
+            };
+            uint4 bq[kAhead + 1];
+#pragma unroll
+            for (int p = 0; p < kAhead; ++p) bq[p] = operand(p);
             uint4 a[2][kPlanes];  // A operands of this q and of the next one (read one q ahead)
 #pragma unroll
             for (int pl = 0; pl < kPlanes; ++pl)
@@ -511,25 +558,41 @@ __global__ __launch_bounds__(64 * W, 2) void jl_project_kernel(
 #pragma unroll
             for (int q = 0; q < 16; ++q) {
 #pragma unroll
-                for (int j = 0; j < kGroups; ++j) {
-                    const int step = q * kGroups + j;
-                    const bool last = step + 1 == 16 * kGroups;
-                    if (!last) shifted_pairs(w01[(step + 1) % kGroups], w23[(step + 1) % kGroups],
-                                             (step + 1) / kGroups, m01, m23);
+                for (int j = 0; j < GPW; ++j) {
+                    const int step = q * GPW + j;
+                    if (step + kAhead < kSteps) bq[(step + kAhead) % (kAhead + 1)] = operand(step + kAhead);
                     if (j == 0 && q + 1 < 16) {
 #pragma unroll
                         for (int pl = 0; pl < kPlanes; ++pl)
                             a[(q + 1) & 1][pl] =
                                 *reinterpret_cast<const uint4*>(a_base + pl * kPlaneElems + 8 * (q + 1));
                     }
+                    // half rounds number first .. first + count - 1 of the kHalfRounds; number
+                    // i is half i % 2 of round 1 + i / (2 GPW) of group (i / 2) % GPW.  Every
+                    // kSteps / extra-th step takes two.
+                    {
+                        constexpr int kExtra = kHalfRounds - kSteps;       // steps that take two
+                        constexpr int kEvery = kSteps / kExtra;
+                        const int twos_before = (step + kEvery - 1) / kEvery;  // steps < step that took two
+                        const int first = step + (twos_before < kExtra ? twos_before : kExtra);
+                        const int count = (step % kEvery == 0 && step / kEvery < kExtra) ? 2 : 1;
+#pragma unroll
+                        for (int i = first; i < first + count; ++i) {
+                            const int r = 1 + i / (2 * GPW), g4 = (i / 2) % GPW, half = i % 2;
+                            philox_half(pc[g4], pn[g4], half, seed + (uint32_t)r * jl::kPhiloxW0,
+                                        (uint32_t)r * jl::kPhiloxW1);
+                            if (half == 1) pc[g4] = pn[g4];
+                        }
+                    }
                     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-                    for (int pl = 0; pl < kPlanes; ++pl) acc[j] = mfma16(a[q & 1][pl], b, acc[j], kBf);
-                    __builtin_amdgcn_sched_barrier(0);
-                    if (!last) b = signs_of(m01, m23, one);
+                    for (int pl = 0; pl < kPlanes; ++pl)
+                        acc[j] = mfma16(a[q & 1][pl], bq[step % (kAhead + 1)], acc[j], kBf);
                     __builtin_amdgcn_sched_barrier(0);
                 }
             }
+#pragma unroll
+            for (int j = 0; j < GPW; ++j) wd[j][0] = pc[j].x, wd[j][1] = pc[j].y, wd[j][2] = pc[j].z, wd[j][3] = pc[j].w;
 
             if (kBuffers == 2) {
                 // the other buffer was last read in the previous iteration, before its barrier
@@ -544,7 +607,7 @@ __global__ __launch_bounds__(64 * W, 2) void jl_project_kernel(
     // m = 8*(r/4) + 4*(lane/32) + r%4.
     float* out = partial + (uint64_t)group * rows * k;
 #pragma unroll
-    for (int j = 0; j < kGroups; ++j) {
+    for (int j = 0; j < GPW; ++j) {
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
             const uint32_t m = 8u * (r >> 2) + 4u * h + (r & 3);
@@ -808,9 +871,9 @@ __global__ __launch_bounds__(512, 2) void jl_project_normal_kernel(
         const uint64_t nf_lo = f_lo + tile_size;
         const uint64_t nf_hi = (nf_lo + tile_size < P) ? nf_lo + tile_size : P;
 
-        uint32_t sseed[GPW];
+        uint32_t sname[GPW];
 #pragma unroll
-        for (int j = 0; j < GPW; ++j) sseed[j] = jl::stream_seed(seed, col0 + 32u * j, tile);
+        for (int j = 0; j < GPW; ++j) sname[j] = jl::stream_name(seed, col0 + 32u * j, tile);
 
         for (uint32_t s = s_begin; s < chunks; ++s) {
             const bool more_here = s + 1 < chunks;
@@ -850,7 +913,7 @@ __global__ __launch_bounds__(512, 2) void jl_project_normal_kernel(
                     a[pl] = *reinterpret_cast<const uint4*>(a_base + pl * kPlaneElems + 8 * q);
 #pragma unroll
                 for (int j = 0; j < GPW; ++j) {
-                    const jl::u32x4 blk = jl::stream_block(sseed[j], n0 + (uint32_t)q);
+                    const jl::u32x4 blk = jl::stream_block(seed, sname[j], n0 + (uint32_t)q);
                     const uint4 b = {normal_pair(blk.x, rt, ct), normal_pair(blk.y, rt, ct),
                                      normal_pair(blk.z, rt, ct), normal_pair(blk.w, rt, ct)};
 #pragma unroll
@@ -953,28 +1016,28 @@ __global__ __launch_bounds__(256) void jl_materialize_kernel(uint32_t seed, uint
     const uint32_t c = c0 + (uint32_t)(idx % nc);
     const uint32_t tile = (uint32_t)(f / tile_size);
     const uint32_t o = (uint32_t)(f % tile_size);
-    const uint32_t ss = jl::stream_seed(seed, c, tile);
-    out[idx] = proj_type == TRAKHIP_RADEMACHER ? jl::entry_rademacher(ss, o) : jl::entry_normal(ss, o);
+    out[idx] = proj_type == TRAKHIP_RADEMACHER ? jl::entry_rademacher(seed, c, tile, o)
+                                               : jl::entry_normal(seed, c, tile, o);
 }
 
 // How a launch is cut into workgroups.  The (tile, chunk) pairs of all feature tiles form one
 // sequence of tiles * chunks_per_tile chunks; every workgroup takes chunks_per_group consecutive
-// ones (adding their products in its accumulators) for one block of 128 * waves columns.  The split
-// depends only on the shape, so results are reproducible; it aims at 2048 resident waves (two per
-// SIMD).
+// ones (adding their products in its accumulators) for one block of 1024 columns (512 when the
+// projection dimension is an odd multiple of 512).  The split depends only on the shape, so results
+// are reproducible; it aims at one workgroup of 8 waves per CU.
 struct Plan {
     jl::Tiling tl;
-    uint32_t waves, col_blocks, chunks_per_tile, chunks_per_group, groups;
+    uint32_t gpw, col_blocks, chunks_per_tile, chunks_per_group, groups;  // gpw: 32-column groups per wave
 };
 
 Plan make_plan(uint64_t P, uint32_t k, uint32_t num_feature_tiles) {
     Plan p;
     p.tl = jl::make_tiling(P, num_feature_tiles);
-    p.waves = (k % (8 * kGroups * 32) == 0) ? 8 : 4;
-    p.col_blocks = k / (p.waves * kGroups * 32);
+    p.gpw = (k % (8 * 4 * 32) == 0) ? 4 : 2;
+    p.col_blocks = k / (8 * p.gpw * 32);
     p.chunks_per_tile = (uint32_t)((p.tl.tile_size + kChunk - 1) / kChunk);
     const uint64_t total = (uint64_t)p.tl.tiles * p.chunks_per_tile;
-    const uint64_t target_wgs = 2048 / p.waves;  // 256 CUs x 8 waves
+    const uint64_t target_wgs = 256;  // one workgroup of 8 waves per CU
     uint64_t groups = (target_wgs + p.col_blocks - 1) / p.col_blocks;
     if (groups > total) groups = total;
     if (groups < 1) groups = 1;
@@ -983,25 +1046,24 @@ Plan make_plan(uint64_t P, uint32_t k, uint32_t num_feature_tiles) {
     return p;
 }
 
-template <int IN, bool GATHER, int W>
+template <int IN, bool GATHER, int GPW>
 hipError_t launch_rademacher(const void* in, uint64_t ld, uint32_t rows, uint64_t P, uint32_t k, uint32_t seed,
                              const Plan& pl, float* partial, hipStream_t s) {
     const uint32_t groups8 = (pl.groups + 7u) / 8u * 8u;
     const uint64_t wgs = (uint64_t)groups8 * pl.col_blocks;
     if (wgs > 0x7FFFFFFFull) return hipErrorInvalidValue;
-    hipLaunchKernelGGL((jl_project_kernel<IN, GATHER, W>), dim3((uint32_t)wgs), dim3(64 * W), 0, s, in, ld, rows, P,
+    hipLaunchKernelGGL((jl_project_kernel<IN, GATHER, GPW>), dim3((uint32_t)wgs), dim3(512), 0, s, in, ld, rows, P,
                        k, seed, pl.tl.tiles, pl.tl.tile_size, pl.chunks_per_tile, pl.chunks_per_group, partial);
     return hipGetLastError();
 }
 
-// W (the plan's waves per 128 columns) selects the column groups per wave; the kernel has 8 waves
-template <int IN, bool GATHER, int W>
+template <int IN, bool GATHER, int GPW>
 hipError_t launch_normal(const void* in, uint64_t ld, uint32_t rows, uint64_t P, uint32_t k, uint32_t seed,
                          const Plan& pl, float* partial, hipStream_t s) {
     const uint32_t groups8 = (pl.groups + 7u) / 8u * 8u;
     const uint64_t wgs = (uint64_t)groups8 * pl.col_blocks;
     if (wgs > 0x7FFFFFFFull) return hipErrorInvalidValue;
-    hipLaunchKernelGGL((jl_project_normal_kernel<IN, GATHER, W / 2>), dim3((uint32_t)wgs), dim3(512), 0, s, in, ld,
+    hipLaunchKernelGGL((jl_project_normal_kernel<IN, GATHER, GPW>), dim3((uint32_t)wgs), dim3(512), 0, s, in, ld,
                        rows, P, k, seed, pl.tl.tiles, pl.tl.tile_size, pl.chunks_per_tile, pl.chunks_per_group,
                        partial);
     return hipGetLastError();
@@ -1010,7 +1072,7 @@ hipError_t launch_normal(const void* in, uint64_t ld, uint32_t rows, uint64_t P,
 typedef hipError_t (*LaunchFn)(const void*, uint64_t, uint32_t, uint64_t, uint32_t, uint32_t,
                                const Plan&, float*, hipStream_t);
 
-template <int W>
+template <int W>  // 32-column groups per wave
 LaunchFn pick_w(int dtype, int proj_type, bool gather) {
     static const LaunchFn table[2][3][2] = {
         {{launch_rademacher<TRAKHIP_F16, false, W>, launch_normal<TRAKHIP_F16, false, W>},
@@ -1024,7 +1086,7 @@ LaunchFn pick_w(int dtype, int proj_type, bool gather) {
 }
 
 LaunchFn pick(const Plan& pl, int dtype, int proj_type, bool gather) {
-    return pl.waves == 8 ? pick_w<8>(dtype, proj_type, gather) : pick_w<4>(dtype, proj_type, gather);
+    return pl.gpw == 4 ? pick_w<4>(dtype, proj_type, gather) : pick_w<2>(dtype, proj_type, gather);
 }
 
 }  // namespace
@@ -1203,9 +1265,8 @@ int materialize_host(uint32_t seed, uint32_t num_feature_tiles, uint64_t P, uint
         const uint64_t f = f0 + i;
         const uint32_t tile = (uint32_t)(f / tl.tile_size), o = (uint32_t)(f % tl.tile_size);
         for (uint32_t j = 0; j < nc; ++j) {
-            const uint32_t ss = jl::stream_seed(seed, c0 + j, tile);
-            out[i * nc + j] =
-                proj_type == TRAKHIP_RADEMACHER ? jl::entry_rademacher(ss, o) : jl::entry_normal(ss, o);
+            out[i * nc + j] = proj_type == TRAKHIP_RADEMACHER ? jl::entry_rademacher(seed, c0 + j, tile, o)
+                                                              : jl::entry_normal(seed, c0 + j, tile, o);
         }
     }
     return TRAKHIP_OK;
