@@ -486,15 +486,44 @@ __global__ __launch_bounds__(512) void jl_project_kernel(
     const uint32_t a_off = n * kLdsRow + 128 * h;
     const uint32_t lane_base = (uint32_t)(lane & 15) << 4;
 
-    Stage st;
-    {
-        const uint64_t lo = (uint64_t)t0 * tile_size;
-        const uint64_t hi = (lo + tile_size < P) ? lo + tile_size : P;
-        if constexpr (GATHER) st.init(g, (uint32_t)ld, lo + (uint64_t)s0 * kChunk, P, tid);
-        st.load(g, ld, rows, lo + (uint64_t)s0 * kChunk, hi, tid);
+    // Position (tile, chunk in tile) of a chunk of the run, and its feature range.
+    struct Pos {
+        uint32_t tile, s;
+    };
+    auto step_pos = [&](Pos& p) {
+        if (++p.s == chunks_per_tile) {
+            p.s = 0;
+            ++p.tile;
+        }
+    };
+    auto load_chunk = [&](Stage& st, const Pos& p) {
+        const uint64_t lo = (uint64_t)p.tile * tile_size;
+        const uint64_t hi = (lo + tile_size < P) ? lo + tile_size : P;  // may be <= lo (loads give zeros)
+        st.load(g, ld, rows, lo + (uint64_t)p.s * kChunk, hi, tid);
+    };
+    const uint32_t n_chunks = (uint32_t)(c_end - c_begin);
+    Pos p0 = {t0, s0}, p1 = p0;
+    step_pos(p1);
+    Pos p2 = p1;
+    step_pos(p2);
+
+    // Two sets of staging registers take turns: with two LDS buffers the loads of chunk i + 2 are
+    // issued at the top of chunk i and stored to LDS at the end of chunk i + 1, so a load has two
+    // chunk times (about 6 us) to arrive before a wave has to wait for it at the barrier.
+    Stage st_a, st_b;
+    if constexpr (GATHER) {
+        const uint64_t first = (uint64_t)t0 * tile_size + (uint64_t)s0 * kChunk;
+        st_a.init(g, (uint32_t)ld, first, P, tid);
+        st_b.init(g, (uint32_t)ld, first, P, tid);
     }
     int cur = 0;
-    if (kBuffers == 2) st.store(lds, tid);
+    if (kBuffers == 2) {
+        load_chunk(st_a, p0);
+        st_a.store(lds, tid);
+        if (n_chunks > 1) load_chunk(st_b, p1);
+    } else {
+        load_chunk(st_b, p0);
+    }
     __syncthreads();  // publishes the table (and the first chunk)
 
     // the first two words of a block are bytes 0..7 = MFMA steps q = 0..7, the other two q = 8..15
@@ -505,102 +534,95 @@ __global__ __launch_bounds__(512) void jl_project_kernel(
         wd[j][0] = w.x, wd[j][1] = w.y, wd[j][2] = w.z, wd[j][3] = w.w;
     }
 
-    for (uint32_t tile = t0; tile <= t_last; ++tile) {
-        const uint64_t f_lo = (uint64_t)tile * tile_size;
-        const uint64_t f_hi = (f_lo + tile_size < P) ? f_lo + tile_size : P;  // may be <= f_lo (loads give zeros)
-        const uint32_t s_begin = tile == t0 ? s0 : 0u;
-        const uint32_t chunks = tile == t_last ? s_last_end : chunks_per_tile;
-        const uint64_t nf_lo = f_lo + tile_size;                               // next tile
-        const uint64_t nf_hi = (nf_lo + tile_size < P) ? nf_lo + tile_size : P;
+    // chunk number i of the run; `fill` is loaded with a later chunk, `drain` goes to LDS
+    auto chunk = [&](uint32_t i, Stage& fill, Stage& drain) __attribute__((always_inline)) {
+        if (kBuffers == 1) {
+            __syncthreads();  // everyone is done reading the previous chunk
+            drain.store(lds, tid);
+            __syncthreads();
+            if (i + 1 < n_chunks) load_chunk(fill, p1);
+        } else {
+            if (i + 2 < n_chunks) load_chunk(fill, p2);
+        }
+        const uint16_t* a_base = lds + cur * kBufElems + a_off;
 
-        for (uint32_t s = s_begin; s < chunks; ++s) {
-            const bool more_here = s + 1 < chunks;
-            const bool more = more_here || tile < t_last;
-            if (kBuffers == 1) {
-                __syncthreads();  // everyone is done reading the previous chunk
-                st.store(lds, tid);
-                __syncthreads();
-            }
-            if (more)
-                st.load(g, ld, rows, more_here ? f_lo + (uint64_t)(s + 1) * kChunk : nf_lo, more_here ? f_hi : nf_hi,
-                        tid);
-            const uint16_t* a_base = lds + cur * kBufElems + a_off;
-
-            // The next chunk's blocks (of the next tile when this one ends here): first round now -
-            // its counter is (block, stream name, 0, 0) and the block number is the same for the
-            // GPW groups, so it is one multiply for all of them and one xor per group - the other
-            // nine under the MFMAs below.
-            jl::u32x4 pc[GPW], pn[GPW];
-            {
-                const uint32_t nblk = more_here ? 2u * (s + 1) + h : h;
-                const uint32_t ntile = more_here ? tile : tile + 1u;
-                const uint64_t p0 = (uint64_t)jl::kPhiloxM0 * nblk;
+        // The next chunk's blocks: first round now - its counter is (block, stream name, 0, 0) and
+        // the block number is the same for the GPW groups, so it is one multiply for all of them
+        // and one xor per group - the other nine under the MFMAs below.
+        jl::u32x4 pc[GPW], pn[GPW];
+        {
+            const uint64_t q0 = (uint64_t)jl::kPhiloxM0 * (2u * p1.s + h);
 #pragma unroll
-                for (int j = 0; j < GPW; ++j) {
-                    pc[j].x = jl::stream_name(seed, col0 + 32u * j, ntile) ^ seed;
-                    pc[j].y = 0u;
-                    pc[j].z = (uint32_t)(p0 >> 32);
-                    pc[j].w = (uint32_t)p0;
-                }
-            }
-
-            auto operand = [&](int step) -> uint4 {
-                const int q = step / GPW, j = step % GPW;
-                return *reinterpret_cast<const uint4*>(smem + sign_entry_address(wd[j][q >> 2], q, lane_base));
-            };
-            uint4 bq[kAhead + 1];
-#pragma unroll
-            for (int p = 0; p < kAhead; ++p) bq[p] = operand(p);
-            uint4 a[2][kPlanes];  // A operands of this q and of the next one (read one q ahead)
-#pragma unroll
-            for (int pl = 0; pl < kPlanes; ++pl)
-                a[0][pl] = *reinterpret_cast<const uint4*>(a_base + pl * kPlaneElems);
-#pragma unroll
-            for (int q = 0; q < 16; ++q) {
-#pragma unroll
-                for (int j = 0; j < GPW; ++j) {
-                    const int step = q * GPW + j;
-                    if (step + kAhead < kSteps) bq[(step + kAhead) % (kAhead + 1)] = operand(step + kAhead);
-                    if (j == 0 && q + 1 < 16) {
-#pragma unroll
-                        for (int pl = 0; pl < kPlanes; ++pl)
-                            a[(q + 1) & 1][pl] =
-                                *reinterpret_cast<const uint4*>(a_base + pl * kPlaneElems + 8 * (q + 1));
-                    }
-                    // half rounds number first .. first + count - 1 of the kHalfRounds; number
-                    // i is half i % 2 of round 1 + i / (2 GPW) of group (i / 2) % GPW.  Every
-                    // kSteps / extra-th step takes two.
-                    {
-                        constexpr int kExtra = kHalfRounds - kSteps;       // steps that take two
-                        constexpr int kEvery = kSteps / kExtra;
-                        const int twos_before = (step + kEvery - 1) / kEvery;  // steps < step that took two
-                        const int first = step + (twos_before < kExtra ? twos_before : kExtra);
-                        const int count = (step % kEvery == 0 && step / kEvery < kExtra) ? 2 : 1;
-#pragma unroll
-                        for (int i = first; i < first + count; ++i) {
-                            const int r = 1 + i / (2 * GPW), g4 = (i / 2) % GPW, half = i % 2;
-                            philox_half(pc[g4], pn[g4], half, seed + (uint32_t)r * jl::kPhiloxW0,
-                                        (uint32_t)r * jl::kPhiloxW1);
-                            if (half == 1) pc[g4] = pn[g4];
-                        }
-                    }
-                    __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-                    for (int pl = 0; pl < kPlanes; ++pl)
-                        acc[j] = mfma16(a[q & 1][pl], bq[step % (kAhead + 1)], acc[j], kBf);
-                    __builtin_amdgcn_sched_barrier(0);
-                }
-            }
-#pragma unroll
-            for (int j = 0; j < GPW; ++j) wd[j][0] = pc[j].x, wd[j][1] = pc[j].y, wd[j][2] = pc[j].z, wd[j][3] = pc[j].w;
-
-            if (kBuffers == 2) {
-                // the other buffer was last read in the previous iteration, before its barrier
-                if (more) st.store(lds + (cur ^ 1) * kBufElems, tid);
-                __syncthreads();
-                cur ^= 1;
+            for (int j = 0; j < GPW; ++j) {
+                pc[j].x = jl::stream_name(seed, col0 + 32u * j, p1.tile) ^ seed;
+                pc[j].y = 0u;
+                pc[j].z = (uint32_t)(q0 >> 32);
+                pc[j].w = (uint32_t)q0;
             }
         }
+
+        auto operand = [&](int step) -> uint4 {
+            const int q = step / GPW, j = step % GPW;
+            return *reinterpret_cast<const uint4*>(smem + sign_entry_address(wd[j][q >> 2], q, lane_base));
+        };
+        uint4 bq[kAhead + 1];
+#pragma unroll
+        for (int p = 0; p < kAhead; ++p) bq[p] = operand(p);
+        uint4 a[2][kPlanes];  // A operands of this q and of the next one (read one q ahead)
+#pragma unroll
+        for (int pl = 0; pl < kPlanes; ++pl) a[0][pl] = *reinterpret_cast<const uint4*>(a_base + pl * kPlaneElems);
+#pragma unroll
+        for (int q = 0; q < 16; ++q) {
+#pragma unroll
+            for (int j = 0; j < GPW; ++j) {
+                const int step = q * GPW + j;
+                if (step + kAhead < kSteps) bq[(step + kAhead) % (kAhead + 1)] = operand(step + kAhead);
+                if (j == 0 && q + 1 < 16) {
+#pragma unroll
+                    for (int pl = 0; pl < kPlanes; ++pl)
+                        a[(q + 1) & 1][pl] =
+                            *reinterpret_cast<const uint4*>(a_base + pl * kPlaneElems + 8 * (q + 1));
+                }
+                // half rounds number first .. first + count - 1 of the kHalfRounds; number
+                // i is half i % 2 of round 1 + i / (2 GPW) of group (i / 2) % GPW.  Every
+                // kSteps / extra-th step takes two.
+                {
+                    constexpr int kExtra = kHalfRounds - kSteps;       // steps that take two
+                    constexpr int kEvery = kSteps / kExtra;
+                    const int twos_before = (step + kEvery - 1) / kEvery;  // steps < step that took two
+                    const int first = step + (twos_before < kExtra ? twos_before : kExtra);
+                    const int count = (step % kEvery == 0 && step / kEvery < kExtra) ? 2 : 1;
+#pragma unroll
+                    for (int u = first; u < first + count; ++u) {
+                        const int r = 1 + u / (2 * GPW), g4 = (u / 2) % GPW, half = u % 2;
+                        philox_half(pc[g4], pn[g4], half, seed + (uint32_t)r * jl::kPhiloxW0,
+                                    (uint32_t)r * jl::kPhiloxW1);
+                        if (half == 1) pc[g4] = pn[g4];
+                    }
+                }
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int pl = 0; pl < kPlanes; ++pl)
+                    acc[j] = mfma16(a[q & 1][pl], bq[step % (kAhead + 1)], acc[j], kBf);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < GPW; ++j) wd[j][0] = pc[j].x, wd[j][1] = pc[j].y, wd[j][2] = pc[j].z, wd[j][3] = pc[j].w;
+
+        if (kBuffers == 2) {
+            // the other buffer was last read in the previous chunk, before its barrier
+            if (i + 1 < n_chunks) drain.store(lds + (cur ^ 1) * kBufElems, tid);
+            __syncthreads();
+            cur ^= 1;
+        }
+        p0 = p1;
+        p1 = p2;
+        step_pos(p2);
+    };
+    for (uint32_t i = 0; i < n_chunks; i += 2) {
+        chunk(i, st_a, st_b);
+        if (i + 1 < n_chunks) chunk(i + 1, st_b, st_a);
     }
 
     // D[m][n] of a 32x32 MFMA: lane holds column n = lane % 32 and, in register r, row
