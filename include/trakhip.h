@@ -221,7 +221,8 @@ int trakhip_gram_split2(const void* A_planes_dev, const float* A_scales_dev, uin
  * (trak/score_computers.py:176) and `features @ target_grads.t()` (trak/utils.py:131).
  *   dtype      TRAKHIP_F16 | TRAKHIP_BF16, both operands
  *   K          a multiple of 64 (TRAKHIP_ERR_SHAPE otherwise; proj_dim is a multiple of 512)
- *   A_dev, B_dev  16-byte aligned, lda and ldb multiples of 8 elements (TRAKHIP_ERR_ALIGN otherwise)
+ *   A_dev, B_dev  16-byte aligned, lda and ldb multiples of 8 elements (TRAKHIP_ERR_ALIGN otherwise) and
+ *              below 2^23 elements (TRAKHIP_ERR_SHAPE otherwise)
  * A caller whose operands do not qualify uses trakhip_split_rows + trakhip_gemm_nt_split; the results
  * are the same bits (same MFMAs in the same order). */
 int trakhip_gemm_nt16(const void* A_dev, uint64_t lda, const void* B_dev, uint64_t ldb, int dtype, float* C_dev,

@@ -455,58 +455,52 @@ template <bool F16, bool ACCUM>
 __global__ __launch_bounds__(64 * kWaves, 2) void gemm_nt16_kernel(
     const piece* __restrict__ A, uint64_t lda8, const piece* __restrict__ B, uint64_t ldb8, uint64_t steps,
     float* __restrict__ C, uint64_t ldc, uint64_t M, uint64_t N, float alpha, float beta,
-    const float* __restrict__ row_scale, uint32_t tiles_n) {
+    const float* __restrict__ row_scale, uint32_t tiles_n, uint32_t tiles) {
     constexpr int JT = BN / kWavesN / 32;
     constexpr int kBufPieces = 8 * (BM + BN);  // 64 KB
     constexpr int kMoves = (BM + BN) / 8 / kWaves, kMovesA = BM / 8 / kWaves;  // chunks per wave and step
     __shared__ piece lds[2][kBufPieces];
 
-    const uint32_t tile_m = blockIdx.x / tiles_n, tile_n = blockIdx.x % tiles_n;
-    const uint64_t m0 = (uint64_t)tile_m * BM, n0 = (uint64_t)tile_n * BN;
     const int tid = threadIdx.x;
-    const int wave = tid >> 6, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;  // the wave number as a scalar
     const int wm = wave / kWavesN, wn = wave % kWavesN;
     const int x = lane & 31, h = lane >> 5;
+    const int a_row = (wm * 64 + x) * 8, b_row = (BM + wn * (32 * JT) + x) * 8;  // first piece of the lane's rows
 
-    // this lane's piece of step 0 in each chunk that its wave moves (chunks wave, wave + 8, ...)
-    const piece* src[kMoves];
-    {
+    // The workgroups are persistent: workgroup w computes tiles w, w + gridDim.x, ...  A load's address is a
+    // scalar base (first row of the tile, advanced by one 128-byte line per step) plus this lane's byte offset
+    // inside the tile's rows.
+    const char* a_tile;
+    const char* b_tile;
+    uint32_t voff[kMoves];
+    auto set_tile = [&](uint32_t t) {
+        const uint64_t m0 = (uint64_t)(t / tiles_n) * BM, n0 = (uint64_t)(t % tiles_n) * BN;
+        a_tile = reinterpret_cast<const char*>(A + m0 * lda8);
+        b_tile = reinterpret_cast<const char*>(B + n0 * ldb8);
         // rows 8c + sub of chunk c = wave + 8 i': (row >> 1) % 8 = 4 (wave % 2) + sub / 2
         const int sub = lane >> 3, oct = (lane & 7) ^ ((4 * (wave & 1) + (sub >> 1)) & 7);
 #pragma unroll
         for (int i = 0; i < kMoves; ++i) {
-            const int row = 8 * (wave + kWaves * (i % kMovesA)) + sub;
+            const uint32_t row = 8 * (wave + kWaves * (i % kMovesA)) + sub;
             if (i < kMovesA) {
-                const uint64_t g = m0 + row < M ? m0 + row : M - 1;
-                src[i] = A + g * lda8 + oct;
+                const uint64_t last = M - 1 - m0;
+                voff[i] = (uint32_t)(((row < last ? row : last) * lda8 + oct) * 16);
             } else {
-                const uint64_t g = n0 + row < N ? n0 + row : N - 1;
-                src[i] = B + g * ldb8 + oct;
+                const uint64_t last = N - 1 - n0;
+                voff[i] = (uint32_t)(((row < last ? row : last) * ldb8 + oct) * 16);
             }
         }
-    }
+    };
     auto dma = [&](uint64_t s, piece* buf) {
 #pragma unroll
         for (int i = 0; i < kMoves; ++i) {
-            const int c = (i < kMovesA ? 0 : BM / 8) + wave + kWaves * (i % kMovesA);  // wave-uniform
-            __builtin_amdgcn_global_load_lds((const void __attribute__((address_space(1)))*)(src[i] + 8 * s),
+            const int c = (i < kMovesA ? 0 : BM / 8) + wave + kWaves * (i % kMovesA);  // scalar
+            const char* base = (i < kMovesA ? a_tile : b_tile) + s * 128;
+            __builtin_amdgcn_global_load_lds((const void __attribute__((address_space(1)))*)(base + voff[i]),
                                              (void __attribute__((address_space(3)))*)(buf + 64 * c), 16, 0, 0);
         }
     };
 
-    floatx16 acc[2][JT];
-#pragma unroll
-    for (int i = 0; i < 2; ++i)
-#pragma unroll
-        for (int j = 0; j < JT; ++j)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
-
-    dma(0, lds[0]);
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    __syncthreads();
-
-    const int a_row = (wm * 64 + x) * 8, b_row = (BM + wn * (32 * JT) + x) * 8;  // first piece of the lane's rows
     // A step is four sub-steps of eight MFMAs (two A fragments x four B fragments).  The six fragments of
     // sub-step u + 1 are requested before the MFMAs of sub-step u are issued, so an LDS read has eight MFMAs
     // (256 cycles) to arrive instead of stalling the wave; the per-step barrier sits in front of the last
@@ -519,38 +513,69 @@ __global__ __launch_bounds__(64 * kWaves, 2) void gemm_nt16_kernel(
 #pragma unroll
         for (int j = 0; j < JT; ++j) fb[set][j] = l[b_row + 256 * j];
     };
-    fetch(0, 0, 0);
-    for (uint64_t s = 0; s < steps; ++s) {
-        const int cur = (int)(s & 1);
-        if (s + 1 < steps) dma(s + 1, lds[cur ^ 1]);
+
+    uint32_t tile = blockIdx.x;
+    if (tile >= tiles) return;
+    set_tile(tile);
+    int first = 0;  // buffer that holds step 0 of the current tile
+    dma(0, lds[0]);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+
+    for (;;) {
+        floatx16 acc[2][JT];
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
-            const int set = u & 1;
-            // Wait for this sub-step's fragments HERE, while they are the only LDS reads in flight: the
-            // compiler waits for all outstanding LDS reads at once (it cannot order them against the
-            // LDS-direct loads), so the next reads are issued after this point and stay in flight under
-            // the MFMAs.
-            asm volatile("" ::"v"(fa[set][0]), "v"(fa[set][1]), "v"(fb[set][0]), "v"(fb[set][1]), "v"(fb[set][2]),
-                         "v"(fb[set][3]));
-            __builtin_amdgcn_sched_barrier(0);
-            if (u < 3) {
-                fetch(cur, u + 1, set ^ 1);
-            } else {
-                // every read of this buffer has completed; wait for this wave's part of the next buffer,
-                // meet the other waves, then start on the next buffer
-                asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-                __syncthreads();
-                if (s + 1 < steps) fetch(cur ^ 1, 0, 0);
-            }
-            __builtin_amdgcn_sched_barrier(0);
+        for (int i = 0; i < 2; ++i)
 #pragma unroll
             for (int j = 0; j < JT; ++j)
 #pragma unroll
-                for (int i = 0; i < 2; ++i) acc[i][j] = mfma16<F16>(fa[set][i], fb[set][j], acc[i][j]);
-            __builtin_amdgcn_sched_barrier(0);
+                for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+        const uint64_t m0 = (uint64_t)(tile / tiles_n) * BM, n0 = (uint64_t)(tile % tiles_n) * BN;
+        const uint32_t next = tile + gridDim.x;
+
+        fetch(first, 0, 0);
+        for (uint64_t s = 0; s < steps; ++s) {
+            const int cur = (int)((s + first) & 1);
+            const bool last_step = s + 1 == steps;
+            if (!last_step) {
+                dma(s + 1, lds[cur ^ 1]);
+            } else if (next < tiles) {
+                // step 0 of the next tile arrives under the last MFMAs and the stores of this one
+                set_tile(next);
+                dma(0, lds[cur ^ 1]);
+            }
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const int set = u & 1;
+                // Wait for this sub-step's fragments HERE, while they are the only LDS reads in flight: the
+                // compiler waits for all outstanding LDS reads at once (it cannot order them against the
+                // LDS-direct loads), so the next reads are issued after this point and stay in flight under
+                // the MFMAs.
+                asm volatile("" ::"v"(fa[set][0]), "v"(fa[set][1]), "v"(fb[set][0]), "v"(fb[set][1]), "v"(fb[set][2]),
+                             "v"(fb[set][3]));
+                __builtin_amdgcn_sched_barrier(0);
+                if (u < 3) {
+                    fetch(cur, u + 1, set ^ 1);
+                } else {
+                    // every read of this buffer has completed; wait for this wave's part of the next buffer,
+                    // meet the other waves, then start on the next buffer
+                    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+                    __syncthreads();
+                    if (!last_step) fetch(cur ^ 1, 0, 0);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int j = 0; j < JT; ++j)
+#pragma unroll
+                    for (int i = 0; i < 2; ++i) acc[i][j] = mfma16<F16>(fa[set][i], fb[set][j], acc[i][j]);
+                __builtin_amdgcn_sched_barrier(0);
+            }
         }
+        store_c<ACCUM, JT>(acc, C, ldc, M, N, m0 + wm * 64, n0 + wn * (32 * JT) + x, h, alpha, beta, row_scale);
+        if (next >= tiles) break;
+        first = (int)((steps + first) & 1);
+        tile = next;
     }
-    store_c<ACCUM, JT>(acc, C, ldc, M, N, m0 + wm * 64, n0 + wn * (32 * JT) + x, h, alpha, beta, row_scale);
 }
 
 // C[i][j] = C[j][i] for j > i: completes a symmetric matrix whose lower triangle was computed.
@@ -818,6 +843,8 @@ int gemm_nt16(const void* A, uint64_t lda, const void* B, uint64_t ldb, int dtyp
     if (dtype != TRAKHIP_F16 && dtype != TRAKHIP_BF16) return TRAKHIP_ERR_DTYPE;
     if (M == 0 || N == 0) return TRAKHIP_OK;
     if (K == 0 || K % 64 || lda < K || ldb < K || ldc < N) return TRAKHIP_ERR_SHAPE;
+    // a lane's byte offset inside the 256 rows of a tile is kept in 32 bits
+    if (lda >= (1ull << 23) || ldb >= (1ull << 23)) return TRAKHIP_ERR_SHAPE;
     if (!A || !B || !C) return TRAKHIP_ERR_NULL;
     if ((reinterpret_cast<uintptr_t>(A) % 16) || (reinterpret_cast<uintptr_t>(B) % 16) || (lda % 8) || (ldb % 8) ||
         (reinterpret_cast<uintptr_t>(C) % 4))
@@ -825,15 +852,21 @@ int gemm_nt16(const void* A, uint64_t lda, const void* B, uint64_t ldb, int dtyp
     const uint64_t tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
     if (tiles_m * tiles_n > 0x7FFFFFFFull) return TRAKHIP_ERR_SHAPE;
     void (*kernel)(const piece*, uint64_t, const piece*, uint64_t, uint64_t, float*, uint64_t, uint64_t, uint64_t, float,
-                   float, const float*, uint32_t);
+                   float, const float*, uint32_t, uint32_t);
     const bool accum = beta != 0.0f;
     if (dtype == TRAKHIP_F16)
         kernel = accum ? gemm_nt16_kernel<true, true> : gemm_nt16_kernel<true, false>;
     else
         kernel = accum ? gemm_nt16_kernel<false, true> : gemm_nt16_kernel<false, false>;
-    hipLaunchKernelGGL(kernel, dim3((uint32_t)(tiles_m * tiles_n)), dim3(64 * kWaves), 0, s,
+    const uint32_t tiles = (uint32_t)(tiles_m * tiles_n);
+    // persistent workgroups, one per CU (128 KB of LDS each)
+    int dev = 0, cus = 0;
+    if (hipGetDevice(&dev) != hipSuccess ||
+        hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
+        cus = 256;
+    hipLaunchKernelGGL(kernel, dim3(tiles < (uint32_t)cus ? tiles : (uint32_t)cus), dim3(64 * kWaves), 0, s,
                        static_cast<const piece*>(A), lda / 8, static_cast<const piece*>(B), ldb / 8, K / 64, C, ldc, M, N,
-                       alpha, beta, row_scale, (uint32_t)tiles_n);
+                       alpha, beta, row_scale, (uint32_t)tiles_n, tiles);
     return hipGetLastError() == hipSuccess ? TRAKHIP_OK : TRAKHIP_ERR_LAUNCH;
 }
 

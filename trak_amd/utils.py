@@ -278,6 +278,8 @@ def nt16_ok(a, b):
     for t in (a, b):
         if t.stride(1) != 1 or t.data_ptr() % 16 or (t.shape[0] > 1 and (t.stride(0) % 8 or t.stride(0) < t.shape[1])):
             return False
+        if max(t.stride(0), t.shape[1]) >= 1 << 23:  # the kernel keeps a lane's offset inside a tile in 32 bits
+            return False
     return True
 
 
