@@ -16,7 +16,7 @@ cpu_baseline = the CPU restatement of trak's BasicProjector (oracle/basic_projec
 sustained = the same calls back to back for --sustain seconds (default 2).
 `scoring` = BasicScoreComputer at N=50_000, M=10_000, k=4096 fp32: GEMM TFLOP/s against the fp32
             MFMA peak, the SPD inverse separately, and a CPU sample beside it.
-`--only NAME` runs one workload alone (for profiler runs): c1 | c2 | c3_dict | c4 | c4_rademacher |
+`--only NAME` runs one workload alone (for profiler runs): c1 | c2 | c3_dict | c4 | c4_rademacher | vendor_gemm |
             scoring | mfma_rate.
 """
 import argparse
@@ -311,6 +311,27 @@ MFMA_RATE_CASES = [
 ]
 
 
+def bench_vendor_gemm(torch, dev, reps=6):
+    """The scores product of the fp16 scoring section through torch.mm (hipBLASLt), fp32 result: the
+    library kernel that `gemm_nt16_kernel` is compared with, on the same operands, for profiler runs."""
+    g = torch.Generator(device=dev).manual_seed(1)
+    out = {}
+    for name, dt in (("fp16", torch.float16), ("bf16", torch.bfloat16)):
+        X = (torch.randn(50_000, 4096, generator=g, device=dev) / 64).to(dt)
+        T = (torch.randn(10_000, 4096, generator=g, device=dev) / 64).to(dt)
+        for _ in range(3):
+            torch.mm(X, T.T, out_dtype=torch.float32)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            torch.mm(X, T.T, out_dtype=torch.float32)
+        torch.cuda.synchronize()
+        ms = (time.perf_counter() - t0) / reps * 1e3
+        out[name] = {"scores_ms": ms, "tflops": 2.0 * 50_000 * 10_000 * 4096 / (ms * 1e-3) / 1e12}
+        del X, T
+    return out
+
+
 def bench_mfma_rate(torch, dev, iters=300_000):
     """What a loop of nothing but independent MFMAs sustains on this machine, by operand data (the
     clock is power limited, so the rate depends on the data): the reference point for the projection
@@ -590,7 +611,8 @@ def main():
                     help="also time the other projection configurations and print them to stderr")
     ap.add_argument("--only", default=None, metavar="NAME",
                     help="run just one workload for --steps calls and print its timing (for profiler runs): "
-                         "c1 | c2 | c3_dict | c4 | c4_rademacher | scoring | mfma_rate")
+                         "c1 | c2 | c3_dict | c4 | c4_rademacher | scoring | mfma_rate | vendor_gemm "
+                         "(torch.mm on the scoring operands, for comparison)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run one 1 GiB device-to-device copy (reference point for rocprofv3 byte counters)")
     args = ap.parse_args()
@@ -614,6 +636,8 @@ def main():
     if args.only:
         if args.only == "mfma_rate":
             print(json.dumps({"only": "mfma_rate", **bench_mfma_rate(torch, dev)}))
+        elif args.only == "vendor_gemm":
+            print(json.dumps({"only": "vendor_gemm", **bench_vendor_gemm(torch, dev)}))
         elif args.only == "scoring":
             print(json.dumps({"only": "scoring", **bench_scoring(torch, dev, reps=max(1, min(args.steps, 3)))}))
         else:
