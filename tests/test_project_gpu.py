@@ -82,8 +82,8 @@ def test_projection_matches_float64_contraction(gpu, c_oracle, proj_type, dtype,
     seed = 123 + B
     out = fn(proj_type)(g, k, seed, tiles)
     assert out.shape == (B, k) and out.dtype == torch.float32 and out.device == g.device  # fast_jl.cu:48-49,78
-    # 512-, 1024- and 1536-column boundaries: four-wave workgroups (k an odd multiple of 512) cover 512
-    # columns, eight-wave ones 1024
+    # 512-, 1024- and 1536-column boundaries: a workgroup covers 512 columns when k is an odd multiple of
+    # 512 (two column groups per wave), 1024 otherwise (four)
     cols = [c for c in (0, 31, 32, 511, 512, 1023, 1024, 1535, 2047, 2559) if c < k]
     g32 = to_f32_numpy(g)
     for c in cols:
