@@ -187,6 +187,7 @@ def test_gemm_nt16_validates_before_touching_the_device():
     assert mm(M=0) == 0 and mm(N=0, dt=BF16) == 0
     assert mm(K=0) == -2 and mm(K=32) == -2 and mm(K=100, lda=104, ldb=104) == -2     # K % 64
     assert mm(lda=56) == -2 and mm(ldb=63) == -2 and mm(ldc=7) == -2
+    assert mm(lda=1 << 23) == -2 and mm(ldb=1 << 23) == -2     # a lane's offset inside a tile stays in 32 bits
     assert mm(a=None) == -5 and mm(b=None) == -5 and mm(c=None) == -5
     assert mm(a=ctypes.c_void_p(4104)) == -7 and mm(b=ctypes.c_void_p(4098)) == -7     # 16-byte rows
     assert mm(lda=68) == -7 and mm(ldb=100) == -7 and mm(c=ctypes.c_void_p(4098)) == -7
