@@ -52,9 +52,18 @@ int trakhip_abi_version(void);
 
 /* ---- JL projection -------------------------------------------------------------------- */
 
-/* Bytes of scratch trakhip_project needs for these sizes.  Stands in for the
- * torch::zeros({B_pad, T, N}) intermediate of fast_jl/fast_jl.cu:48-49. */
+/* Bytes of scratch a caller should bring to trakhip_project for these sizes: room for passes of
+ * trakhip_project_rows_per_pass() = 64 rows.  Stands in for the torch::zeros({B_pad, T, N})
+ * intermediate of fast_jl/fast_jl.cu:48-49.  trakhip_project_workspace_min: the least that
+ * trakhip_project accepts (passes of 32 rows: half as much once B >= 64; the call then runs 32 rows
+ * at a time, with the same results). */
 size_t trakhip_project_workspace(uint64_t B, uint64_t P, uint32_t proj_dim, uint32_t num_feature_tiles);
+size_t trakhip_project_workspace_min(uint64_t B, uint64_t P, uint32_t proj_dim, uint32_t num_feature_tiles);
+
+/* Rows that one pass of the projection kernel takes: 64 for fp16 / bf16 gradients under a Rademacher
+ * matrix (two 32-row MFMA blocks share every generated matrix entry), 32 otherwise.  The reference
+ * has passes of 8, 16 or 32 rows (fast_jl/fast_jl.cu:44-76). */
+uint32_t trakhip_project_rows_per_pass(int in_dtype, int proj_type);
 
 /* out[B, proj_dim] (fp32) = in[B, P] x S, S generated on the fly from (seed, proj_dim,
  * num_feature_tiles, P).  Stands in for the six functions project_{rademacher,normal}_{8,16,32}
@@ -63,7 +72,8 @@ size_t trakhip_project_workspace(uint64_t B, uint64_t P, uint32_t proj_dim, uint
  *   in_dev      row-major [B, P] with row pitch ld_in >= P elements, aligned to its element size
  *   in_dtype    TRAKHIP_F16 | TRAKHIP_BF16 | TRAKHIP_F32
  *   out_dev     [B, proj_dim] fp32, contiguous, 16-byte aligned; fully overwritten
- *   workspace   >= trakhip_project_workspace(...) bytes, 16-byte aligned
+ *   workspace   >= trakhip_project_workspace_min(...) bytes, 16-byte aligned (trakhip_project_workspace(...)
+ *               bytes for the fastest path)
  *   proj_dim    multiple of 512;  P < 2^32;  any B >= 1
  */
 int trakhip_project(const void* in_dev, int in_dtype, uint64_t B, uint64_t P, uint64_t ld_in,
@@ -75,8 +85,8 @@ int trakhip_project(const void* in_dev, int in_dtype, uint64_t B, uint64_t P, ui
  * fast_jl allocates its intermediate with torch::zeros on every call (fast_jl/fast_jl.cu:48-49).
  * Same arguments, checks and results (bit for bit) as trakhip_project, minus the workspace: the
  * partial sums live in a static device array of trakhip_project_static_limit() bytes (36 MiB) that
- * each GPU the library runs on holds until the process ends.  A shape whose
- * trakhip_project_workspace() exceeds that is refused with TRAKHIP_ERR_STATIC_LIMIT (every shape
+ * each GPU the library runs on holds until the process ends (rows go 32 at a time).  A shape whose
+ * trakhip_project_workspace_min() exceeds that is refused with TRAKHIP_ERR_STATIC_LIMIT (every shape
  * with proj_dim <= 65536 fits).  Calls no hipMalloc / hipFree or any allocating routine.  All calls
  * on one GPU share the one array: calls that overlap in time on the same GPU (different streams
  * or threads) race and give wrong results; calls that follow one another on a stream do not. */
@@ -85,7 +95,8 @@ int trakhip_project_static(const void* in_dev, int in_dtype, uint64_t B, uint64_
                            float* out_dev, uint32_t proj_dim, uint32_t seed, uint32_t num_feature_tiles,
                            int proj_type, void* stream);
 
-/* The two phases of trakhip_project as separate calls, for B <= 32 rows: phase 1 writes partial
+/* The two phases of trakhip_project as separate calls, for one pass of B <= trakhip_project_rows_per_pass()
+ * rows (workspace >= trakhip_project_workspace(B, ...)): phase 1 writes partial
  * sums [G, B, proj_dim] over G runs of consecutive features to the workspace (the kernel of
  * fast_jl/fast_jl_kernel.cuh:24-105 writing `output[row][tile][col]`; G depends only on the shape),
  * phase 2 adds them up in order into out_dev (the `.sum(1)` of fast_jl/fast_jl.cu:78), multiplied by
@@ -123,7 +134,7 @@ typedef struct trakhip_segment {
  * dense matrix: the flatten-and-copy of trak.utils.vectorize (trak/utils.py:80-110) and the chunk
  * packing of ChunkedCudaProjector.project (trak/projectors.py:479-503) disappear.  segs_dev is a
  * device array of n_segs segments, sorted by `first`, contiguous (first[i+1] = first[i] + numel[i])
- * and covering [0, P); all of element type in_dtype; B <= 32.  Result and workspace as for
+ * and covering [0, P); all of element type in_dtype; B <= trakhip_project_rows_per_pass().  Result and workspace as for
  * trakhip_project_partials; finish with trakhip_project_reduce. */
 int trakhip_project_gather_partials(const trakhip_segment* segs_dev, uint32_t n_segs, int in_dtype, uint64_t B,
                                     uint64_t P, void* workspace_dev, size_t workspace_bytes, uint32_t proj_dim,

@@ -78,7 +78,14 @@ def test_workspace_size():
     lib = _lib.load()
     # G * min(B, 32) * k floats, G = number of feature runs (about 512 workgroups / (k / 512))
     assert lib.trakhip_project_workspace(32, 11_689_512, 4096, 256) == 64 * 32 * 4096 * 4
-    assert lib.trakhip_project_workspace(48, 1000, 512, 256) == 256 * 32 * 512 * 4      # 256 tiles x 1 chunk
+    assert lib.trakhip_project_workspace(48, 1000, 512, 256) == 256 * 48 * 512 * 4      # 256 tiles x 1 chunk
+    assert lib.trakhip_project_workspace_min(48, 1000, 512, 256) == 256 * 32 * 512 * 4
+    assert lib.trakhip_project_workspace(200, 1000, 512, 256) == 256 * 64 * 512 * 4
+    assert lib.trakhip_project_workspace_min(8, 25, 1024, 256) == 25 * 8 * 1024 * 4
+    F16, BF16, F32 = _lib.F16, _lib.BF16, _lib.F32
+    rpp = lib.trakhip_project_rows_per_pass
+    assert rpp(F16, _lib.RADEMACHER) == 64 and rpp(BF16, _lib.RADEMACHER) == 64 and rpp(F32, _lib.RADEMACHER) == 32
+    assert rpp(F16, _lib.NORMAL) == 32 and rpp(BF16, _lib.NORMAL) == 32 and rpp(F32, _lib.NORMAL) == 32
     assert lib.trakhip_project_workspace(8, 25, 1024, 256) == 25 * 8 * 1024 * 4
     assert lib.trakhip_project_workspace(16, 1_048_576, 512, 256) == 256 * 16 * 512 * 4  # one 512-column block
     assert lib.trakhip_project_workspace(0, 25, 1024, 256) == 0
@@ -125,7 +132,7 @@ def test_store_entry_points_validate_before_touching_the_device():
         kw.get("ws", p), kw.get("B", 8), kw.get("P", 1000), kw.get("k", 512), kw.get("tiles", 256), 1.0,
         kw.get("dt", 0), kw.get("out", p), kw.get("ld", 512), None)
     assert red(k=100) == -1
-    assert red(B=0) == -2 and red(B=33) == -2 and red(ld=508) == -2 and red(P=0) == -2
+    assert red(B=0) == -2 and red(B=65) == -2 and red(ld=508) == -2 and red(P=0) == -2
     assert red(dt=3) == -3
     assert red(ws=None) == -5 and red(out=None) == -5
     assert red(out=ctypes.c_void_p(4100)) == -7 and red(ld=514) == -7

@@ -532,19 +532,23 @@ def test_gather_equals_vectorize_then_project(gpu, c_oracle, proj_type, dtype):
     assert torch.equal(proj.project(flat, model_id=0), dense)
 
 
-def test_gather_many_rows_and_tiny_segments(gpu):
-    # B > 32 walks the rows in blocks of 32; segments of one feature straddle every 16-byte piece
+@pytest.mark.parametrize("B,k", [(45, 512), (70, 1024), (64, 2048)])
+def test_gather_many_rows_and_tiny_segments(gpu, B, k):
+    # B > 32: 16-bit gradients under a Rademacher matrix go through the kernel 64 rows at a time (two 32-row
+    # blocks per generated operand); segments of one feature straddle every 16-byte piece
     from trak_amd import vectorize
 
     gen = torch.Generator(device="cpu").manual_seed(78)
-    B = 45
     grads = {i: torch.randn(B, n, generator=gen).half().to(gpu) for i, n in enumerate([1, 1, 3, 1, 5, 2, 900, 1, 1, 7, 4000, 3])}
     flat = vectorize(grads, device=gpu)
-    dense = fn(R)(flat, 512, 11, 256)
-    assert torch.equal(fast_jl.project_gather(list(grads.values()), 512, 11, 256, "rademacher"), dense)
+    dense = fn(R)(flat, k, 11, 256)
+    assert torch.equal(fast_jl.project_gather(list(grads.values()), k, 11, 256, "rademacher"), dense)
+    # the same rows 32 at a time (the other kernel instance) give the same bits
+    for b0 in range(0, B, 32):
+        assert torch.equal(fn(R)(flat[b0:b0 + 32].contiguous(), k, 11, 256), dense[b0:b0 + 32])
 
 
-# ---- more than 32 rows: the batch is walked 32 rows at a time ------------------------------------
+# ---- more than 32 rows: the batch is walked 64 or 32 rows at a time -----------------------------
 
 
 @pytest.mark.parametrize("proj_type", [R, G])

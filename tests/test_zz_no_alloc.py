@@ -35,7 +35,8 @@ def _project(lib, x, k, seed, tiles, pt, static):
 def test_static_entry_point_equals_workspace_entry_point_twice(gpu, pt):
     lib = _lib.load()
     gen = torch.Generator(device="cpu").manual_seed(5)
-    # first call: 40 rows (two passes of 32 + 8 through the array), ragged P; second: smaller in every way
+    # first call: 40 rows (two passes of 32 + 8 through the array, against one 40-row pass with the workspace),
+    # ragged P; second: smaller in every way
     shapes = [(40, 300_001, 1024, torch.float16), (7, 20_011, 512, torch.float32)]
     for B, P, k, dt in shapes:
         x = (torch.randn(B, P, generator=gen) * 1e-2).to(dt).to(gpu)

@@ -40,6 +40,10 @@ def load():
     lib.trakhip_abi_version.restype = i32
     lib.trakhip_project_workspace.argtypes = [u64, u64, u32, u32]
     lib.trakhip_project_workspace.restype = sz
+    lib.trakhip_project_workspace_min.argtypes = [u64, u64, u32, u32]
+    lib.trakhip_project_workspace_min.restype = sz
+    lib.trakhip_project_rows_per_pass.argtypes = [i32, i32]
+    lib.trakhip_project_rows_per_pass.restype = u32
     lib.trakhip_project.argtypes = [vp, i32, u64, u64, u64, vp, vp, sz, u32, u32, u32, i32, vp]
     lib.trakhip_project.restype = i32
     lib.trakhip_project_static_limit.argtypes = []

@@ -32,6 +32,14 @@ size_t trakhip_project_workspace(uint64_t B, uint64_t P, uint32_t proj_dim, uint
     return trakhip::project_workspace_bytes(B, P, proj_dim, num_feature_tiles);
 }
 
+size_t trakhip_project_workspace_min(uint64_t B, uint64_t P, uint32_t proj_dim, uint32_t num_feature_tiles) {
+    return trakhip::project_workspace_min_bytes(B, P, proj_dim, num_feature_tiles);
+}
+
+uint32_t trakhip_project_rows_per_pass(int in_dtype, int proj_type) {
+    return trakhip::project_rows_per_pass(in_dtype, proj_type);
+}
+
 int trakhip_project(const void* in_dev, int in_dtype, uint64_t B, uint64_t P, uint64_t ld_in, float* out_dev,
                     void* workspace_dev, size_t workspace_bytes, uint32_t proj_dim, uint32_t seed,
                     uint32_t num_feature_tiles, int proj_type, void* stream) {

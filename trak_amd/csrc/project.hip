@@ -48,6 +48,7 @@ constexpr int kPieces = 32 * 32;                      // 16-byte pieces of a [32
 constexpr int kChunk = 256;                           // features per staged chunk
 constexpr int kLdsRow = kChunk + 8;                   // 16-bit elements; 528 B keeps b128 reads conflict free
 constexpr int kPlaneElems = 32 * kLdsRow;
+constexpr int kPlaneElems32 = kPlaneElems;
 
 struct __attribute__((packed, aligned(2))) Raw16 {
     uint32_t x, y, z, w;
@@ -84,16 +85,17 @@ __device__ __forceinline__ floatx16 mfma16(const uint4& a, const uint4& b, float
 
 // ---- staging of a [32 x 256] gradient chunk ------------------------------------------------
 
-// 16-bit inputs: every thread moves N = 16 / W 16-byte pieces, 2 W rows apart.
-template <int W>
+// 16-bit inputs: every thread moves N = ROWS / (2 W) 16-byte pieces, 2 W rows apart (ROWS = 32, or 64
+// for the kernel that multiplies two 32-row blocks by every operand).
+template <int W, int ROWS = 32>
 struct Stage16 {
-    static constexpr int N = kPieces / (64 * W);
+    static constexpr int N = ROWS * 32 / (64 * W);
     static constexpr int kThreads = 64 * W;
     uint4 v[N];
 
     __device__ __forceinline__ void load(const uint16_t* __restrict__ g, uint64_t ld, uint32_t rows,
                                          uint64_t f_begin, uint64_t f_end, int tid) {
-        if (rows == 32 && f_begin + kChunk <= f_end) {
+        if (rows == ROWS && f_begin + kChunk <= f_end) {
             // whole chunk in range (uniform test): unguarded 16-byte loads
             const uint16_t* p = g + (uint64_t)(tid >> 5) * ld + f_begin + 8u * (tid & 31);
 #pragma unroll
@@ -258,10 +260,10 @@ __device__ __noinline__ uint4 gather_piece(const trakhip_segment* segs, uint32_t
     return {e[0], e[1], e[2], e[3]};
 }
 
-template <int W>
-struct Gather16 : Stage16<W> {
-    static constexpr int N = Stage16<W>::N;
-    using Stage16<W>::v;
+template <int W, int ROWS = 32>
+struct Gather16 : Stage16<W, ROWS> {
+    static constexpr int N = Stage16<W, ROWS>::N;
+    using Stage16<W, ROWS>::v;
     SegCursor<N> cur;
     __device__ __forceinline__ void init(const trakhip_segment* segs, uint32_t n, uint64_t f_begin, uint64_t P,
                                          int tid) {
@@ -330,28 +332,28 @@ struct Gather32 : Stage32<W> {
     }
 };
 
-template <int IN, bool GATHER, int W>
+template <int IN, bool GATHER, int W, int ROWS = 32>
 struct StageOf {
-    typedef Stage16<W> type;
+    typedef Stage16<W, ROWS> type;
     typedef uint16_t elem;
 };
-template <int W>
-struct StageOf<TRAKHIP_F32, false, W> {
+template <int W, int ROWS>
+struct StageOf<TRAKHIP_F32, false, W, ROWS> {
     typedef Stage32<W> type;
     typedef float elem;
 };
-template <int W>
-struct StageOf<TRAKHIP_F16, true, W> {
-    typedef Gather16<W> type;
+template <int W, int ROWS>
+struct StageOf<TRAKHIP_F16, true, W, ROWS> {
+    typedef Gather16<W, ROWS> type;
     typedef trakhip_segment elem;
 };
-template <int W>
-struct StageOf<TRAKHIP_BF16, true, W> {
-    typedef Gather16<W> type;
+template <int W, int ROWS>
+struct StageOf<TRAKHIP_BF16, true, W, ROWS> {
+    typedef Gather16<W, ROWS> type;
     typedef trakhip_segment elem;
 };
-template <int W>
-struct StageOf<TRAKHIP_F32, true, W> {
+template <int W, int ROWS>
+struct StageOf<TRAKHIP_F32, true, W, ROWS> {
     typedef Gather32<W> type;
     typedef trakhip_segment elem;
 };
@@ -419,21 +421,26 @@ __device__ __forceinline__ void philox_half(const jl::u32x4& c, jl::u32x4& next,
 // MFMAs of a wave fit into the time of one MFMA of each of the two waves of the SIMD (8 issue
 // slots of 4 cycles each, two of them for a 64-bit multiply), which is why the generator is cut
 // that fine.
-template <int IN, bool GATHER, int GPW>
+//
+// RB = 32-row blocks per pass: 1, or 2 for 16-bit gradients when the batch has more than 32 rows - every
+// looked-up operand (and the generator behind it) then feeds two MFMAs.
+template <int IN, bool GATHER, int GPW, int RB>
 __global__ __launch_bounds__(512) void jl_project_kernel(
     const void* __restrict__ g_in, uint64_t ld, uint32_t rows, uint64_t P, uint32_t k,
     uint32_t seed, uint32_t tiles, uint64_t tile_size, uint32_t chunks_per_tile,
     uint32_t chunks_per_group, float* __restrict__ partial) {
     constexpr int W = 8;
     typedef InTraits<IN> Tr;
-    typedef typename StageOf<IN, GATHER, W>::type Stage;
-    typedef typename StageOf<IN, GATHER, W>::elem Elem;
+    typedef typename StageOf<IN, GATHER, W, 32 * RB>::type Stage;
+    typedef typename StageOf<IN, GATHER, W, 32 * RB>::elem Elem;
     constexpr int kColsPerWG = W * GPW * 32;
     constexpr bool kBf = Tr::bf16;
     constexpr int kPlanes = Tr::planes;
+    static_assert(RB == 1 || kPlanes == 1, "two row blocks: 16-bit gradients only (LDS)");
     // 16-bit inputs: two LDS buffers, one barrier per chunk.  fp32 inputs (three planes) keep one
     // buffer and two barriers: two buffers of three planes do not fit next to the table.
     constexpr int kBuffers = kPlanes == 1 ? 2 : 1;
+    constexpr int kPlaneElems = RB * kPlaneElems32;  // this kernel's plane: 32 RB rows
     constexpr int kBufElems = kPlanes * kPlaneElems;
     constexpr int kSteps = 16 * GPW;
     constexpr int kAhead = 3;                       // operand reads in flight
@@ -476,14 +483,16 @@ __global__ __launch_bounds__(512) void jl_project_kernel(
         }
     }
 
-    floatx16 acc[GPW];
+    floatx16 acc[RB][GPW];
 #pragma unroll
-    for (int j = 0; j < GPW; ++j)
+    for (int rb = 0; rb < RB; ++rb)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) acc[j][r] = 0.0f;
+        for (int j = 0; j < GPW; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[rb][j][r] = 0.0f;
 
     const Elem* g = reinterpret_cast<const Elem*>(g_in);
-    const uint32_t a_off = n * kLdsRow + 128 * h;
+    const uint32_t a_off = n * kLdsRow + 128 * h;  // row block rb: + 32 rb rows
     const uint32_t lane_base = (uint32_t)(lane & 15) << 4;
 
     // Position (tile, chunk in tile) of a chunk of the run, and its feature range.
@@ -509,18 +518,22 @@ __global__ __launch_bounds__(512) void jl_project_kernel(
 
     // Two sets of staging registers take turns: with two LDS buffers the loads of chunk i + 2 are
     // issued at the top of chunk i and stored to LDS at the end of chunk i + 1, so a load has two
-    // chunk times (about 6 us) to arrive before a wave has to wait for it at the barrier.
-    Stage st_a, st_b;
+    // chunk times (about 6 us) to arrive before a wave has to wait for it at the barrier.  With two row
+    // blocks the registers do not allow a second set: the loads of chunk i + 1 are issued at the top of
+    // chunk i (a chunk takes twice as long there).
+    constexpr bool kTwoSets = RB == 1;
+    Stage st_a, st_b_storage;
+    Stage& st_b = kTwoSets ? st_b_storage : st_a;
     if constexpr (GATHER) {
         const uint64_t first = (uint64_t)t0 * tile_size + (uint64_t)s0 * kChunk;
         st_a.init(g, (uint32_t)ld, first, P, tid);
-        st_b.init(g, (uint32_t)ld, first, P, tid);
+        if (kTwoSets) st_b_storage.init(g, (uint32_t)ld, first, P, tid);
     }
     int cur = 0;
     if (kBuffers == 2) {
         load_chunk(st_a, p0);
         st_a.store(lds, tid);
-        if (n_chunks > 1) load_chunk(st_b, p1);
+        if (kTwoSets && n_chunks > 1) load_chunk(st_b, p1);
     } else {
         load_chunk(st_b, p0);
     }
@@ -541,8 +554,10 @@ __global__ __launch_bounds__(512) void jl_project_kernel(
             drain.store(lds, tid);
             __syncthreads();
             if (i + 1 < n_chunks) load_chunk(fill, p1);
-        } else {
+        } else if (kTwoSets) {
             if (i + 2 < n_chunks) load_chunk(fill, p2);
+        } else {
+            if (i + 1 < n_chunks) load_chunk(fill, p1);
         }
         const uint16_t* a_base = lds + cur * kBufElems + a_off;
 
@@ -568,9 +583,12 @@ __global__ __launch_bounds__(512) void jl_project_kernel(
         uint4 bq[kAhead + 1];
 #pragma unroll
         for (int p = 0; p < kAhead; ++p) bq[p] = operand(p);
-        uint4 a[2][kPlanes];  // A operands of this q and of the next one (read one q ahead)
+        uint4 a[2][RB][kPlanes];  // A operands of this q and of the next one (read one q ahead)
 #pragma unroll
-        for (int pl = 0; pl < kPlanes; ++pl) a[0][pl] = *reinterpret_cast<const uint4*>(a_base + pl * kPlaneElems);
+        for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+            for (int pl = 0; pl < kPlanes; ++pl)
+                a[0][rb][pl] = *reinterpret_cast<const uint4*>(a_base + rb * 32 * kLdsRow + pl * kPlaneElems);
 #pragma unroll
         for (int q = 0; q < 16; ++q) {
 #pragma unroll
@@ -579,9 +597,11 @@ __global__ __launch_bounds__(512) void jl_project_kernel(
                 if (step + kAhead < kSteps) bq[(step + kAhead) % (kAhead + 1)] = operand(step + kAhead);
                 if (j == 0 && q + 1 < 16) {
 #pragma unroll
-                    for (int pl = 0; pl < kPlanes; ++pl)
-                        a[(q + 1) & 1][pl] =
-                            *reinterpret_cast<const uint4*>(a_base + pl * kPlaneElems + 8 * (q + 1));
+                    for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+                        for (int pl = 0; pl < kPlanes; ++pl)
+                            a[(q + 1) & 1][rb][pl] = *reinterpret_cast<const uint4*>(
+                                a_base + rb * 32 * kLdsRow + pl * kPlaneElems + 8 * (q + 1));
                 }
                 // half rounds number first .. first + count - 1 of the kHalfRounds; number
                 // i is half i % 2 of round 1 + i / (2 GPW) of group (i / 2) % GPW.  Every
@@ -602,8 +622,10 @@ __global__ __launch_bounds__(512) void jl_project_kernel(
                 }
                 __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-                for (int pl = 0; pl < kPlanes; ++pl)
-                    acc[j] = mfma16(a[q & 1][pl], bq[step % (kAhead + 1)], acc[j], kBf);
+                for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+                    for (int pl = 0; pl < kPlanes; ++pl)
+                        acc[rb][j] = mfma16(a[q & 1][rb][pl], bq[step % (kAhead + 1)], acc[rb][j], kBf);
                 __builtin_amdgcn_sched_barrier(0);
             }
         }
@@ -629,11 +651,14 @@ __global__ __launch_bounds__(512) void jl_project_kernel(
     // m = 8*(r/4) + 4*(lane/32) + r%4.
     float* out = partial + (uint64_t)group * rows * k;
 #pragma unroll
-    for (int j = 0; j < GPW; ++j) {
+    for (int rb = 0; rb < RB; ++rb) {
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-            const uint32_t m = 8u * (r >> 2) + 4u * h + (r & 3);
-            if (m < rows) out[(uint64_t)m * k + col0 + 32u * j] = acc[j][r];
+        for (int j = 0; j < GPW; ++j) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const uint32_t m = 32u * rb + 8u * (r >> 2) + 4u * h + (r & 3);
+                if (m < rows) out[(uint64_t)m * k + col0 + 32u * j] = acc[rb][j][r];
+            }
         }
     }
 }
@@ -1074,8 +1099,18 @@ hipError_t launch_rademacher(const void* in, uint64_t ld, uint32_t rows, uint64_
     const uint32_t groups8 = (pl.groups + 7u) / 8u * 8u;
     const uint64_t wgs = (uint64_t)groups8 * pl.col_blocks;
     if (wgs > 0x7FFFFFFFull) return hipErrorInvalidValue;
-    hipLaunchKernelGGL((jl_project_kernel<IN, GATHER, GPW>), dim3((uint32_t)wgs), dim3(512), 0, s, in, ld, rows, P,
-                       k, seed, pl.tl.tiles, pl.tl.tile_size, pl.chunks_per_tile, pl.chunks_per_group, partial);
+    if (rows > 32) {
+        // two 32-row blocks per pass (16-bit gradients only)
+        if constexpr (IN == TRAKHIP_F32) {
+            return hipErrorInvalidValue;
+        } else {
+            hipLaunchKernelGGL((jl_project_kernel<IN, GATHER, GPW, 2>), dim3((uint32_t)wgs), dim3(512), 0, s, in, ld, rows,
+                               P, k, seed, pl.tl.tiles, pl.tl.tile_size, pl.chunks_per_tile, pl.chunks_per_group, partial);
+        }
+    } else {
+        hipLaunchKernelGGL((jl_project_kernel<IN, GATHER, GPW, 1>), dim3((uint32_t)wgs), dim3(512), 0, s, in, ld, rows, P,
+                           k, seed, pl.tl.tiles, pl.tl.tile_size, pl.chunks_per_tile, pl.chunks_per_group, partial);
+    }
     return hipGetLastError();
 }
 
@@ -1122,12 +1157,27 @@ static std::atomic<void*> static_scratch_ptr[kMaxDevices];
 
 namespace trakhip {
 
-size_t project_workspace_bytes(uint64_t B, uint64_t P, uint32_t k, uint32_t num_feature_tiles) {
+// Rows of one pass of the projection kernel: 16-bit gradients under a Rademacher matrix go 64 rows at a
+// time (two 32-row MFMA blocks share every generated operand), everything else 32.
+uint32_t project_rows_per_pass(int dtype, int proj_type) {
+    return (dtype == TRAKHIP_F16 || dtype == TRAKHIP_BF16) && proj_type == TRAKHIP_RADEMACHER ? 64u : 32u;
+}
+
+static size_t workspace_for_rows(uint64_t B, uint64_t P, uint32_t k, uint32_t num_feature_tiles, uint64_t pass_rows) {
     if (B == 0 || P == 0 || k == 0 || num_feature_tiles == 0) return 0;
     if (k % kColsMultiple != 0 || P > 0xFFFFFFFFull) return 0;
     const Plan pl = make_plan(P, k, num_feature_tiles);
-    const uint64_t rows = B < 32 ? B : 32;
+    const uint64_t rows = B < pass_rows ? B : pass_rows;
     return (size_t)pl.groups * rows * k * sizeof(float);
+}
+
+// What a caller should bring: room for passes of 64 rows.  Passes of 32 rows (half of it for B >= 64) are
+// the minimum every entry point accepts.
+size_t project_workspace_bytes(uint64_t B, uint64_t P, uint32_t k, uint32_t num_feature_tiles) {
+    return workspace_for_rows(B, P, k, num_feature_tiles, 64);
+}
+size_t project_workspace_min_bytes(uint64_t B, uint64_t P, uint32_t k, uint32_t num_feature_tiles) {
+    return workspace_for_rows(B, P, k, num_feature_tiles, 32);
 }
 
 static int check_project_args(const void* in, int dtype, uint64_t B, uint64_t P, uint64_t ld, const void* ws,
@@ -1138,7 +1188,7 @@ static int check_project_args(const void* in, int dtype, uint64_t B, uint64_t P,
     if (B == 0 || P == 0 || P > 0xFFFFFFFFull || num_feature_tiles == 0) return TRAKHIP_ERR_SHAPE;
     if (ld < P) return TRAKHIP_ERR_SHAPE;
     if (!in || !ws) return TRAKHIP_ERR_NULL;
-    if (ws_bytes < project_workspace_bytes(B, P, k, num_feature_tiles)) return TRAKHIP_ERR_WORKSPACE;
+    if (ws_bytes < project_workspace_min_bytes(B, P, k, num_feature_tiles)) return TRAKHIP_ERR_WORKSPACE;
     const size_t esz = dtype == TRAKHIP_F32 ? 4 : 2;
     if ((reinterpret_cast<uintptr_t>(in) % esz) || (reinterpret_cast<uintptr_t>(ws) % 16)) return TRAKHIP_ERR_ALIGN;
     return TRAKHIP_OK;
@@ -1148,7 +1198,8 @@ int project_partials(const void* in, int dtype, uint64_t B, uint64_t P, uint64_t
                      uint32_t k, uint32_t seed, uint32_t num_feature_tiles, int proj_type, hipStream_t s) {
     const int e = check_project_args(in, dtype, B, P, ld, ws, ws_bytes, k, num_feature_tiles, proj_type);
     if (e) return e;
-    if (B > 32) return TRAKHIP_ERR_SHAPE;
+    if (B > project_rows_per_pass(dtype, proj_type)) return TRAKHIP_ERR_SHAPE;
+    if (ws_bytes < workspace_for_rows(B, P, k, num_feature_tiles, 64)) return TRAKHIP_ERR_WORKSPACE;
     const Plan pl = make_plan(P, k, num_feature_tiles);
     if (pick(pl, dtype, proj_type, false)(in, ld, (uint32_t)B, P, k, seed, pl, static_cast<float*>(ws), s) != hipSuccess)
         return TRAKHIP_ERR_LAUNCH;
@@ -1161,7 +1212,8 @@ int project_gather_partials(const trakhip_segment* segs, uint32_t n_segs, int dt
     // segs is device memory: its contents (sorted, contiguous, covering [0, P)) are the caller's contract
     const int e = check_project_args(segs, dtype, B, P, P, ws, ws_bytes, k, num_feature_tiles, proj_type);
     if (e) return e;
-    if (B > 32 || n_segs == 0) return TRAKHIP_ERR_SHAPE;
+    if (B > project_rows_per_pass(dtype, proj_type) || n_segs == 0) return TRAKHIP_ERR_SHAPE;
+    if (ws_bytes < workspace_for_rows(B, P, k, num_feature_tiles, 64)) return TRAKHIP_ERR_WORKSPACE;
     if (reinterpret_cast<uintptr_t>(segs) % 8) return TRAKHIP_ERR_ALIGN;
     const Plan pl = make_plan(P, k, num_feature_tiles);
     if (pick(pl, dtype, proj_type, true)(segs, n_segs, (uint32_t)B, P, k, seed, pl, static_cast<float*>(ws), s) !=
@@ -1174,7 +1226,7 @@ int project_reduce_store(const void* ws, uint64_t B, uint64_t P, uint32_t k, uin
                          float scale, int out_dtype, void* out, uint64_t ld_out, hipStream_t s,
                          bool check_destination) {
     if (k == 0 || k % kColsMultiple != 0) return TRAKHIP_ERR_PROJ_DIM;
-    if (B == 0 || B > 32 || P == 0 || P > 0xFFFFFFFFull || num_feature_tiles == 0 || ld_out < k)
+    if (B == 0 || B > 64 || P == 0 || P > 0xFFFFFFFFull || num_feature_tiles == 0 || ld_out < k)
         return TRAKHIP_ERR_SHAPE;
     if (out_dtype != TRAKHIP_F16 && out_dtype != TRAKHIP_BF16 && out_dtype != TRAKHIP_F32) return TRAKHIP_ERR_DTYPE;
     if (!ws || !out) return TRAKHIP_ERR_NULL;
@@ -1209,9 +1261,12 @@ int project(const void* in, int dtype, uint64_t B, uint64_t P, uint64_t ld, floa
     if (!out) return TRAKHIP_ERR_NULL;
     if (reinterpret_cast<uintptr_t>(out) % 16) return TRAKHIP_ERR_ALIGN;
     const size_t esz = dtype == TRAKHIP_F32 ? 4 : 2;
-    // rows are walked 32 at a time (the reference walks 8, 16 or 32 at a time: fast_jl/fast_jl.cu:44-76)
-    for (uint64_t b0 = 0; b0 < B; b0 += 32) {
-        const uint64_t rows = (B - b0) < 32 ? (B - b0) : 32;
+    // rows are walked 64 or 32 at a time (the reference walks 8, 16 or 32 at a time: fast_jl/fast_jl.cu:44-76);
+    // a workspace sized for 32-row passes only is accepted and used that way
+    uint64_t pass = project_rows_per_pass(dtype, proj_type);
+    if (pass > 32 && ws_bytes < workspace_for_rows(B, P, k, num_feature_tiles, pass)) pass = 32;
+    for (uint64_t b0 = 0; b0 < B; b0 += pass) {
+        const uint64_t rows = (B - b0) < pass ? (B - b0) : pass;
         const char* src = static_cast<const char*>(in) + b0 * ld * esz;
         int r = project_partials(src, dtype, rows, P, ld, ws, ws_bytes, k, seed, num_feature_tiles, proj_type, s);
         if (!r) r = project_reduce(ws, rows, P, k, num_feature_tiles, 1.0f, out + b0 * k, s);
@@ -1253,7 +1308,7 @@ int project_static(const void* in, int dtype, uint64_t B, uint64_t P, uint64_t l
     if (e) return e;
     if (!out) return TRAKHIP_ERR_NULL;
     if (reinterpret_cast<uintptr_t>(out) % 16) return TRAKHIP_ERR_ALIGN;
-    if (project_workspace_bytes(B, P, k, num_feature_tiles) > kStaticScratchBytes) return TRAKHIP_ERR_STATIC_LIMIT;
+    if (project_workspace_min_bytes(B, P, k, num_feature_tiles) > kStaticScratchBytes) return TRAKHIP_ERR_STATIC_LIMIT;
     void* ws = nullptr;
     const int d = static_scratch(&ws);
     if (d) return d;

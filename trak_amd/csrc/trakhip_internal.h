@@ -9,6 +9,8 @@
 namespace trakhip {
 
 size_t project_workspace_bytes(uint64_t B, uint64_t P, uint32_t k, uint32_t num_feature_tiles);
+size_t project_workspace_min_bytes(uint64_t B, uint64_t P, uint32_t k, uint32_t num_feature_tiles);
+uint32_t project_rows_per_pass(int dtype, int proj_type);
 int project(const void* in, int dtype, uint64_t B, uint64_t P, uint64_t ld, float* out, void* ws,
             size_t ws_bytes, uint32_t k, uint32_t seed, uint32_t num_feature_tiles, int proj_type,
             hipStream_t s);

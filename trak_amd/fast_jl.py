@@ -2,8 +2,8 @@
 
 `project_{rademacher,normal}_{8,16,32}(input, N, seed, num_feature_tiles) -> Tensor`
 (fast_jl/fast_jl.cu:81-110).  The numeric suffix is the number of rows the reference
-processes per kernel launch; here every variant walks the batch in groups of 32 rows and
-the suffix does not change the result.
+processes per kernel launch; here every variant walks the batch in passes of 64 rows (16-bit
+gradients, Rademacher) or 32 rows and the suffix does not change the result.
 """
 import ctypes
 
@@ -189,8 +189,9 @@ def project_into(source, N, seed, num_feature_tiles, proj_type, out, scale=1.0):
         nbytes = lib.trakhip_project_workspace(B, P, N, tiles)
         ws = _workspace(device, nbytes)
         stream = torch.cuda.current_stream(device).cuda_stream
-        for b0 in range(0, B, 32):
-            nb = min(32, B - b0)
+        step = int(lib.trakhip_project_rows_per_pass(_DTYPES[dtype], pt))
+        for b0 in range(0, B, step):
+            nb = min(step, B - b0)
             if rows is None:
                 code = lib.trakhip_project_partials(
                     ctypes.c_void_p(source.data_ptr() + b0 * ld * esz), _DTYPES[dtype], nb, P, ld,
