@@ -463,8 +463,6 @@ __global__ __launch_bounds__(512) void jl_project_kernel(
     if (c_begin >= total_chunks) return;  // padding of the group count to a multiple of 8
     const uint64_t c_end = c_begin + chunks_per_group < total_chunks ? c_begin + chunks_per_group : total_chunks;
     const uint32_t t0 = (uint32_t)(c_begin / chunks_per_tile), s0 = (uint32_t)(c_begin % chunks_per_tile);
-    const uint32_t t_last = (uint32_t)((c_end - 1) / chunks_per_tile);
-    const uint32_t s_last_end = (uint32_t)((c_end - 1) % chunks_per_tile) + 1;
 
     const int tid = threadIdx.x;
     const int wave = tid >> 6, lane = tid & 63;
@@ -1053,8 +1051,7 @@ __global__ __launch_bounds__(256) void jl_reduce_kernel(const float* __restrict_
 }
 
 // S[f0 + i, c0 + j] for i < nf, j < nc, written as binary32, row-major [nf, nc].
-__global__ __launch_bounds__(256) void jl_materialize_kernel(uint32_t seed, uint32_t tiles,
-                                                             uint64_t tile_size, uint64_t f0,
+__global__ __launch_bounds__(256) void jl_materialize_kernel(uint32_t seed, uint64_t tile_size, uint64_t f0,
                                                              uint64_t nf, uint32_t c0, uint32_t nc,
                                                              int proj_type, float* __restrict__ out) {
     const uint64_t idx = (uint64_t)blockIdx.x * 256 + threadIdx.x;
@@ -1327,7 +1324,7 @@ int materialize_device(uint32_t seed, uint32_t num_feature_tiles, uint64_t P, ui
     const uint64_t total = nf * nc;
     if ((total + 255) / 256 > 0x7FFFFFFFull) return TRAKHIP_ERR_SHAPE;
     hipLaunchKernelGGL(jl_materialize_kernel, dim3((uint32_t)((total + 255) / 256)), dim3(256), 0, s, seed,
-                       tl.tiles, tl.tile_size, f0, nf, c0, nc, proj_type, out);
+                       tl.tile_size, f0, nf, c0, nc, proj_type, out);
     return hipGetLastError() == hipSuccess ? TRAKHIP_OK : TRAKHIP_ERR_LAUNCH;
 }
 
