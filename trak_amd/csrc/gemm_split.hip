@@ -368,7 +368,7 @@ __global__ __launch_bounds__(64 * kWaves, 2) void gemm_split_kernel(
     // a symmetric product needs only the tiles that touch the lower triangle
     if ((flags & trakhip::kGemmLowerTilesOnly) && n0 > m0 + BM - 1) return;
     const int tid = threadIdx.x;
-    const int wave = tid >> 6, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;  // the wave number as a scalar
     const int wm = wave / kWavesN, wn = wave % kWavesN;
     const int x = lane & 31, h = lane >> 5;
 
