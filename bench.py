@@ -16,7 +16,7 @@ cpu_baseline = the CPU restatement of trak's BasicProjector (oracle/basic_projec
 sustained = the same calls back to back for --sustain seconds (default 2).
 `scoring` = BasicScoreComputer at N=50_000, M=10_000, k=4096 fp32: GEMM TFLOP/s against the fp32
             MFMA peak, the SPD inverse separately, and a CPU sample beside it.
-`--only NAME` runs one workload alone (for profiler runs): c1 | c2 | c3_b64 | c3_dict | c4 | c4_rademacher | vendor_gemm |
+`--only NAME` runs one workload alone (for profiler runs): c1 | c2 | c3_b64 | c3_normal_b32 | c3_normal_b64 | c3_dict | c4 | c4_rademacher | vendor_gemm |
             scoring | mfma_rate.
 """
 import argparse
@@ -267,6 +267,12 @@ def _config_calls(torch, dev, name):
         g = (torch.randn(64, P, generator=gen, device=dev) * 1e-3).half()
         p = CudaProjector(P, 4096, 7, ProjectionType.rademacher, dev, 32)
         return (lambda: p.project(g, 0)), 2.0 * 64 * P * 4096, "fp16 rademacher [64,11689512] -> 4096 (one pass of 64 rows)"
+    if name in ("c3_normal_b32", "c3_normal_b64"):
+        B = int(name[-2:])
+        P = sum(math.prod(sh) for sh in resnet18_param_shapes())
+        g = (torch.randn(B, P, generator=gen, device=dev) * 1e-3).bfloat16()
+        p = CudaProjector(P, 4096, 7, ProjectionType.normal, dev, 32)
+        return (lambda: p.project(g, 0)), 2.0 * B * P * 4096, f"bf16 normal [{B},11689512] -> 4096 (one pass)"
     if name == "c3_dict":
         shapes = resnet18_param_shapes()
         P = sum(math.prod(sh) for sh in shapes)
@@ -616,7 +622,7 @@ def main():
                     help="also time the other projection configurations and print them to stderr")
     ap.add_argument("--only", default=None, metavar="NAME",
                     help="run just one workload for --steps calls and print its timing (for profiler runs): "
-                         "c1 | c2 | c3_b64 | c3_dict | c4 | c4_rademacher | scoring | mfma_rate | vendor_gemm "
+                         "c1 | c2 | c3_b64 | c3_normal_b32 | c3_normal_b64 | c3_dict | c4 | c4_rademacher | scoring | mfma_rate | vendor_gemm "
                          "(torch.mm on the scoring operands, for comparison)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run one 1 GiB device-to-device copy (reference point for rocprofv3 byte counters)")

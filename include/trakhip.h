@@ -60,9 +60,9 @@ int trakhip_abi_version(void);
 size_t trakhip_project_workspace(uint64_t B, uint64_t P, uint32_t proj_dim, uint32_t num_feature_tiles);
 size_t trakhip_project_workspace_min(uint64_t B, uint64_t P, uint32_t proj_dim, uint32_t num_feature_tiles);
 
-/* Rows that one pass of the projection kernel takes: 64 for fp16 / bf16 gradients under a Rademacher
- * matrix (two 32-row MFMA blocks share every generated matrix entry), 32 otherwise.  The reference
- * has passes of 8, 16 or 32 rows (fast_jl/fast_jl.cu:44-76). */
+/* Rows that one pass of the projection kernels takes: 64 for fp16 / bf16 gradients (two 32-row MFMA
+ * blocks share every generated matrix entry, Rademacher or normal), 32 for fp32 gradients.  The
+ * reference has passes of 8, 16 or 32 rows (fast_jl/fast_jl.cu:44-76). */
 uint32_t trakhip_project_rows_per_pass(int in_dtype, int proj_type);
 
 /* out[B, proj_dim] (fp32) = in[B, P] x S, S generated on the fly from (seed, proj_dim,

@@ -85,7 +85,7 @@ def test_workspace_size():
     F16, BF16, F32 = _lib.F16, _lib.BF16, _lib.F32
     rpp = lib.trakhip_project_rows_per_pass
     assert rpp(F16, _lib.RADEMACHER) == 64 and rpp(BF16, _lib.RADEMACHER) == 64 and rpp(F32, _lib.RADEMACHER) == 32
-    assert rpp(F16, _lib.NORMAL) == 32 and rpp(BF16, _lib.NORMAL) == 32 and rpp(F32, _lib.NORMAL) == 32
+    assert rpp(F16, _lib.NORMAL) == 64 and rpp(BF16, _lib.NORMAL) == 64 and rpp(F32, _lib.NORMAL) == 32
     assert lib.trakhip_project_workspace(8, 25, 1024, 256) == 25 * 8 * 1024 * 4
     assert lib.trakhip_project_workspace(16, 1_048_576, 512, 256) == 256 * 16 * 512 * 4  # one 512-column block
     assert lib.trakhip_project_workspace(0, 25, 1024, 256) == 0

@@ -74,7 +74,8 @@ def test_one_hot_rows_read_the_matrix_back_exactly(gpu, c_oracle, proj_type, dty
 @pytest.mark.parametrize(
     "B,P,k,tiles",
     [(32, 20_000, 512, 256), (16, 10_002, 1024, 256), (9, 10_001, 512, 108), (1, 25, 512, 256), (45, 1049, 512, 256),
-     (8, 70_001, 512, 7), (32, 9_000, 1536, 256), (12, 5_003, 2048, 64), (32, 6_001, 2560, 256)],
+     (8, 70_001, 512, 7), (32, 9_000, 1536, 256), (12, 5_003, 2048, 64), (32, 6_001, 2560, 256),
+     (64, 4_100, 1024, 16), (50, 3_001, 512, 5)],
 )
 def test_projection_matches_float64_contraction(gpu, c_oracle, proj_type, dtype, B, P, k, tiles):
     gen = torch.Generator(device="cpu").manual_seed(1000 + B + P)
@@ -112,13 +113,15 @@ def test_tiny_values_and_exact_zeros(gpu, c_oracle, dtype):
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
-@pytest.mark.parametrize("k", [512, 1024])
-def test_normal_projection_follows_the_rows_scale_from_chunk_to_chunk(gpu, c_oracle, dtype, k):
+@pytest.mark.parametrize("k,B", [(512, 23), (1024, 23), (512, 55), (1024, 64)])
+def test_normal_projection_follows_the_rows_scale_from_chunk_to_chunk(gpu, c_oracle, dtype, k, B):
     # The normal kernel brings every 256-feature chunk of a row to fp16 with the row's own power of two
     # and carries the accumulators from one chunk's factor to the next.  Blocks of features whose sizes
     # differ by up to 2^±80 (far outside fp16), rows of different magnitude, all-zero stretches and
     # rows that are zero throughout must all come out as the float64 contraction says.
-    B, P, tiles, seed = 23, 9_000, 7, 31
+    # More than 32 rows of a 16-bit dtype go through the kernel 64 at a time (two 32-row blocks with their
+    # own exponent lists); the special rows are repeated in the second block.
+    P, tiles, seed = 9_000, 7, 31
     gen = torch.Generator(device="cpu").manual_seed(12)
     expo = torch.randint(-80, 81, (P // 300,), generator=gen).double()
     expo[::7] = 0
@@ -135,6 +138,11 @@ def test_normal_projection_follows_the_rows_scale_from_chunk_to_chunk(gpu, c_ora
     g[9, :256] = torch.randn(256, generator=gen).double() * 2.0 ** 90
     g[10] = torch.randn(P, generator=gen).double() * 2.0 ** -90
     g[10, P - 256 :] = torch.randn(256, generator=gen).double() * 2.0 ** 90
+    if B > 50:
+        g[37], g[41] = 0.0, g[9]
+        g[39, :] = 0.0
+        g[39, 8999] = -3.0
+        g[50] = g[10]
     g = g.to(dtype)
     assert torch.isfinite(g).all()
     out = fn(G)(g.to(gpu), k, seed, tiles)
@@ -147,6 +155,13 @@ def test_normal_projection_follows_the_rows_scale_from_chunk_to_chunk(gpu, c_ora
     # the one-hot row reads the matrix row back exactly (3 * entry is exact in fp32)
     s_row = c_oracle.materialize(seed, tiles, P, 4321, 1, 0, k, G)[0]
     assert np.array_equal(out[7].cpu().numpy(), 3.0 * s_row)
+    if B > 50:
+        assert not live[37] and not got[37].any()
+        assert torch.equal(out[41], out[9]) and torch.equal(out[50], out[10])
+        assert np.array_equal(out[39].cpu().numpy(), -3.0 * c_oracle.materialize(seed, tiles, P, 8999, 1, 0, k, G)[0])
+        # a row's result does not depend on the rows it shares a pass with
+        assert torch.equal(fn(G)(g[:32].to(gpu), k, seed, tiles), out[:32])
+        assert torch.equal(fn(G)(g[32:].to(gpu), k, seed, tiles), out[32:])
     # scaling a row by a power of two scales its projection exactly
     g2 = g.clone()
     g2[3] *= 2.0 ** 9

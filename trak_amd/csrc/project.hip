@@ -731,19 +731,23 @@ __device__ __forceinline__ RowScale next_row_scale(uint32_t emax, int& ref) {
 
 // Slot of row m in the per-chunk exponent lists: lane half h reads its sixteen accumulator rows
 // m = 8*(r/4) + 4*h + r%4 (r = 0..15) as sixteen consecutive ints.
-__device__ __forceinline__ int row_slot(uint32_t row) { return ((row >> 2) & 1) * 16 + (row >> 3) * 4 + (row & 3); }
+__device__ __forceinline__ int row_slot(uint32_t row) {
+    return (int)(row & ~31u) + ((row >> 2) & 1) * 16 + ((row & 31u) >> 3) * 4 + (row & 3);  // 32-row blocks one after another
+}
 
 __device__ __forceinline__ uint32_t pack_f16_rne(float a, float b) {
     const half2_t v = {(_Float16)a, (_Float16)b};
     return __builtin_bit_cast(uint32_t, v);
 }
 
-// bf16 chunk -> one scaled fp16 plane.  The 32 threads that share tid / 32 hold one row (two rows
-// per thread, 16 apart); sh_ref[] is the row's reference exponent so far.
-__device__ __forceinline__ void store_scaled_bf16(const uint4 (&v)[2], uint16_t* lds, int (*sh)[32], int tid,
-                                                  int (&sh_ref)[2]) {
+// bf16 chunk -> one scaled fp16 plane.  The 32 threads that share tid / 32 hold one row (N rows
+// per thread, 16 apart); sh_ref[] is the row's reference exponent so far; sh_delta / sh_use are the
+// per-row lists of this buffer (16 N entries each).
+template <int N>
+__device__ __forceinline__ void store_scaled_bf16(const uint4 (&v)[N], uint16_t* lds, int* sh_delta, int* sh_use,
+                                                  int tid, int (&sh_ref)[N]) {
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
+    for (int i = 0; i < N; ++i) {
         const uint32_t row = (tid >> 5) + 16 * i, sg = tid & 31;
         const uint32_t w[4] = {v[i].x, v[i].y, v[i].z, v[i].w};
         ushort2_t m = __builtin_bit_cast(ushort2_t, w[0] & 0x7F807F80u);
@@ -763,15 +767,15 @@ __device__ __forceinline__ void store_scaled_bf16(const uint4 (&v)[2], uint16_t*
                                 ldexpf(__uint_as_float(w[t] & 0xFFFF0000u), rs.use));
         *reinterpret_cast<uint4*>(lds + row * kLdsRow + 8 * sg) = uint4{h[0], h[1], h[2], h[3]};
         if (sg == 0) {
-            sh[0][row_slot(row)] = rs.delta;
-            sh[1][row_slot(row)] = rs.use;
+            sh_delta[row_slot(row)] = rs.delta;
+            sh_use[row_slot(row)] = rs.use;
         }
     }
 }
 
 // fp32 chunk -> two scaled fp16 planes.  The 64 threads of a wave hold one row (four rows per
 // thread, 8 apart).
-__device__ __forceinline__ void store_scaled_f32(const uint4 (&v)[4], uint16_t* lds, int (*sh)[32], int tid,
+__device__ __forceinline__ void store_scaled_f32(const uint4 (&v)[4], uint16_t* lds, int* sh_delta, int* sh_use, int tid,
                                                  int (&sh_ref)[4]) {
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
@@ -803,8 +807,8 @@ __device__ __forceinline__ void store_scaled_f32(const uint4 (&v)[4], uint16_t* 
         *reinterpret_cast<uint2*>(lds + kPlaneElems + row * kLdsRow + 4 * sg) =
             uint2{pack_f16_rne(r[0], r[1]), pack_f16_rne(r[2], r[3])};
         if (sg == 0) {
-            sh[0][row_slot(row)] = rs.delta;
-            sh[1][row_slot(row)] = rs.use;
+            sh_delta[row_slot(row)] = rs.delta;
+            sh_use[row_slot(row)] = rs.use;
         }
     }
 }
@@ -822,32 +826,38 @@ __device__ __forceinline__ uint32_t normal_pair(uint32_t w, const char* r_tab, c
 }
 
 // GPW = 32-column groups per wave: 4 (workgroup = 1024 columns) or 2 (512 columns, for projection
-// dimensions that are an odd multiple of 512).  Always 8 waves; arguments as jl_project_kernel.
-template <int IN, bool GATHER, int GPW>
-__global__ __launch_bounds__(512, 2) void jl_project_normal_kernel(
+// dimensions that are an odd multiple of 512).  RB = 32-row blocks per pass: 2 for fp16 / bf16 gradients
+// when the batch has more than 32 rows - every generated entry then feeds two MFMAs, which is worth
+// almost a factor of two to a kernel bound by the cost of making an entry (one LDS buffer then: two
+// do not fit next to the tables).  Always 8 waves; arguments as jl_project_kernel.
+template <int IN, bool GATHER, int GPW, int RB>
+__global__ __launch_bounds__(512) void jl_project_normal_kernel(
     const void* __restrict__ g_in, uint64_t ld, uint32_t rows, uint64_t P, uint32_t k, uint32_t seed,
     uint32_t tiles, uint64_t tile_size, uint32_t chunks_per_tile, uint32_t chunks_per_group,
     float* __restrict__ partial) {
     constexpr int W = 8;
     typedef NormalTraits<IN> Tr;
-    typedef typename StageOf<IN, GATHER, W>::type Stage;
-    typedef typename StageOf<IN, GATHER, W>::elem Elem;
+    typedef typename StageOf<IN, GATHER, W, 32 * RB>::type Stage;
+    typedef typename StageOf<IN, GATHER, W, 32 * RB>::elem Elem;
     constexpr int kColsPerWG = W * GPW * 32;
     constexpr int kPlanes = Tr::planes;
-    constexpr int kBuffers = Tr::buffers;
+    static_assert(RB == 1 || kPlanes == 1, "two row blocks: 16-bit gradients only (LDS)");
+    constexpr int kBuffers = RB == 2 ? 1 : Tr::buffers;
+    constexpr int kPlaneElems = RB * kPlaneElems32;  // this kernel's plane: 32 RB rows
     constexpr int kBufElems = kPlanes * kPlaneElems;
     constexpr bool kScaled = Tr::scaled;
+    constexpr int kRows = 32 * RB;
 
     // One LDS block, tables first: a DS instruction adds a 16-bit immediate to the address register,
     // so a table that starts below 64 KB is indexed without an extra addition per lookup.
     constexpr int kCsBytes = kAngleEntries * 4, kRBytes = kRadiusEntries * 2;
     constexpr int kStageBytes = kBuffers * kBufElems * 2;
-    __shared__ __attribute__((aligned(16))) char smem[kCsBytes + kRBytes + kStageBytes + kBuffers * 2 * 32 * 4];
+    __shared__ __attribute__((aligned(16))) char smem[kCsBytes + kRBytes + kStageBytes + kBuffers * 2 * kRows * 4];
     uint32_t* cs_tab = reinterpret_cast<uint32_t*>(smem);
     uint16_t* r_tab = reinterpret_cast<uint16_t*>(smem + kCsBytes);
     uint16_t* lds = reinterpret_cast<uint16_t*>(smem + kCsBytes + kRBytes);
     // per buffer and row: change of the row's exponent against the previous chunk, and the exponent
-    int (*sh_lds)[2][32] = reinterpret_cast<int (*)[2][32]>(smem + kCsBytes + kRBytes + kStageBytes);
+    int (*sh_lds)[2][kRows] = reinterpret_cast<int (*)[2][kRows]>(smem + kCsBytes + kRBytes + kStageBytes);
 
     const uint32_t col_blocks = k / kColsPerWG;
     uint32_t cb, group;
@@ -875,14 +885,16 @@ __global__ __launch_bounds__(512, 2) void jl_project_normal_kernel(
     const char* rt = reinterpret_cast<const char*>(r_tab);
     const char* ct = reinterpret_cast<const char*>(cs_tab);
 
-    floatx16 acc[GPW];
+    floatx16 acc[RB][GPW];
 #pragma unroll
-    for (int j = 0; j < GPW; ++j)
+    for (int rb = 0; rb < RB; ++rb)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) acc[j][r] = 0.0f;
+        for (int j = 0; j < GPW; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[rb][j][r] = 0.0f;
 
     const Elem* g = reinterpret_cast<const Elem*>(g_in);
-    const uint32_t a_off = n * kLdsRow + 128 * h;
+    const uint32_t a_off = n * kLdsRow + 128 * h;  // row block rb: + 32 rb rows
 
     Stage st;
     int sh_ref[Stage::N];
@@ -892,9 +904,9 @@ __global__ __launch_bounds__(512, 2) void jl_project_normal_kernel(
         if constexpr (IN == TRAKHIP_F16)
             st.store(lds + buf * kBufElems, tid);
         else if constexpr (IN == TRAKHIP_BF16)
-            store_scaled_bf16(st.v, lds + buf * kBufElems, sh_lds[buf], tid, sh_ref);
+            store_scaled_bf16(st.v, lds + buf * kBufElems, sh_lds[buf][0], sh_lds[buf][1], tid, sh_ref);
         else
-            store_scaled_f32(st.v, lds + buf * kBufElems, sh_lds[buf], tid, sh_ref);
+            store_scaled_f32(st.v, lds + buf * kBufElems, sh_lds[buf][0], sh_lds[buf][1], tid, sh_ref);
     };
     {
         const uint64_t lo = (uint64_t)t0 * tile_size;
@@ -935,34 +947,41 @@ __global__ __launch_bounds__(512, 2) void jl_project_normal_kernel(
 
             if (kScaled) {
                 // rows whose reference exponent moved with this chunk: bring their sums along (down only)
-                const int4* dp = reinterpret_cast<const int4*>(&sh_lds[cur][0][16 * h]);
-                int d[16];
 #pragma unroll
-                for (int t = 0; t < 4; ++t) {
-                    const int4 x = dp[t];
-                    d[4 * t] = x.x, d[4 * t + 1] = x.y, d[4 * t + 2] = x.z, d[4 * t + 3] = x.w;
+                for (int rb = 0; rb < RB; ++rb) {
+                    const int4* dp = reinterpret_cast<const int4*>(&sh_lds[cur][0][32 * rb + 16 * h]);
+                    int d[16];
+#pragma unroll
+                    for (int t = 0; t < 4; ++t) {
+                        const int4 x = dp[t];
+                        d[4 * t] = x.x, d[4 * t + 1] = x.y, d[4 * t + 2] = x.z, d[4 * t + 3] = x.w;
+                    }
+#pragma unroll
+                    for (int j = 0; j < GPW; ++j)
+#pragma unroll
+                        for (int r = 0; r < 16; ++r) acc[rb][j][r] = ldexpf(acc[rb][j][r], d[r]);
                 }
-#pragma unroll
-                for (int j = 0; j < GPW; ++j)
-#pragma unroll
-                    for (int r = 0; r < 16; ++r) acc[j][r] = ldexpf(acc[j][r], d[r]);
             }
 
             // Philox block of (column, offset o): o / 8 with o = 256 s + 128 h + 8 q
             const uint32_t n0 = 32u * s + 16u * h;
 #pragma unroll kNormalUnroll
             for (int q = 0; q < 16; ++q) {
-                uint4 a[kPlanes];
+                uint4 a[RB][kPlanes];
 #pragma unroll
-                for (int pl = 0; pl < kPlanes; ++pl)
-                    a[pl] = *reinterpret_cast<const uint4*>(a_base + pl * kPlaneElems + 8 * q);
+                for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+                    for (int pl = 0; pl < kPlanes; ++pl)
+                        a[rb][pl] = *reinterpret_cast<const uint4*>(a_base + rb * 32 * kLdsRow + pl * kPlaneElems + 8 * q);
 #pragma unroll
                 for (int j = 0; j < GPW; ++j) {
                     const jl::u32x4 blk = jl::stream_block(seed, sname[j], n0 + (uint32_t)q);
                     const uint4 b = {normal_pair(blk.x, rt, ct), normal_pair(blk.y, rt, ct),
                                      normal_pair(blk.z, rt, ct), normal_pair(blk.w, rt, ct)};
 #pragma unroll
-                    for (int pl = 0; pl < kPlanes; ++pl) acc[j] = mfma16(a[pl], b, acc[j], false);
+                    for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+                        for (int pl = 0; pl < kPlanes; ++pl) acc[rb][j] = mfma16(a[rb][pl], b, acc[rb][j], false);
                 }
             }
 
@@ -976,23 +995,27 @@ __global__ __launch_bounds__(512, 2) void jl_project_normal_kernel(
     }
 
     float* out = partial + (uint64_t)group * rows * k;
-    int ex[16];
 #pragma unroll
-    for (int r = 0; r < 16; ++r) ex[r] = 0;
-    if (kScaled) {
-        const int4* ep = reinterpret_cast<const int4*>(&sh_lds[last][1][16 * h]);
+    for (int rb = 0; rb < RB; ++rb) {
+        int ex[16];
 #pragma unroll
-        for (int t = 0; t < 4; ++t) {
-            const int4 x = ep[t];
-            ex[4 * t] = x.x, ex[4 * t + 1] = x.y, ex[4 * t + 2] = x.z, ex[4 * t + 3] = x.w;
+        for (int r = 0; r < 16; ++r) ex[r] = 0;
+        if (kScaled) {
+            const int4* ep = reinterpret_cast<const int4*>(&sh_lds[last][1][32 * rb + 16 * h]);
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+                const int4 x = ep[t];
+                ex[4 * t] = x.x, ex[4 * t + 1] = x.y, ex[4 * t + 2] = x.z, ex[4 * t + 3] = x.w;
+            }
         }
-    }
 #pragma unroll
-    for (int j = 0; j < GPW; ++j) {
+        for (int j = 0; j < GPW; ++j) {
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-            const uint32_t m = 8u * (r >> 2) + 4u * h + (r & 3);
-            if (m < rows) out[(uint64_t)m * k + col0 + 32u * j] = kScaled ? ldexpf(acc[j][r], -ex[r]) : acc[j][r];
+            for (int r = 0; r < 16; ++r) {
+                const uint32_t m = 32u * rb + 8u * (r >> 2) + 4u * h + (r & 3);
+                if (m < rows)
+                    out[(uint64_t)m * k + col0 + 32u * j] = kScaled ? ldexpf(acc[rb][j][r], -ex[r]) : acc[rb][j][r];
+            }
         }
     }
 }
@@ -1117,9 +1140,19 @@ hipError_t launch_normal(const void* in, uint64_t ld, uint32_t rows, uint64_t P,
     const uint32_t groups8 = (pl.groups + 7u) / 8u * 8u;
     const uint64_t wgs = (uint64_t)groups8 * pl.col_blocks;
     if (wgs > 0x7FFFFFFFull) return hipErrorInvalidValue;
-    hipLaunchKernelGGL((jl_project_normal_kernel<IN, GATHER, GPW>), dim3((uint32_t)wgs), dim3(512), 0, s, in, ld,
-                       rows, P, k, seed, pl.tl.tiles, pl.tl.tile_size, pl.chunks_per_tile, pl.chunks_per_group,
-                       partial);
+    if (rows > 32) {
+        if constexpr (IN == TRAKHIP_F32) {
+            return hipErrorInvalidValue;
+        } else {
+            hipLaunchKernelGGL((jl_project_normal_kernel<IN, GATHER, GPW, 2>), dim3((uint32_t)wgs), dim3(512), 0, s, in,
+                               ld, rows, P, k, seed, pl.tl.tiles, pl.tl.tile_size, pl.chunks_per_tile,
+                               pl.chunks_per_group, partial);
+        }
+    } else {
+        hipLaunchKernelGGL((jl_project_normal_kernel<IN, GATHER, GPW, 1>), dim3((uint32_t)wgs), dim3(512), 0, s, in, ld,
+                           rows, P, k, seed, pl.tl.tiles, pl.tl.tile_size, pl.chunks_per_tile, pl.chunks_per_group,
+                           partial);
+    }
     return hipGetLastError();
 }
 
@@ -1154,10 +1187,11 @@ static std::atomic<void*> static_scratch_ptr[kMaxDevices];
 
 namespace trakhip {
 
-// Rows of one pass of the projection kernel: 16-bit gradients under a Rademacher matrix go 64 rows at a
-// time (two 32-row MFMA blocks share every generated operand), everything else 32.
+// Rows of one pass of the projection kernels: 16-bit gradients go 64 rows at a time (two 32-row MFMA
+// blocks share every generated operand), fp32 gradients 32 (their planes do not fit twice in LDS).
 uint32_t project_rows_per_pass(int dtype, int proj_type) {
-    return (dtype == TRAKHIP_F16 || dtype == TRAKHIP_BF16) && proj_type == TRAKHIP_RADEMACHER ? 64u : 32u;
+    (void)proj_type;
+    return dtype == TRAKHIP_F16 || dtype == TRAKHIP_BF16 ? 64u : 32u;
 }
 
 static size_t workspace_for_rows(uint64_t B, uint64_t P, uint32_t k, uint32_t num_feature_tiles, uint64_t pass_rows) {

@@ -3,7 +3,7 @@
 `project_{rademacher,normal}_{8,16,32}(input, N, seed, num_feature_tiles) -> Tensor`
 (fast_jl/fast_jl.cu:81-110).  The numeric suffix is the number of rows the reference
 processes per kernel launch; here every variant walks the batch in passes of 64 rows (16-bit
-gradients, Rademacher) or 32 rows and the suffix does not change the result.
+gradients) or 32 rows (fp32) and the suffix does not change the result.
 """
 import ctypes
 
