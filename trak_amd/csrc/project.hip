@@ -28,6 +28,7 @@
 #include <stdint.h>
 
 #include <atomic>
+#include <type_traits>
 
 #include "jl_stream.h"
 #include "store_cast.h"
@@ -93,18 +94,26 @@ struct Stage16 {
     static constexpr int kThreads = 64 * W;
     uint4 v[N];
 
+    // all ROWS rows and the whole chunk in range: unguarded 16-byte loads
+    __device__ __forceinline__ void load_whole(const uint16_t* __restrict__ g, uint64_t ld, uint64_t f_begin, int tid) {
+        const uint16_t* p = g + (uint64_t)(tid >> 5) * ld + f_begin + 8u * (tid & 31);
+#pragma unroll
+        for (int i = 0; i < N; ++i) {
+            const Raw16 r = *reinterpret_cast<const Raw16*>(p + (uint64_t)(2 * W * i) * ld);
+            v[i] = {r.x, r.y, r.z, r.w};
+        }
+    }
     __device__ __forceinline__ void load(const uint16_t* __restrict__ g, uint64_t ld, uint32_t rows,
                                          uint64_t f_begin, uint64_t f_end, int tid) {
-        if (rows == ROWS && f_begin + kChunk <= f_end) {
-            // whole chunk in range (uniform test): unguarded 16-byte loads
-            const uint16_t* p = g + (uint64_t)(tid >> 5) * ld + f_begin + 8u * (tid & 31);
-#pragma unroll
-            for (int i = 0; i < N; ++i) {
-                const Raw16 r = *reinterpret_cast<const Raw16*>(p + (uint64_t)(2 * W * i) * ld);
-                v[i] = {r.x, r.y, r.z, r.w};
-            }
+        if (rows == ROWS && f_begin + kChunk <= f_end) {  // uniform test
+            load_whole(g, ld, f_begin, tid);
             return;
         }
+        load_edge(g, ld, rows, f_begin, f_end, tid);
+    }
+    // rows beyond `rows` and features beyond f_end read as zero
+    __device__ __forceinline__ void load_edge(const uint16_t* __restrict__ g, uint64_t ld, uint32_t rows,
+                                              uint64_t f_begin, uint64_t f_end, int tid) {
 #pragma unroll
         for (int i = 0; i < N; ++i) {
             const int id = tid + kThreads * i;
@@ -493,47 +502,66 @@ __global__ __launch_bounds__(512) void jl_project_kernel(
     const uint32_t a_off = n * kLdsRow + 128 * h;  // row block rb: + 32 rb rows
     const uint32_t lane_base = (uint32_t)(lane & 15) << 4;
 
-    // Position (tile, chunk in tile) of a chunk of the run, and its feature range.
-    struct Pos {
-        uint32_t tile, s;
+    // Position of a chunk of the run: tile, chunk in tile, first feature, end of the tile's features and
+    // the number of chunks of the tile that lie wholly below that end.  Uniform values (scalar registers)
+    // that move from chunk to chunk with a few additions: the 64-bit products are redone only when the
+    // tile changes.  Every scalar instruction between the last MFMA of a chunk and the first of the next
+    // is paid for with about eight idle cycles of the matrix pipe (all waves are there at the same time).
+    struct Cursor {
+        uint32_t tile, s, whole;
+        uint64_t f, hi;
     };
-    auto step_pos = [&](Pos& p) {
-        if (++p.s == chunks_per_tile) {
-            p.s = 0;
-            ++p.tile;
+    auto open_tile = [&](Cursor& c) {
+        const uint64_t lo = (uint64_t)c.tile * tile_size;
+        c.hi = (lo + tile_size < P) ? lo + tile_size : P;  // may be <= lo (loads give zeros)
+        c.whole = c.hi > lo ? (uint32_t)((c.hi - lo) / kChunk) : 0u;
+        c.f = lo + (uint64_t)c.s * kChunk;
+    };
+    auto advance = [&](Cursor& c) {
+        if (++c.s == chunks_per_tile) {
+            c.s = 0;
+            ++c.tile;
+            open_tile(c);
+        } else {
+            c.f += kChunk;
         }
     };
-    auto load_chunk = [&](Stage& st, const Pos& p) {
-        const uint64_t lo = (uint64_t)p.tile * tile_size;
-        const uint64_t hi = (lo + tile_size < P) ? lo + tile_size : P;  // may be <= lo (loads give zeros)
-        st.load(g, ld, rows, lo + (uint64_t)p.s * kChunk, hi, tid);
+    const bool full_rows = rows == 32u * RB;
+    Stage st;
+    auto load_chunk = [&](const Cursor& c) {
+        if constexpr (!GATHER && kPlanes == 1) {
+            if (full_rows && c.s < c.whole)
+                st.load_whole(g, ld, c.f, tid);
+            else
+                st.load_edge(g, ld, rows, c.f, c.hi, tid);
+        } else {
+            st.load(g, ld, rows, c.f, c.hi, tid);
+        }
     };
     const uint32_t n_chunks = (uint32_t)(c_end - c_begin);
-    Pos p0 = {t0, s0}, p1 = p0;
-    step_pos(p1);
-    Pos p2 = p1;
-    step_pos(p2);
 
-    // Two sets of staging registers take turns: with two LDS buffers the loads of chunk i + 2 are
-    // issued at the top of chunk i and stored to LDS at the end of chunk i + 1, so a load has two
-    // chunk times (about 6 us) to arrive before a wave has to wait for it at the barrier.  With two row
-    // blocks the registers do not allow a second set: the loads of chunk i + 1 are issued at the top of
-    // chunk i (a chunk takes twice as long there).
-    constexpr bool kTwoSets = RB == 1;
-    Stage st_a, st_b_storage;
-    Stage& st_b = kTwoSets ? st_b_storage : st_a;
-    if constexpr (GATHER) {
-        const uint64_t first = (uint64_t)t0 * tile_size + (uint64_t)s0 * kChunk;
-        st_a.init(g, (uint32_t)ld, first, P, tid);
-        if (kTwoSets) st_b_storage.init(g, (uint32_t)ld, first, P, tid);
-    }
-    int cur = 0;
-    if (kBuffers == 2) {
-        load_chunk(st_a, p0);
-        st_a.store(lds, tid);
-        if (kTwoSets && n_chunks > 1) load_chunk(st_b, p1);
-    } else {
-        load_chunk(st_b, p0);
+    // Two LDS buffers (16-bit gradients): the chunk loop is one uninterrupted stream of steps.  Chunk
+    // i + 1 is stored to the other buffer in the middle of chunk i (it was loaded in the middle of chunk
+    // i - 1: one chunk time, about 2 us, in flight), the loads of chunk i + 2 follow the store into the
+    // same registers, the one barrier of the chunk stands in front of the first step of its last q -
+    // every wave has finished reading the current buffer by then, and the other one is published for the
+    // operand reads of the next chunk, which start right there: the rings of A and B operands run on
+    // across the chunk boundary.  One buffer (fp32 gradients): store between two barriers at the top of
+    // the chunk, the rings start anew.
+    constexpr bool kRing = kBuffers == 2;
+    constexpr int kSyncStep = 15 * GPW;
+    constexpr int kStoreStep = 10 * GPW, kLoadStep = kStoreStep + 1;
+    Cursor nx = {t0, s0, 0u, 0u, 0u};  // the chunk after the current one (tile and s: its generator blocks)
+    open_tile(nx);
+    Cursor ld2 = nx;                   // kRing: the chunk after that (the next one to load)
+    if constexpr (GATHER) st.init(g, (uint32_t)ld, nx.f, P, tid);
+    load_chunk(nx);
+    advance(nx);
+    if (kRing) {
+        st.store(lds, tid);
+        if (n_chunks > 1) load_chunk(nx);
+        ld2 = nx;
+        advance(ld2);
     }
     __syncthreads();  // publishes the table (and the first chunk)
 
@@ -545,71 +573,88 @@ __global__ __launch_bounds__(512) void jl_project_kernel(
         wd[j][0] = w.x, wd[j][1] = w.y, wd[j][2] = w.z, wd[j][3] = w.w;
     }
 
-    // chunk number i of the run; `fill` is loaded with a later chunk, `drain` goes to LDS
-    auto chunk = [&](uint32_t i, Stage& fill, Stage& drain) __attribute__((always_inline)) {
-        if (kBuffers == 1) {
+    uint4 bq[kAhead + 1];       // B operands (sign look-ups), read kAhead steps ahead
+    uint4 a[2][RB][kPlanes];    // A operands of this q and of the next one (read one q ahead)
+    auto read_a = [&](const uint16_t* base, int slot, int q) {
+#pragma unroll
+        for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+            for (int pl = 0; pl < kPlanes; ++pl)
+                a[slot][rb][pl] = *reinterpret_cast<const uint4*>(base + rb * 32 * kLdsRow + pl * kPlaneElems + 8 * q);
+    };
+    auto lookup = [&](uint32_t word, int q) -> uint4 {
+        return *reinterpret_cast<const uint4*>(smem + sign_entry_address(word, q, lane_base));
+    };
+    if (kRing) {
+#pragma unroll
+        for (int p = 0; p < kAhead; ++p) bq[p] = lookup(wd[p % GPW][0], p / GPW);
+        read_a(lds + a_off, 0, 0);
+    }
+
+    // chunk number i of the run; cur_c: its LDS buffer (a constant: immediate offsets in the DS instructions)
+    auto chunk = [&](uint32_t i, auto cur_c) __attribute__((always_inline)) {
+        constexpr int kCur = decltype(cur_c)::value;
+        if (!kRing) {
             __syncthreads();  // everyone is done reading the previous chunk
-            drain.store(lds, tid);
+            st.store(lds, tid);
             __syncthreads();
-            if (i + 1 < n_chunks) load_chunk(fill, p1);
-        } else if (kTwoSets) {
-            if (i + 2 < n_chunks) load_chunk(fill, p2);
-        } else {
-            if (i + 1 < n_chunks) load_chunk(fill, p1);
+            if (i + 1 < n_chunks) load_chunk(nx);
         }
-        const uint16_t* a_base = lds + cur * kBufElems + a_off;
+        const uint16_t* a_base = lds + kCur * kBufElems + a_off;
+        const uint16_t* a_next = lds + (kCur ^ 1) * kBufElems + a_off;
 
         // The next chunk's blocks: first round now - its counter is (block, stream name, 0, 0) and
         // the block number is the same for the GPW groups, so it is one multiply for all of them
         // and one xor per group - the other nine under the MFMAs below.
         jl::u32x4 pc[GPW], pn[GPW];
         {
-            const uint64_t q0 = (uint64_t)jl::kPhiloxM0 * (2u * p1.s + h);
+            const uint64_t q0 = (uint64_t)jl::kPhiloxM0 * (2u * nx.s + h);
 #pragma unroll
             for (int j = 0; j < GPW; ++j) {
-                pc[j].x = jl::stream_name(seed, col0 + 32u * j, p1.tile) ^ seed;
+                pc[j].x = jl::stream_name(seed, col0 + 32u * j, nx.tile) ^ seed;
                 pc[j].y = 0u;
                 pc[j].z = (uint32_t)(q0 >> 32);
                 pc[j].w = (uint32_t)q0;
             }
         }
 
-        auto operand = [&](int step) -> uint4 {
-            const int q = step / GPW, j = step % GPW;
-            return *reinterpret_cast<const uint4*>(smem + sign_entry_address(wd[j][q >> 2], q, lane_base));
-        };
-        uint4 bq[kAhead + 1];
+        if (!kRing) {
 #pragma unroll
-        for (int p = 0; p < kAhead; ++p) bq[p] = operand(p);
-        uint4 a[2][RB][kPlanes];  // A operands of this q and of the next one (read one q ahead)
-#pragma unroll
-        for (int rb = 0; rb < RB; ++rb)
-#pragma unroll
-            for (int pl = 0; pl < kPlanes; ++pl)
-                a[0][rb][pl] = *reinterpret_cast<const uint4*>(a_base + rb * 32 * kLdsRow + pl * kPlaneElems);
+            for (int p = 0; p < kAhead; ++p) bq[p] = lookup(wd[p % GPW][(p / GPW) >> 2], p / GPW);
+            read_a(a_base, 0, 0);
+        }
 #pragma unroll
         for (int q = 0; q < 16; ++q) {
 #pragma unroll
             for (int j = 0; j < GPW; ++j) {
                 const int step = q * GPW + j;
-                if (step + kAhead < kSteps) bq[(step + kAhead) % (kAhead + 1)] = operand(step + kAhead);
-                if (j == 0 && q + 1 < 16) {
-#pragma unroll
-                    for (int rb = 0; rb < RB; ++rb)
-#pragma unroll
-                        for (int pl = 0; pl < kPlanes; ++pl)
-                            a[(q + 1) & 1][rb][pl] = *reinterpret_cast<const uint4*>(
-                                a_base + rb * 32 * kLdsRow + pl * kPlaneElems + 8 * (q + 1));
+                if (kRing && step == kSyncStep) __syncthreads();
+                {
+                    const int t = step + kAhead;  // the look-up issued now; beyond this chunk: the next one's
+                    if (t < kSteps)
+                        bq[t % (kAhead + 1)] = lookup(wd[t % GPW][(t / GPW) >> 2], t / GPW);
+                    else if (kRing)
+                        bq[t % (kAhead + 1)] = lookup(pc[(t - kSteps) % GPW].x, (t - kSteps) / GPW);
+                }
+                if (j == 0) {
+                    if (q + 1 < 16)
+                        read_a(a_base, (q + 1) & 1, q + 1);
+                    else if (kRing)
+                        read_a(a_next, 0, 0);
                 }
                 // half rounds number first .. first + count - 1 of the kHalfRounds; number
-                // i is half i % 2 of round 1 + i / (2 GPW) of group (i / 2) % GPW.  Every
-                // kSteps / extra-th step takes two.
+                // i is half i % 2 of round 1 + i / (2 GPW) of group (i / 2) % GPW.  They are
+                // spread over the first kSpan steps, one per step and two in every kEvery-th:
+                // group g's block must be complete when its first look-up for the next chunk
+                // is issued, kAhead steps before the end.
                 {
-                    constexpr int kExtra = kHalfRounds - kSteps;       // steps that take two
-                    constexpr int kEvery = kSteps / kExtra;
-                    const int twos_before = (step + kEvery - 1) / kEvery;  // steps < step that took two
-                    const int first = step + (twos_before < kExtra ? twos_before : kExtra);
-                    const int count = (step % kEvery == 0 && step / kEvery < kExtra) ? 2 : 1;
+                    constexpr int kSpan = GPW == 4 ? kSteps : kSteps - 4;
+                    constexpr int kExtra = kHalfRounds - kSpan;        // steps that take two
+                    constexpr int kEvery = kSpan / kExtra;
+                    static_assert(kExtra * kEvery <= kSpan, "half-round schedule");
+                    const int twos = (step + kEvery - 1) / kEvery;     // steps < step that took two
+                    const int first = step + (twos < kExtra ? twos : kExtra);
+                    const int count = step >= kSpan ? 0 : (step % kEvery == 0 && step / kEvery < kExtra) ? 2 : 1;
 #pragma unroll
                     for (int u = first; u < first + count; ++u) {
                         const int r = 1 + u / (2 * GPW), g4 = (u / 2) % GPW, half = u % 2;
@@ -617,6 +662,15 @@ __global__ __launch_bounds__(512) void jl_project_kernel(
                                     (uint32_t)r * jl::kPhiloxW1);
                         if (half == 1) pc[g4] = pn[g4];
                     }
+                }
+                if (kRing && step == kStoreStep) {
+                    if (i + 1 < n_chunks) st.store(lds + (kCur ^ 1) * kBufElems, tid);
+                }
+                if (kRing && step == kLoadStep) {
+                    if (i + 2 < n_chunks) load_chunk(ld2);
+                    nx.tile = ld2.tile;
+                    nx.s = ld2.s;
+                    advance(ld2);
                 }
                 __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
@@ -629,20 +683,11 @@ __global__ __launch_bounds__(512) void jl_project_kernel(
         }
 #pragma unroll
         for (int j = 0; j < GPW; ++j) wd[j][0] = pc[j].x, wd[j][1] = pc[j].y, wd[j][2] = pc[j].z, wd[j][3] = pc[j].w;
-
-        if (kBuffers == 2) {
-            // the other buffer was last read in the previous chunk, before its barrier
-            if (i + 1 < n_chunks) drain.store(lds + (cur ^ 1) * kBufElems, tid);
-            __syncthreads();
-            cur ^= 1;
-        }
-        p0 = p1;
-        p1 = p2;
-        step_pos(p2);
+        if (!kRing) advance(nx);
     };
     for (uint32_t i = 0; i < n_chunks; i += 2) {
-        chunk(i, st_a, st_b);
-        if (i + 1 < n_chunks) chunk(i + 1, st_b, st_a);
+        chunk(i, std::integral_constant<int, 0>{});
+        if (i + 1 < n_chunks) chunk(i + 1, std::integral_constant<int, kRing ? 1 : 0>{});
     }
 
     // D[m][n] of a 32x32 MFMA: lane holds column n = lane % 32 and, in register r, row
