@@ -29,6 +29,7 @@
 
 #include <atomic>
 #include <type_traits>
+#include <utility>
 
 #include "jl_stream.h"
 #include "store_cast.h"
@@ -399,22 +400,37 @@ __device__ __forceinline__ uint32_t sign_entry_address(uint32_t word, int q, uin
 // of the next state), half 1 the multiply of c.z (gives x, y).  The empty asm statements tie the
 // instructions to the place in the instruction stream where the call stands: without them the
 // compiler moves all the generator arithmetic of a chunk in front of its first MFMA.
-__device__ __forceinline__ void philox_half(const jl::u32x4& c, jl::u32x4& next, int half, uint32_t k0, uint32_t k1) {
+//
+// In two parts, so that other instructions of the step can stand between the asm that ties down the
+// inputs and the multiply: the compiler assumes that a register written by inline asm may not be read
+// by the very next vector instruction (one wait state on this target) and would put an s_nop there.
+struct PhiloxHalfIn {
+    uint32_t m, o;  // the word that is multiplied and the word that is xored into the high half
+};
+__device__ __forceinline__ PhiloxHalfIn philox_half_in(const jl::u32x4& c, int half) {
+    PhiloxHalfIn in = {half == 0 ? c.x : c.z, half == 0 ? c.w : c.y};
+    asm volatile("" : "+v"(in.m), "+v"(in.o));
+    return in;
+}
+__device__ __forceinline__ void philox_half_out(const PhiloxHalfIn& in, jl::u32x4& next, int half, uint32_t k0,
+                                                uint32_t k1) {
     if (half == 0) {
-        uint32_t x = c.x, w = c.w;
-        asm volatile("" : "+v"(x), "+v"(w));
-        const uint64_t p0 = (uint64_t)jl::kPhiloxM0 * x;
-        next.z = jl::xor3((uint32_t)(p0 >> 32), w, k1);
+        const uint64_t p0 = (uint64_t)jl::kPhiloxM0 * in.m;
+        next.z = jl::xor3((uint32_t)(p0 >> 32), in.o, k1);
         next.w = (uint32_t)p0;
         asm volatile("" : "+v"(next.z), "+v"(next.w));
     } else {
-        uint32_t z = c.z, y = c.y;
-        asm volatile("" : "+v"(z), "+v"(y));
-        const uint64_t p1 = (uint64_t)jl::kPhiloxM1 * z;
-        next.x = jl::xor3((uint32_t)(p1 >> 32), y, k0);
+        const uint64_t p1 = (uint64_t)jl::kPhiloxM1 * in.m;
+        next.x = jl::xor3((uint32_t)(p1 >> 32), in.o, k0);
         next.y = (uint32_t)p1;
         asm volatile("" : "+v"(next.x), "+v"(next.y));
     }
+}
+
+// f(integral_constant<int, 0>), f(integral_constant<int, 1>), ... in this order
+template <class F, int... S>
+__device__ __forceinline__ void for_each_step(F& f, std::integer_sequence<int, S...>) {
+    (f(std::integral_constant<int, S>{}), ...);
 }
 
 // GATHER: g_in is a device array of trakhip_segment and ld their number; otherwise g_in is the
@@ -623,50 +639,54 @@ __global__ __launch_bounds__(512) void jl_project_kernel(
             for (int p = 0; p < kAhead; ++p) bq[p] = lookup(wd[p % GPW][(p / GPW) >> 2], p / GPW);
             read_a(a_base, 0, 0);
         }
-#pragma unroll
-        for (int q = 0; q < 16; ++q) {
-#pragma unroll
-            for (int j = 0; j < GPW; ++j) {
-                const int step = q * GPW + j;
-                if (kRing && step == kSyncStep) __syncthreads();
-                {
-                    const int t = step + kAhead;  // the look-up issued now; beyond this chunk: the next one's
-                    if (t < kSteps)
-                        bq[t % (kAhead + 1)] = lookup(wd[t % GPW][(t / GPW) >> 2], t / GPW);
-                    else if (kRing)
-                        bq[t % (kAhead + 1)] = lookup(pc[(t - kSteps) % GPW].x, (t - kSteps) / GPW);
-                }
-                if (j == 0) {
-                    if (q + 1 < 16)
-                        read_a(a_base, (q + 1) & 1, q + 1);
-                    else if (kRing)
-                        read_a(a_next, 0, 0);
-                }
+        // one step; the step number is a constant (the steps are written out through for_each_step, which
+        // does not depend on the optimizer's unrolling limits)
+        auto do_step = [&](auto step_c) __attribute__((always_inline)) {
+            {
+                constexpr int step = decltype(step_c)::value;
+                constexpr int q = step / GPW, j = step % GPW;
+                if constexpr (kRing && step == kSyncStep) __syncthreads();
                 // half rounds number first .. first + count - 1 of the kHalfRounds; number
                 // i is half i % 2 of round 1 + i / (2 GPW) of group (i / 2) % GPW.  They are
                 // spread over the first kSpan steps, one per step and two in every kEvery-th:
                 // group g's block must be complete when its first look-up for the next chunk
                 // is issued, kAhead steps before the end.
+                constexpr int kSpan = GPW == 4 ? kSteps : kSteps - 4;
+                constexpr int kExtra = kHalfRounds - kSpan;        // steps that take two
+                constexpr int kEvery = kSpan / kExtra;
+                static_assert(kExtra * kEvery <= kSpan, "half-round schedule");
+                constexpr int twos = (step + kEvery - 1) / kEvery;     // steps < step that took two
+                constexpr int first = step + (twos < kExtra ? twos : kExtra);
+                constexpr int count = step >= kSpan ? 0 : (step % kEvery == 0 && step / kEvery < kExtra) ? 2 : 1;
+                PhiloxHalfIn hin0 = {0u, 0u}, hin1 = {0u, 0u};
+                if constexpr (count >= 1) hin0 = philox_half_in(pc[(first / 2) % GPW], first % 2);
+                if constexpr (count == 2) hin1 = philox_half_in(pc[((first + 1) / 2) % GPW], (first + 1) % 2);
                 {
-                    constexpr int kSpan = GPW == 4 ? kSteps : kSteps - 4;
-                    constexpr int kExtra = kHalfRounds - kSpan;        // steps that take two
-                    constexpr int kEvery = kSpan / kExtra;
-                    static_assert(kExtra * kEvery <= kSpan, "half-round schedule");
-                    const int twos = (step + kEvery - 1) / kEvery;     // steps < step that took two
-                    const int first = step + (twos < kExtra ? twos : kExtra);
-                    const int count = step >= kSpan ? 0 : (step % kEvery == 0 && step / kEvery < kExtra) ? 2 : 1;
-#pragma unroll
-                    for (int u = first; u < first + count; ++u) {
-                        const int r = 1 + u / (2 * GPW), g4 = (u / 2) % GPW, half = u % 2;
-                        philox_half(pc[g4], pn[g4], half, seed + (uint32_t)r * jl::kPhiloxW0,
-                                    (uint32_t)r * jl::kPhiloxW1);
-                        if (half == 1) pc[g4] = pn[g4];
-                    }
+                    constexpr int t = step + kAhead;  // the look-up issued now; beyond this chunk: the next one's
+                    if constexpr (t < kSteps)
+                        bq[t % (kAhead + 1)] = lookup(wd[t % GPW][(t / GPW) >> 2], t / GPW);
+                    else if constexpr (kRing)
+                        bq[t % (kAhead + 1)] = lookup(pc[(t - kSteps) % GPW].x, (t - kSteps) / GPW);
                 }
-                if (kRing && step == kStoreStep) {
+                if constexpr (j == 0) {
+                    if constexpr (q + 1 < 16)
+                        read_a(a_base, (q + 1) & 1, q + 1);
+                    else if constexpr (kRing)
+                        read_a(a_next, 0, 0);
+                }
+                auto half_out = [&](const PhiloxHalfIn& in, int u) {
+                    const int r = 1 + u / (2 * GPW), g4 = (u / 2) % GPW;
+                    philox_half_out(in, pn[g4], u % 2, seed + (uint32_t)r * jl::kPhiloxW0, (uint32_t)r * jl::kPhiloxW1);
+                };
+                if constexpr (count >= 1) half_out(hin0, first);
+                if constexpr (count == 2) half_out(hin1, first + 1);
+#pragma unroll
+                for (int u = first; u < first + count; ++u)
+                    if (u % 2 == 1) pc[(u / 2) % GPW] = pn[(u / 2) % GPW];
+                if constexpr (kRing && step == kStoreStep) {
                     if (i + 1 < n_chunks) st.store(lds + (kCur ^ 1) * kBufElems, tid);
                 }
-                if (kRing && step == kLoadStep) {
+                if constexpr (kRing && step == kLoadStep) {
                     if (i + 2 < n_chunks) load_chunk(ld2);
                     nx.tile = ld2.tile;
                     nx.s = ld2.s;
@@ -680,7 +700,8 @@ __global__ __launch_bounds__(512) void jl_project_kernel(
                         acc[rb][j] = mfma16(a[q & 1][rb][pl], bq[step % (kAhead + 1)], acc[rb][j], kBf);
                 __builtin_amdgcn_sched_barrier(0);
             }
-        }
+        };
+        for_each_step(do_step, std::make_integer_sequence<int, kSteps>{});
 #pragma unroll
         for (int j = 0; j < GPW; ++j) wd[j][0] = pc[j].x, wd[j][1] = pc[j].y, wd[j][2] = pc[j].z, wd[j][3] = pc[j].w;
         if (!kRing) advance(nx);
