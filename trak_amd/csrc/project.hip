@@ -59,6 +59,20 @@ struct __attribute__((packed, aligned(4))) Raw16f {
     uint32_t x, y, z, w;
 };
 
+// Gradient data is device (global) memory.  Reading it through a pointer that says so keeps the loads
+// from becoming FLAT instructions where the pointer comes out of a segment table: a FLAT load counts as
+// an LDS operation too, and every wait for an LDS operand would then wait for all the gradient loads in
+// flight.
+template <typename T>
+__device__ __forceinline__ T gload(const void* p) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    typedef const T __attribute__((address_space(1))) * global_ptr;
+    return *(global_ptr)(uintptr_t)p;  // (a direct pointer cast is folded back into a generic pointer)
+#else
+    return *static_cast<const T*>(p);  // host pass of the compiler: never executed
+#endif
+}
+
 template <int IN>
 struct InTraits;
 template <>
@@ -100,7 +114,7 @@ struct Stage16 {
         const uint16_t* p = g + (uint64_t)(tid >> 5) * ld + f_begin + 8u * (tid & 31);
 #pragma unroll
         for (int i = 0; i < N; ++i) {
-            const Raw16 r = *reinterpret_cast<const Raw16*>(p + (uint64_t)(2 * W * i) * ld);
+            const Raw16 r = gload<Raw16>(p + (uint64_t)(2 * W * i) * ld);
             v[i] = {r.x, r.y, r.z, r.w};
         }
     }
@@ -124,12 +138,12 @@ struct Stage16 {
             if (row < rows && f < f_end) {
                 const uint16_t* p = g + (uint64_t)row * ld + f;
                 if (f + 8 <= f_end) {
-                    const Raw16 r = *reinterpret_cast<const Raw16*>(p);
+                    const Raw16 r = gload<Raw16>(p);
                     val = {r.x, r.y, r.z, r.w};
                 } else {
                     uint32_t e[8];
 #pragma unroll
-                    for (int t = 0; t < 8; ++t) e[t] = (f + t < f_end) ? (uint32_t)p[t] : 0u;
+                    for (int t = 0; t < 8; ++t) e[t] = (f + t < f_end) ? (uint32_t)gload<uint16_t>(p + t) : 0u;
                     val = {e[0] | (e[1] << 16), e[2] | (e[3] << 16), e[4] | (e[5] << 16),
                            e[6] | (e[7] << 16)};
                 }
@@ -166,12 +180,12 @@ struct Stage32 {
             if (row < rows && f < f_end) {
                 const float* p = g + (uint64_t)row * ld + f;
                 if (f + 4 <= f_end) {
-                    const Raw16f r = *reinterpret_cast<const Raw16f*>(p);
+                    const Raw16f r = gload<Raw16f>(p);
                     val = {r.x, r.y, r.z, r.w};
                 } else {
-                    val.x = __float_as_uint(p[0]);
-                    val.y = (f + 1 < f_end) ? __float_as_uint(p[1]) : 0u;
-                    val.z = (f + 2 < f_end) ? __float_as_uint(p[2]) : 0u;
+                    val.x = gload<uint32_t>(p);
+                    val.y = (f + 1 < f_end) ? gload<uint32_t>(p + 1) : 0u;
+                    val.z = (f + 2 < f_end) ? gload<uint32_t>(p + 2) : 0u;
                     val.w = 0u;
                 }
             }
@@ -261,7 +275,7 @@ __device__ __noinline__ uint4 gather_piece(const trakhip_segment* segs, uint32_t
         if (ff >= f_end) break;
         while (idx + 1 < n && ff >= segs[idx + 1].first) ++idx;
         const trakhip_segment sg = segs[idx];
-        const uint32_t val = (uint32_t) reinterpret_cast<const T*>(sg.ptr)[(uint64_t)row * sg.ld + (ff - sg.first)];
+        const uint32_t val = (uint32_t)gload<T>(reinterpret_cast<const T*>(sg.ptr) + (uint64_t)row * sg.ld + (ff - sg.first));
         if (sizeof(T) == 2)
             e[t >> 1] |= val << (16 * (t & 1));
         else
@@ -269,6 +283,37 @@ __device__ __noinline__ uint4 gather_piece(const trakhip_segment* segs, uint32_t
     }
     return {e[0], e[1], e[2], e[3]};
 }
+
+// The segment the workgroup's current chunk starts in, as uniform values (scalar registers): when the
+// whole chunk lies inside it, the chunk is loaded like a chunk of a dense matrix, without the per-thread
+// cursors below.
+struct UniformSeg {
+    uint32_t idx;
+    uint64_t first, end, ld;
+    const void* ptr;
+    __device__ __forceinline__ void set(const trakhip_segment* segs, uint32_t i) {
+        const trakhip_segment sg = segs[i];
+        idx = i;
+        first = sg.first;
+        end = sg.first + sg.numel;
+        ld = sg.ld;
+        ptr = sg.ptr;
+    }
+    __device__ __forceinline__ void seek(const trakhip_segment* segs, uint32_t n, uint64_t f) {
+        uint32_t lo = 0, hi = n - 1;
+        while (lo < hi) {
+            const uint32_t mid = (lo + hi + 1) >> 1;
+            if (segs[mid].first <= f)
+                lo = mid;
+            else
+                hi = mid - 1;
+        }
+        set(segs, lo);
+    }
+    __device__ __forceinline__ void advance(const trakhip_segment* segs, uint32_t n, uint64_t f) {
+        while (f >= end && idx + 1 < n) set(segs, idx + 1);
+    }
+};
 
 template <int W, int ROWS = 32>
 struct Gather16 : Stage16<W, ROWS> {
@@ -287,7 +332,23 @@ struct Gather16 : Stage16<W, ROWS> {
         const bool live = f64 < f_end;
         const uint32_t f = (uint32_t)f64;
         if (live) cur.advance(segs, n, f, tid >> 5, 2 * W, 2);
-        const uint32_t lim = (uint32_t)f_end < cur.end ? (uint32_t)f_end : cur.end;  // f_end <= P < 2^32
+        load_at(segs, n, cur, rows, f64, f_end, live, tid);
+    }
+    // The same with a cursor that lives for this call only and starts at segment `start`, one that begins
+    // at or before f_begin: for a caller that takes this path rarely and saves the registers.
+    __device__ __forceinline__ void load_from(const trakhip_segment* segs, uint32_t n, uint32_t start, uint32_t rows,
+                                              uint64_t f_begin, uint64_t f_end, int tid) {
+        const uint64_t f64 = f_begin + 8u * (tid & 31);
+        const bool live = f64 < f_end;
+        SegCursor<N> c;
+        c.set(segs, start, tid >> 5, 2 * W, 2);
+        if (live) c.advance(segs, n, (uint32_t)f64, tid >> 5, 2 * W, 2);
+        load_at(segs, n, c, rows, f64, f_end, live, tid);
+    }
+    __device__ __forceinline__ void load_at(const trakhip_segment* segs, uint32_t n, const SegCursor<N>& c, uint32_t rows,
+                                            uint64_t f64, uint64_t f_end, bool live, int tid) {
+        const uint32_t f = (uint32_t)f64;
+        const uint32_t lim = (uint32_t)f_end < c.end ? (uint32_t)f_end : c.end;  // f_end <= P < 2^32
         const bool whole = live && f + 8u <= lim && f + 8u > f;
 #pragma unroll
         for (int i = 0; i < N; ++i) {
@@ -295,10 +356,10 @@ struct Gather16 : Stage16<W, ROWS> {
             uint4 val = {0u, 0u, 0u, 0u};
             if (live && row < rows) {
                 if (whole) {
-                    const Raw16 r = *reinterpret_cast<const Raw16*>(cur.base[i] + (uint64_t)f * 2);
+                    const Raw16 r = gload<Raw16>(c.base[i] + (uint64_t)f * 2);
                     val = {r.x, r.y, r.z, r.w};
                 } else {
-                    val = gather_piece<uint16_t, 8>(segs, n, cur.idx, row, f64, f_end);
+                    val = gather_piece<uint16_t, 8>(segs, n, c.idx, row, f64, f_end);
                 }
             }
             v[i] = val;
@@ -331,7 +392,7 @@ struct Gather32 : Stage32<W> {
             uint4 val = {0u, 0u, 0u, 0u};
             if (live && row < rows) {
                 if (whole) {
-                    const Raw16f r = *reinterpret_cast<const Raw16f*>(cur.base[i] + (uint64_t)f * 4);
+                    const Raw16f r = gload<Raw16f>(cur.base[i] + (uint64_t)f * 4);
                     val = {r.x, r.y, r.z, r.w};
                 } else {
                     val = gather_piece<uint32_t, 4>(segs, n, cur.idx, row, f64, f_end);
@@ -544,12 +605,19 @@ __global__ __launch_bounds__(512) void jl_project_kernel(
     };
     const bool full_rows = rows == 32u * RB;
     Stage st;
+    UniformSeg useg = {0u, 0u, 0u, 0u, nullptr};  // GATHER, 16-bit gradients
     auto load_chunk = [&](const Cursor& c) {
         if constexpr (!GATHER && kPlanes == 1) {
             if (full_rows && c.s < c.whole)
                 st.load_whole(g, ld, c.f, tid);
             else
                 st.load_edge(g, ld, rows, c.f, c.hi, tid);
+        } else if constexpr (GATHER && kPlanes == 1) {
+            useg.advance(g, (uint32_t)ld, c.f);
+            if (full_rows && c.s < c.whole && c.f >= useg.first && c.f + kChunk <= useg.end)
+                st.load_whole(static_cast<const uint16_t*>(useg.ptr), useg.ld, c.f - useg.first, tid);
+            else  // chunks that cross a segment or tile end: per-thread cursors, set up for this chunk only
+                st.load_from(g, (uint32_t)ld, useg.idx, rows, c.f, c.hi, tid);
         } else {
             st.load(g, ld, rows, c.f, c.hi, tid);
         }
@@ -570,7 +638,12 @@ __global__ __launch_bounds__(512) void jl_project_kernel(
     Cursor nx = {t0, s0, 0u, 0u, 0u};  // the chunk after the current one (tile and s: its generator blocks)
     open_tile(nx);
     Cursor ld2 = nx;                   // kRing: the chunk after that (the next one to load)
-    if constexpr (GATHER) st.init(g, (uint32_t)ld, nx.f, P, tid);
+    if constexpr (GATHER) {
+        if constexpr (kPlanes == 1)
+            useg.seek(g, (uint32_t)ld, nx.f < P ? nx.f : P - 1);
+        else
+            st.init(g, (uint32_t)ld, nx.f, P, tid);
+    }
     load_chunk(nx);
     advance(nx);
     if (kRing) {
