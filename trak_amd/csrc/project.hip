@@ -118,6 +118,14 @@ struct Stage16 {
             v[i] = {r.x, r.y, r.z, r.w};
         }
     }
+    // the same from the address of the thread's first piece and the distance in bytes to its next one
+    __device__ __forceinline__ void load_pieces(const char* p, uint64_t piece_pitch) {
+#pragma unroll
+        for (int i = 0; i < N; ++i) {
+            const Raw16 r = gload<Raw16>(p + i * piece_pitch);
+            v[i] = {r.x, r.y, r.z, r.w};
+        }
+    }
     __device__ __forceinline__ void load(const uint16_t* __restrict__ g, uint64_t ld, uint32_t rows,
                                          uint64_t f_begin, uint64_t f_end, int tid) {
         if (rows == ROWS && f_begin + kChunk <= f_end) {  // uniform test
@@ -287,31 +295,37 @@ __device__ __noinline__ uint4 gather_piece(const trakhip_segment* segs, uint32_t
 // The segment the workgroup's current chunk starts in, as uniform values (scalar registers): when the
 // whole chunk lies inside it, the chunk is loaded like a chunk of a dense matrix, without the per-thread
 // cursors below.
+// 16-bit elements; a thread's pieces are at row tid / 32 + row_step * i, features 8 (tid % 32) .. + 7 of the chunk.
 struct UniformSeg {
     uint32_t idx;
-    uint64_t first, end, ld;
-    const void* ptr;
-    __device__ __forceinline__ void set(const trakhip_segment* segs, uint32_t i) {
+    uint32_t first, end;   // feature range of segs[idx] (P < 2^32)
+    uint64_t piece_pitch;  // bytes from one piece of a thread to its next (row_step rows)
+    const char* tbase;     // per thread: tbase + 2 f = address of its first piece of the chunk that starts at feature f
+    __device__ __forceinline__ void set(const trakhip_segment* segs, uint32_t i, int tid, uint32_t row_step) {
         const trakhip_segment sg = segs[i];
+        // the same values in every lane; said so, they live in scalar registers (a load that follows a
+        // barrier is never a scalar load by itself)
         idx = i;
-        first = sg.first;
-        end = sg.first + sg.numel;
-        ld = sg.ld;
-        ptr = sg.ptr;
+        first = __builtin_amdgcn_readfirstlane((uint32_t)sg.first);
+        end = __builtin_amdgcn_readfirstlane((uint32_t)(sg.first + sg.numel));
+        const uint64_t pp = (uint64_t)row_step * sg.ld * 2;
+        piece_pitch = ((uint64_t)__builtin_amdgcn_readfirstlane((uint32_t)(pp >> 32)) << 32) |
+                      __builtin_amdgcn_readfirstlane((uint32_t)pp);
+        tbase = static_cast<const char*>(sg.ptr) + ((uint64_t)(tid >> 5) * sg.ld + 8u * (tid & 31)) * 2 - sg.first * 2;
     }
-    __device__ __forceinline__ void seek(const trakhip_segment* segs, uint32_t n, uint64_t f) {
+    __device__ __forceinline__ void seek(const trakhip_segment* segs, uint32_t n, uint32_t f, int tid, uint32_t row_step) {
         uint32_t lo = 0, hi = n - 1;
         while (lo < hi) {
             const uint32_t mid = (lo + hi + 1) >> 1;
-            if (segs[mid].first <= f)
+            if ((uint32_t)segs[mid].first <= f)
                 lo = mid;
             else
                 hi = mid - 1;
         }
-        set(segs, lo);
+        set(segs, lo, tid, row_step);
     }
-    __device__ __forceinline__ void advance(const trakhip_segment* segs, uint32_t n, uint64_t f) {
-        while (f >= end && idx + 1 < n) set(segs, idx + 1);
+    __device__ __forceinline__ void advance(const trakhip_segment* segs, uint32_t n, uint32_t f, int tid, uint32_t row_step) {
+        while (f >= end && idx + 1 < n) set(segs, idx + 1, tid, row_step);
     }
 };
 
@@ -613,9 +627,10 @@ __global__ __launch_bounds__(512) void jl_project_kernel(
             else
                 st.load_edge(g, ld, rows, c.f, c.hi, tid);
         } else if constexpr (GATHER && kPlanes == 1) {
-            useg.advance(g, (uint32_t)ld, c.f);
-            if (full_rows && c.s < c.whole && c.f >= useg.first && c.f + kChunk <= useg.end)
-                st.load_whole(static_cast<const uint16_t*>(useg.ptr), useg.ld, c.f - useg.first, tid);
+            const uint32_t f32 = (uint32_t)c.f;  // P < 2^32 with segments; beyond P: c.whole is 0
+            useg.advance(g, (uint32_t)ld, f32, tid, 2 * W);
+            if (full_rows && c.s < c.whole && f32 >= useg.first && f32 + (uint32_t)kChunk <= useg.end)
+                st.load_pieces(useg.tbase + 2 * (uint64_t)f32, useg.piece_pitch);
             else  // chunks that cross a segment or tile end: per-thread cursors, set up for this chunk only
                 st.load_from(g, (uint32_t)ld, useg.idx, rows, c.f, c.hi, tid);
         } else {
@@ -640,7 +655,7 @@ __global__ __launch_bounds__(512) void jl_project_kernel(
     Cursor ld2 = nx;                   // kRing: the chunk after that (the next one to load)
     if constexpr (GATHER) {
         if constexpr (kPlanes == 1)
-            useg.seek(g, (uint32_t)ld, nx.f < P ? nx.f : P - 1);
+            useg.seek(g, (uint32_t)ld, (uint32_t)(nx.f < P ? nx.f : P - 1), tid, 2 * W);
         else
             st.init(g, (uint32_t)ld, nx.f, P, tid);
     }
