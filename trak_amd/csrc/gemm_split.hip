@@ -310,29 +310,58 @@ __device__ __forceinline__ void store_c(const floatx16 (&acc)[2][JT], float* __r
 // lanes of a wave fetch 64 consecutive rows of one (plane, octet), which land at 64 consecutive
 // 16-byte slots starting at a wave-uniform LDS address; no staging registers, no LDS store
 // instructions.  Wave w moves chunks w, w + 8, ...
+//
+// A chunk's 64 pieces are consecutive in memory as well (64 rows of one plane and octet), so its address
+// is a wave-uniform base plus 16 bytes per lane, and the base moves by a fixed number of bytes from step
+// to step: the bases live in scalar registers and a load costs two scalar additions.  (Computing the
+// piece address per lane from plane, octet and row took about thirty instructions per load, in front of
+// the MFMAs of every step.)
 template <int P, int S>
-__device__ __forceinline__ void dma_step(const piece* __restrict__ A, uint64_t Rpa, const piece* __restrict__ B,
-                                         uint64_t Rpb, uint64_t K8, uint64_t m0, uint64_t n0, uint64_t s,
-                                         int wave, int lane, piece* lds) {
-    constexpr int kAChunks = P * 2 * BM / 64, kBChunks = P * 2 * BN / 64;
-    constexpr int kSubChunks = kAChunks + kBChunks, kChunks = S * kSubChunks;
-    static_assert(kChunks % kWaves == 0, "every wave moves the same number of chunks");
+struct StepMover {
+    static constexpr int kAChunks = P * 2 * BM / 64, kBChunks = P * 2 * BN / 64;
+    static constexpr int kSubChunks = kAChunks + kBChunks, kChunks = S * kSubChunks;
+    // the first kLoaders waves move the chunks: wave w chunks w, w + kLoaders, ...  (all eight: leaving the loads
+    // to four waves, so that the other four start their MFMAs at once, measured 1 % faster on the three-plane
+    // product and is not worth a second code path)
+    static constexpr int kLoaders = kWaves;
+    static_assert(kChunks % kLoaders == 0, "every loading wave moves the same number of chunks");
+    static_assert(BM % 64 == 0 && BN % 64 == 0, "a chunk lies in one (plane, half)");
+    static constexpr int kPerWave = kChunks / kLoaders;
+    const char* base[kPerWave];  // of this wave's chunks at the next step to load (wave-uniform)
+    uint64_t step_a, step_b;     // bytes from one step to the next
+
+    __device__ __forceinline__ void init(const piece* A, uint64_t Rpa, const piece* B, uint64_t Rpb, uint64_t K8,
+                                         uint64_t m0, uint64_t n0, uint64_t s, int wave) {
+        step_a = 2 * S * Rpa * sizeof(piece);
+        step_b = 2 * S * Rpb * sizeof(piece);
 #pragma unroll
-    for (int i = 0; i < kChunks / kWaves; ++i) {
-        const int c = wave + kWaves * i;  // wave-uniform
-        const int u = c / kSubChunks, cc = c % kSubChunks;
-        const piece* src;
-        if (cc < kAChunks) {
-            const int e = 64 * cc + lane, row = e % BM, ph = e / BM;  // ph = plane * 2 + half
-            src = A + ((uint64_t)(ph >> 1) * K8 + 2 * (s * S + u) + (ph & 1)) * Rpa + m0 + row;
-        } else {
-            const int e = 64 * (cc - kAChunks) + lane, row = e % BN, ph = e / BN;
-            src = B + ((uint64_t)(ph >> 1) * K8 + 2 * (s * S + u) + (ph & 1)) * Rpb + n0 + row;
+        for (int i = 0; i < kPerWave; ++i) {
+            const int c = wave % kLoaders + kLoaders * i;  // wave-uniform
+            const int u = c / kSubChunks, cc = c % kSubChunks;
+            if (cc < kAChunks) {
+                const int e = 64 * cc, row = e % BM, ph = e / BM;  // ph = plane * 2 + half
+                base[i] = reinterpret_cast<const char*>(A + ((uint64_t)(ph >> 1) * K8 + 2 * (s * S + u) + (ph & 1)) * Rpa + m0 + row);
+            } else {
+                const int e = 64 * (cc - kAChunks), row = e % BN, ph = e / BN;
+                base[i] = reinterpret_cast<const char*>(B + ((uint64_t)(ph >> 1) * K8 + 2 * (s * S + u) + (ph & 1)) * Rpb + n0 + row);
+            }
         }
-        __builtin_amdgcn_global_load_lds((const void __attribute__((address_space(1)))*)src,
-                                         (void __attribute__((address_space(3)))*)(lds + 64 * c), 16, 0, 0);
     }
-}
+    // chunk i of the wave for the step the bases point at; then the base moves on to the step after
+    __device__ __forceinline__ void move(int i, int wave, uint32_t lane_bytes, piece* lds) {
+        const int c = wave % kLoaders + kLoaders * i;
+        __builtin_amdgcn_global_load_lds((const void __attribute__((address_space(1)))*)(base[i] + lane_bytes),
+                                         (void __attribute__((address_space(3)))*)(lds + 64 * c), 16, 0, 0);
+        // kAChunks is a multiple of kLoaders: which operand chunk i belongs to does not depend on the wave
+        base[i] += ((kLoaders * i) % kSubChunks) < kAChunks ? step_a : step_b;
+    }
+    static_assert(kAChunks % kLoaders == 0 && kSubChunks % kLoaders == 0, "operand of a chunk: the same for all waves");
+    __device__ __forceinline__ void move_all(int wave, uint32_t lane_bytes, piece* lds) {
+        if (wave >= kLoaders) return;
+#pragma unroll
+        for (int i = 0; i < kPerWave; ++i) move(i, wave, lane_bytes, lds);
+    }
+};
 
 // P planes per operand (3: split fp32, 1: a 16-bit type), F16 selects the fp16 MFMA, S sub-steps
 // per barrier.
@@ -382,7 +411,10 @@ __global__ __launch_bounds__(64 * kWaves, 2) void gemm_split_kernel(
 
     const uint64_t all_steps = K8 / (2 * S);
     const uint64_t first = all_steps * part / parts, steps = all_steps * (part + 1) / parts;  // [first, steps)
-    dma_step<P, S>(A, Rpa, B, Rpb, K8, m0, n0, first, wave, lane, lds[0]);
+    StepMover<P, S> mover;
+    mover.init(A, Rpa, B, Rpb, K8, m0, n0, first, wave);
+    const uint32_t lane_bytes = (uint32_t)lane * (uint32_t)sizeof(piece);
+    mover.move_all(wave, lane_bytes, lds[0]);
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
 
@@ -393,7 +425,7 @@ __global__ __launch_bounds__(64 * kWaves, 2) void gemm_split_kernel(
     for (uint64_t s = first; s < steps; ++s) {
         const int cur = (int)((s - first) & 1);
         // the other buffer was last read before the barrier that ended the previous step
-        if (s + 1 < steps) dma_step<P, S>(A, Rpa, B, Rpb, K8, m0, n0, s + 1, wave, lane, lds[cur ^ 1]);
+        if (s + 1 < steps) mover.move_all(wave, lane_bytes, lds[cur ^ 1]);
 #pragma unroll
         for (int u = 0; u < S; ++u) {
             const piece* l = lds[cur] + u * kSubPieces;
