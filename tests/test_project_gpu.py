@@ -563,6 +563,31 @@ def test_gather_many_rows_and_tiny_segments(gpu, B, k):
         assert torch.equal(fn(R)(flat[b0:b0 + 32].contiguous(), k, 11, 256), dense[b0:b0 + 32])
 
 
+@pytest.mark.parametrize("proj_type", [R, G])
+@pytest.mark.parametrize("dtype,B", [(torch.float16, 32), (torch.bfloat16, 64), (torch.float16, 40)])
+def test_gather_long_tiles_and_segment_boundaries(gpu, proj_type, dtype, B):
+    # Few feature tiles, so that most chunks lie wholly inside a tile and inside one tensor (they are loaded like
+    # the chunks of a dense matrix, from the segment the workgroup keeps in scalar registers), with tensor
+    # boundaries on and off multiples of 256 features, tensors shorter than a chunk in between, row pitches
+    # larger than the tensor (column slices) and a last tensor that ends inside a chunk.
+    from trak_amd import vectorize
+
+    gen = torch.Generator(device="cpu").manual_seed(79)
+    sizes = [256 * 40, 256 * 3, 5, 256 * 17 + 1, 255, 256 * 60 - 6, 1, 256 * 25, 31_003, 256, 256 * 9 + 130]
+    grads = []
+    for i, n in enumerate(sizes):
+        if i % 3 == 1:   # a column slice of a wider buffer: row pitch > n, rows not 16-byte aligned
+            wide = (torch.randn(B, n + 37, generator=gen) * 1e-2).to(dtype).to(gpu)
+            grads.append(wide[:, 5:5 + n])
+        else:
+            grads.append((torch.randn(B, n, generator=gen) * 1e-2).to(dtype).to(gpu))
+    flat = vectorize({i: g for i, g in enumerate(grads)}, device=gpu)
+    for tiles, k in ((7, 1024), (1, 512), (64, 2048)):
+        dense = fn(proj_type)(flat, k, 21, tiles)
+        gathered = fast_jl.project_gather(grads, k, 21, tiles, NAMES[proj_type])
+        assert torch.equal(dense, gathered), (tiles, k)
+
+
 # ---- more than 32 rows: the batch is walked 64 or 32 rows at a time -----------------------------
 
 
