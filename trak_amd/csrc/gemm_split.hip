@@ -243,6 +243,27 @@ __device__ __forceinline__ floatx16 mfma16(const piece& a, const piece& b, float
                                                        c, 0, 0, 0);
 }
 
+typedef float float4u __attribute__((ext_vector_type(4), aligned(4)));
+
+// 4 x 4 transpose inside every quad of lanes: lane q of a quad holds M[a][q] in v[a] and ends up with
+// M[q][c] in v[c].  Two exchanges, over lane distance 2 and 1: (register r, lane q) trades places with
+// (register r ^ d, lane q ^ d) where bit d of r and q differ.
+__device__ __forceinline__ void quad_transpose(float (&v)[4], int lane) {
+    const bool b1 = lane & 2, b0 = lane & 1;
+#pragma unroll
+    for (int r = 0; r < 2; ++r) {
+        const float send = b1 ? v[r] : v[r + 2];
+        const float recv = __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, send), 0x4E, 0xF, 0xF, true));  // quad_perm [2,3,0,1]
+        if (b1) v[r] = recv; else v[r + 2] = recv;
+    }
+#pragma unroll
+    for (int r = 0; r < 4; r += 2) {
+        const float send = b0 ? v[r] : v[r + 1];
+        const float recv = __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, send), 0xB1, 0xF, 0xF, true));  // quad_perm [1,0,3,2]
+        if (b0) v[r] = recv; else v[r + 1] = recv;
+    }
+}
+
 // Epilogue of a wave's 64 x (32 JT) part of C.  D[m][n] of a 32x32 MFMA: lane holds column
 // n = lane % 32; register r holds row 8*(r/4) + 4*(lane/32) + r%4.  When C is accumulated into (ACCUM),
 // its old values are fetched for 32 rows at a time before any of them is overwritten (loads and stores
@@ -252,10 +273,12 @@ __device__ __forceinline__ floatx16 mfma16(const piece& a, const piece& b, float
 // intermediate leaves the binary32 range when the result does not).
 //
 // A wave whose part of C lies wholly inside the matrix (all but the last row and column of tiles) takes
-// the path without bounds tests: the row factors of 32 rows are fetched together, then the stores of
-// those rows follow one another with nothing to wait for in between.  (With a load and a wait in front
-// of every row's stores - the vector-memory counter counts stores as well - the epilogue of a tile took
-// 33 000 cycles, a seventh of the product with 4096 values of k.)
+// the path without bounds tests and with 16-byte stores: a store instruction costs the texture path about
+// 32 cycles whatever it carries, and with one 4-byte store per accumulator register (1024 per tile and
+// CU) the epilogue of a tile took 33 000 cycles, a seventh of a product with 4096 values of k.  Four
+// registers of a lane are four rows of one column; a 4 x 4 transpose inside every quad of lanes (DPP
+// quad_perm, 16 vector instructions) turns them into four columns of one row, i.e. one 16-byte store,
+// and a store instruction then writes eight whole 128-byte lines.
 template <bool ACCUM, int JT, bool SCALED = false>
 __device__ __forceinline__ void store_c(const floatx16 (&acc)[2][JT], float* __restrict__ C, uint64_t ldc, uint64_t M,
                                         uint64_t N, uint64_t row_base, uint64_t col0, int h, float alpha, float beta,
@@ -265,36 +288,34 @@ __device__ __forceinline__ void store_c(const floatx16 (&acc)[2][JT], float* __r
     // wave-uniform: col0 = first column of the wave's part + lane % 32
     const bool inside = row_base + 64 <= M && col0 - (threadIdx.x & 31) + 32 * JT <= N;
     if (!SCALED && inside) {
+        const int lane = threadIdx.x & 63, q = lane & 3;
 #pragma unroll
         for (int i = 0; i < 2; ++i) {
-            const uint64_t row0 = row_base + 32 * i + 4 * h;
-            float* p = C + row0 * ldc + col0;
-            float rs[16];
 #pragma unroll
-            for (int r = 0; r < 16; ++r) rs[r] = row_scale ? row_scale[row0 + 8 * (r >> 2) + (r & 3)] : 1.0f;
-            // old values of C: two 32-column groups at a time (32 registers), fetched before they are overwritten
-            constexpr int JG = ACCUM ? (JT + 1) / 2 : JT;
-#pragma unroll
-            for (int j0 = 0; j0 < JT; j0 += JG) {
-                floatx16 prev[ACCUM ? JG : 1];
+            for (int g = 0; g < 4; ++g) {
+                // registers 4g .. 4g+3 are rows 8g + 4h + (0..3) of the lane's column; after the transpose inside
+                // the quad the lane holds row 8g + 4h + q, columns 4 (x / 4) .. + 3 of every 32-column group
+                const uint64_t row = row_base + 32 * i + 8 * g + 4 * h + q;
+                const float rs = row_scale ? row_scale[row] : 1.0f;
+                float* p = C + row * ldc + (col0 - q);
+                float4u prev[ACCUM ? JT : 1];
                 if constexpr (ACCUM) {
 #pragma unroll
-                    for (int j = 0; j < JG; ++j)
-#pragma unroll
-                        for (int r = 0; r < 16; ++r)
-                            if (j0 + j < JT) prev[j][r] = p[(uint64_t)(8 * (r >> 2) + (r & 3)) * ldc + 32 * (j0 + j)];
+                    for (int j = 0; j < JT; ++j) prev[j] = *reinterpret_cast<const float4u*>(p + 32 * j);
                 }
 #pragma unroll
-                for (int r = 0; r < 16; ++r) {
-                    float* q = p + (uint64_t)(8 * (r >> 2) + (r & 3)) * ldc;
+                for (int j = 0; j < JT; ++j) {
+                    float v[4] = {acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]};
+                    quad_transpose(v, lane);
+                    float4u o;
 #pragma unroll
-                    for (int j = 0; j < JG; ++j) {
-                        if (j0 + j >= JT) continue;
+                    for (int c = 0; c < 4; ++c) {
                         if constexpr (ACCUM)
-                            q[32 * (j0 + j)] = (alpha * acc[i][j0 + j][r] + beta * prev[j][r]) * rs[r];
+                            o[c] = (alpha * v[c] + beta * prev[j][c]) * rs;
                         else
-                            q[32 * (j0 + j)] = alpha * acc[i][j0 + j][r] * rs[r];
+                            o[c] = alpha * v[c] * rs;
                     }
+                    *reinterpret_cast<float4u*>(p + 32 * j) = o;
                 }
             }
         }
