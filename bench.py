@@ -16,8 +16,12 @@ cpu_baseline = the CPU restatement of trak's BasicProjector (oracle/basic_projec
 sustained = the same calls back to back for --sustain seconds (default 2).
 `scoring` = BasicScoreComputer at N=50_000, M=10_000, k=4096 fp32: GEMM TFLOP/s against the fp32
             MFMA peak, the SPD inverse separately, and a CPU sample beside it.
-`--only NAME` runs one workload alone (for profiler runs): c1 | c2 | c3_b64 | c3_normal_b32 | c3_normal_b64 | c3_dict | c4 | c4_rademacher | vendor_gemm |
-            scoring | mfma_rate.
+other_configs = whole calls (Python wrapper included) of the other benchmark configurations: c1 (fp32
+            [16, 1_048_576] -> 512), c2 (ResNet-9-sized), c4 (BERT-sized chunked normal), the headline shape as
+            a gradient dict, and projection dimensions 3072 and 15 360.
+`--only NAME` runs one workload alone (for profiler runs): c1 | c2 | c3_b40 | c3_b48 | c3_b64 | c3_k1536 | c3_k3072 |
+            c3_k15360 | c3_k40960 | c3_normal_b32 | c3_normal_b64 | c3_dict | c4 | c4_rademacher | vendor_gemm | scoring |
+            mfma_rate.
 """
 import argparse
 import ctypes
@@ -267,6 +271,15 @@ def _config_calls(torch, dev, name):
         g = (torch.randn(64, P, generator=gen, device=dev) * 1e-3).half()
         p = CudaProjector(P, 4096, 7, ProjectionType.rademacher, dev, 32)
         return (lambda: p.project(g, 0)), 2.0 * 64 * P * 4096, "fp16 rademacher [64,11689512] -> 4096 (one pass of 64 rows)"
+    if name in ("c3_k1536", "c3_k3072", "c3_k15360", "c3_k40960", "c3_b40", "c3_b48"):
+        # the benchmark shape at other projection dimensions (the reference's tests use 15 360, its
+        # documentation recommends 1 000 - 40 000) and at batch sizes between one and two 32-row blocks
+        P = sum(math.prod(sh) for sh in resnet18_param_shapes())
+        k = int(name[4:]) if name[3] == "k" else 4096
+        B = int(name[4:]) if name[3] == "b" else 32
+        g = (torch.randn(B, P, generator=gen, device=dev) * 1e-3).half()
+        p = CudaProjector(P, k, 7, ProjectionType.rademacher, dev, 32)
+        return (lambda: p.project(g, 0)), 2.0 * B * P * k, f"fp16 rademacher [{B},{P}] -> {k}"
     if name in ("c3_normal_b32", "c3_normal_b64"):
         B = int(name[-2:])
         P = sum(math.prod(sh) for sh in resnet18_param_shapes())
@@ -297,9 +310,19 @@ def _config_calls(torch, dev, name):
     raise ValueError(f"unknown configuration {name}")
 
 
-def bench_config(torch, dev, name, reps):
+def bench_config(torch, dev, name, reps, warm_seconds=0.1, min_seconds=0.25):
+    """Whole calls back to back: at least `warm_seconds` of untimed calls first (the clocks of an idle GPU take
+    tens of milliseconds to come up), then at least `reps` calls and `min_seconds` between two events."""
     call, flop, what = _config_calls(torch, dev, name)
     call()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    call()
+    torch.cuda.synchronize()
+    one = max(time.perf_counter() - t0, 1e-5)
+    for _ in range(min(2000, int(warm_seconds / one))):
+        call()
+    reps = max(reps, min(5000, int(min_seconds / one)))
     torch.cuda.synchronize()
     a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     a.record()
@@ -308,7 +331,7 @@ def bench_config(torch, dev, name, reps):
     b.record()
     torch.cuda.synchronize()
     ms = a.elapsed_time(b) / reps
-    return {"what": what, "ms": ms, "tflops": flop / ms / 1e9}
+    return {"what": what, "ms": ms, "tflops": flop / ms / 1e9, "calls": reps}
 
 
 MFMA_RATE_CASES = [
@@ -348,8 +371,10 @@ def bench_mfma_rate(torch, dev, iters=300_000):
     clock is power limited, so the rate depends on the data): the reference point for the projection
     and GEMM kernels.  One dispatch per case, timed with events on the launch stream."""
     path = os.path.join(ROOT, "trak_amd", "libtrakhip_diag.so")
-    if not os.path.exists(path):
-        raise ImportError(f"{path} is missing: build it with `python -m trak_amd.build`")
+    if not os.path.exists(path):  # not part of the product build: made when this workload asks for it
+        from trak_amd.build import build_diag
+
+        build_diag(verbose=False)
     lib = ctypes.CDLL(path)
     lib.trakhip_diag_mfma_rate_out_floats.restype = ctypes.c_size_t
     lib.trakhip_diag_mfma_rate.restype = ctypes.c_double
@@ -371,13 +396,30 @@ def bench_mfma_rate(torch, dev, iters=300_000):
     return res
 
 
-def bench_other_configs(torch, dev):
-    """Throughput of the other projection configurations (the CPU-runnable fp32 case, the
-    ResNet-9-sized case and the BERT-sized chunked normal case); not part of the default line,
-    `--all-configs` prints them to stderr."""
+OTHER_CONFIGS = (
+    # name, timed calls, what bounds the kernel (the peak its TFLOP/s is a fraction of)
+    ("c1", 200, "bf16 MFMA (fp32 gradients split exactly into three bf16 terms: three MFMAs per step)"),
+    ("c2", 100, "fp16 MFMA"),
+    ("c3_dict", 10, "fp16 MFMA"),
+    ("c3_k3072", 10, "fp16 MFMA"),
+    ("c3_k15360", 6, "fp16 MFMA"),
+    ("c4", 3, "vector ALU (a normal entry costs about 8 issue slots and is used for 32 multiply-adds); "
+              "fraction of the fp16 MFMA peak given for comparison"),
+)
+
+
+def bench_other_configs(torch, dev, names=None):
+    """Whole-call throughput (Python wrapper included) of the other benchmark configurations - the
+    CPU-runnable fp32 case, the ResNet-9-sized case, the BERT-sized chunked normal case -, of the
+    headline shape given as a gradient dict, and of projection dimensions whose column-block count
+    does not divide the CU count."""
     res = {}
-    for name, reps in (("c1", 50), ("c2", 30), ("c4", 3), ("c4_rademacher", 5)):
-        res[name] = bench_config(torch, dev, name, reps)
+    for name, reps, bound in OTHER_CONFIGS:
+        if names is not None and name not in names:
+            continue
+        r = bench_config(torch, dev, name, reps)
+        res[name] = {"what": r["what"], "ms": round(r["ms"], 4), "tflops": round(r["tflops"], 1),
+                     "frac_fp16_mfma_peak": round(r["tflops"] / PEAK_FP16_TFLOPS, 4), "bound": bound, "calls": r["calls"]}
         torch.cuda.empty_cache()
     return res
 
@@ -618,11 +660,14 @@ def main():
                     help="also time the BERT-sized normal configuration's BasicProjector sample on the CPU (about a minute)")
     ap.add_argument("--no-scoring", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--no-other-configs", action="store_true",
+                    help="skip the other projection configurations (`other_configs` of the JSON line)")
     ap.add_argument("--all-configs", action="store_true",
-                    help="also time the other projection configurations and print them to stderr")
+                    help="also time the featurize / store paths and batch scaling and print them to stderr")
     ap.add_argument("--only", default=None, metavar="NAME",
                     help="run just one workload for --steps calls and print its timing (for profiler runs): "
-                         "c1 | c2 | c3_b64 | c3_normal_b32 | c3_normal_b64 | c3_dict | c4 | c4_rademacher | scoring | mfma_rate | vendor_gemm "
+                         "c1 | c2 | c3_b40 | c3_b48 | c3_b64 | c3_k1536 | c3_k3072 | c3_k15360 | c3_k40960 | c3_normal_b32 | "
+                         "c3_normal_b64 | c3_dict | c4 | c4_rademacher | scoring | mfma_rate | vendor_gemm "
                          "(torch.mm on the scoring operands, for comparison)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run one 1 GiB device-to-device copy (reference point for rocprofv3 byte counters)")
@@ -656,8 +701,9 @@ def main():
         return
     proj = bench_projection(torch, dev, args.steps, args.warmup, args.batches, args.sustain)
     torch.cuda.empty_cache()
+    other = None if args.no_other_configs else bench_other_configs(torch, dev)
     if args.all_configs:
-        print(json.dumps(bench_other_configs(torch, dev), indent=1), file=sys.stderr)
+        print(json.dumps(bench_config(torch, dev, "c4_rademacher", 5), indent=1), file=sys.stderr)
         print(json.dumps({"featurize_path": bench_featurize_path(torch, dev)}, indent=1), file=sys.stderr)
         print(json.dumps({"batch_scaling": bench_batch_scaling(torch, dev)}, indent=1), file=sys.stderr)
         torch.cuda.empty_cache()
@@ -702,6 +748,7 @@ def main():
             "kernel_ms_min": round(proj["kernel_ms_min"], 4),
         },
         "sustained": proj["sustained"],
+        "other_configs": other,
         "cpu_baseline": cpu,
         "scoring": scoring,
     }

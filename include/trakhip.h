@@ -53,7 +53,9 @@ int trakhip_abi_version(void);
 /* ---- JL projection -------------------------------------------------------------------- */
 
 /* Bytes of scratch a caller should bring to trakhip_project for these sizes: room for passes of
- * trakhip_project_rows_per_pass() = 64 rows.  Stands in for the torch::zeros({B_pad, T, N})
+ * trakhip_project_rows_per_pass() = 64 rows.  The size depends on the shape and on the number of compute
+ * units of the current HIP device (the launch is cut into at most that many workgroups; 256 is assumed
+ * when the process has no device), so ask with the device current that will run the projection.  Stands in for the torch::zeros({B_pad, T, N})
  * intermediate of fast_jl/fast_jl.cu:48-49.  trakhip_project_workspace_min: the least that
  * trakhip_project accepts (passes of 32 rows: half as much once B >= 64; the call then runs 32 rows
  * at a time, with the same results). */
@@ -85,9 +87,11 @@ int trakhip_project(const void* in_dev, int in_dtype, uint64_t B, uint64_t P, ui
  * fast_jl allocates its intermediate with torch::zeros on every call (fast_jl/fast_jl.cu:48-49).
  * Same arguments, checks and results (bit for bit) as trakhip_project, minus the workspace: the
  * partial sums live in a static device array of trakhip_project_static_limit() bytes (36 MiB) that
- * each GPU the library runs on holds until the process ends (rows go 32 at a time).  A shape whose
+ * each GPU the library runs on holds until the process ends (rows go 64 at a time when the partial
+ * sums of a 64-row pass fit into the array, else 32 at a time; same results either way).  A shape whose
  * trakhip_project_workspace_min() exceeds that is refused with TRAKHIP_ERR_STATIC_LIMIT (every shape
- * with proj_dim <= 65536 fits).  Calls no hipMalloc / hipFree or any allocating routine.  All calls
+ * with proj_dim <= 262144 fits: a launch never has more partial blocks of 1024 columns than the device
+ * has compute units).  Calls no hipMalloc / hipFree or any allocating routine.  All calls
  * on one GPU share the one array: calls that overlap in time on the same GPU (different streams
  * or threads) race and give wrong results; calls that follow one another on a stream do not. */
 size_t trakhip_project_static_limit(void);

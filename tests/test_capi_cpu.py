@@ -68,15 +68,17 @@ def test_static_entry_point_validates_before_touching_the_device():
     assert lib.trakhip_project_static_limit() == 36 << 20
     assert call(k=100) == -1 and call(B=0) == -2 and call(dtype=5) == -3 and call(pt=9) == -4
     assert call(inp=None) == -5 and call(out=None) == -5 and call(out=ctypes.c_void_p(4100)) == -7
-    # two runs of 150 column blocks: 37.5 MiB of partial sums, more than the 36 MiB array
-    assert lib.trakhip_project_workspace(32, 1024, 153_600, 2) == 2 * 32 * 153_600 * 4
-    assert call(k=153_600) == -12
+    # 300 column blocks are more than the 256 CUs: one run, 37.5 MiB of partial sums, more than the 36 MiB array
+    assert lib.trakhip_project_workspace(32, 1024, 307_200, 2) == 32 * 307_200 * 4
+    assert call(k=307_200) == -12
+    assert lib.trakhip_project_workspace_min(64, 1024, 262_144, 2) == 32 << 20  # the largest below that
     assert "static" in _lib.strerror(-12)
 
 
 def test_workspace_size():
     lib = _lib.load()
-    # G * min(B, 32) * k floats, G = number of feature runs (about 512 workgroups / (k / 512))
+    # G * min(B, 64) * k floats, G = runs of consecutive feature chunks = floor(256 CUs / column blocks),
+    # at most one per chunk (no device in this process: the library assumes the 256 CUs of an MI355X)
     assert lib.trakhip_project_workspace(32, 11_689_512, 4096, 256) == 64 * 32 * 4096 * 4
     assert lib.trakhip_project_workspace(48, 1000, 512, 256) == 256 * 48 * 512 * 4      # 256 tiles x 1 chunk
     assert lib.trakhip_project_workspace_min(48, 1000, 512, 256) == 256 * 32 * 512 * 4
@@ -89,6 +91,10 @@ def test_workspace_size():
     assert lib.trakhip_project_workspace(8, 25, 1024, 256) == 25 * 8 * 1024 * 4
     assert lib.trakhip_project_workspace(16, 1_048_576, 512, 256) == 256 * 16 * 512 * 4  # one 512-column block
     assert lib.trakhip_project_workspace(0, 25, 1024, 256) == 0
+    # column-block counts that do not divide 256: never more workgroups than CUs
+    for k, blocks in ((1536, 3), (3072, 3), (5120, 5), (15_360, 15), (40_960, 40)):
+        groups = 256 // blocks
+        assert lib.trakhip_project_workspace(32, 11_689_512, k, 256) == groups * 32 * k * 4, k
     assert lib.trakhip_spd_inverse_workspace(4096) >= 3 * 4096 * 4096 * 4
     assert lib.trakhip_spd_inverse_workspace(100) >= 3 * 128 * 128 * 4
 

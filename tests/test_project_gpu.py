@@ -474,7 +474,7 @@ def test_full_size_bert_normal_chunked_shape(gpu, c_oracle):
 # ---- the reference's uint32-overflow shapes (tests/test_jl.py:59-73, tests/test_jl_additional.py:11-44) ----
 
 
-@pytest.mark.parametrize("shape", [(8, 180_645_096), (31, 180_645_096), (2, 780_645_096)])
+@pytest.mark.parametrize("shape", [(8, 180_645_096), (31, 180_645_096), (32, 180_645_096), (2, 780_645_096)])
 def test_uint32_overflow_shapes_through_chunks(gpu, c_oracle, shape):
     # B * P >= 2^31 / 2^32: the reference's kernel indexes with uint32 `row * features`
     # (fast_jl/data_loading.cuh:37-41) and therefore chunks P; here addressing is 64-bit, and the

@@ -35,9 +35,10 @@ def _project(lib, x, k, seed, tiles, pt, static):
 def test_static_entry_point_equals_workspace_entry_point_twice(gpu, pt):
     lib = _lib.load()
     gen = torch.Generator(device="cpu").manual_seed(5)
-    # first call: 40 rows (two passes of 32 + 8 through the array, against one 40-row pass with the workspace),
-    # ragged P; second: smaller in every way
-    shapes = [(40, 300_001, 1024, torch.float16), (7, 20_011, 512, torch.float32)]
+    # first call: 40 rows (two passes of 32 + 8 through the array - a 40-row pass would need 40 MiB -, against
+    # one 40-row pass with the workspace), ragged P; second: smaller in every way; third: 70 rows whose 64-row
+    # pass fits into the array (64 + 6, the same passes as with the workspace)
+    shapes = [(40, 300_001, 1024, torch.float16), (7, 20_011, 512, torch.float32), (70, 50_001, 512, torch.bfloat16)]
     for B, P, k, dt in shapes:
         x = (torch.randn(B, P, generator=gen) * 1e-2).to(dt).to(gpu)
         want = _project(lib, x, k, 11, 256, pt, static=False)
@@ -50,9 +51,9 @@ def test_static_entry_point_limit_and_validation(gpu):
     lib = _lib.load()
     assert lib.trakhip_project_static_limit() == 36 << 20
     x = torch.zeros(32, 1024, dtype=torch.float16, device=gpu)
-    out = torch.zeros(32, 153_600, dtype=torch.float32, device=gpu)
+    out = torch.zeros(32, 307_200, dtype=torch.float32, device=gpu)
     args = lambda k, tiles: (ctypes.c_void_p(x.data_ptr()), _lib.F16, 32, 1024, 1024, ctypes.c_void_p(out.data_ptr()),
                              k, 0, tiles, 0, None)
-    assert lib.trakhip_project_workspace(32, 1024, 153_600, 2) > 36 << 20
-    assert lib.trakhip_project_static(*args(153_600, 2)) == -12
+    assert lib.trakhip_project_workspace(32, 1024, 307_200, 2) > 36 << 20
+    assert lib.trakhip_project_static(*args(307_200, 2)) == -12
     assert lib.trakhip_project_static(*args(100, 2)) == -1

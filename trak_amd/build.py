@@ -1,6 +1,8 @@
 """Builds trak_amd/libtrakhip.so from trak_amd/csrc/*.hip with hipcc for gfx950.
 
 Run as `python -m trak_amd.build`.  hipcc cross-compiles, so no GPU is needed to build.
+`python -m trak_amd.build --diag` also builds libtrakhip_diag.so, the measurement aid behind
+`bench.py --only mfma_rate` (not part of the product library; bench.py builds it when it is asked for).
 """
 import os
 import subprocess
@@ -25,7 +27,15 @@ FLAGS = [
 ]
 
 
-def build(verbose=True, jobs=4):
+# hipcc's host pass does not know the device-only target feature and says so once per source: noise
+_KNOWN_NOISE = "'-packed-fp32-ops' is not a recognized feature for this target (ignoring feature)"
+
+
+def _without_noise(text):
+    return "\n".join(l for l in text.splitlines() if l.strip() != _KNOWN_NOISE)
+
+
+def build(verbose=True, jobs=4, diag=False):
     """Compile every source to an object (in parallel) and link the shared library."""
     hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
     objdir = os.path.join(HERE, "build")
@@ -46,25 +56,31 @@ def build(verbose=True, jobs=4):
     if verbose:
         print(" ".join(cmd), flush=True)
     subprocess.check_call(cmd)
+    if diag:
+        build_diag(verbose)
+    return LIB
+
+
+def build_diag(verbose=True):
+    """The measurement aid (a loop of nothing but MFMAs, for `bench.py --only mfma_rate`)."""
+    hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
     cmd = [hipcc, *FLAGS, "-shared", "-o", DIAG_LIB, *[os.path.join(CSRC, s) for s in DIAG_SOURCES]]
     if verbose:
         print(" ".join(cmd), flush=True)
     out = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT)
-    text = "\n".join(l for l in out.stdout.decode(errors="replace").splitlines() if "packed-fp32-ops" not in l)
+    text = _without_noise(out.stdout.decode(errors="replace"))
     if text.strip():
         print(text)
     if out.returncode != 0:
         raise RuntimeError("hipcc failed on the measurement aid")
-    return LIB
+    return DIAG_LIB
 
 
 def _drain(procs):
     while procs:
         src, p = procs.pop(0)
         out, _ = p.communicate()
-        text = out.decode(errors="replace")
-        # hipcc's host pass does not know the device-only target feature; that line is noise
-        text = "\n".join(l for l in text.splitlines() if "packed-fp32-ops" not in l)
+        text = _without_noise(out.decode(errors="replace"))
         if text.strip():
             print(text)
         if p.returncode != 0:
@@ -72,6 +88,6 @@ def _drain(procs):
 
 
 if __name__ == "__main__":
-    build()
+    build(diag="--diag" in sys.argv[1:])
     print(LIB)
     sys.exit(0)

@@ -445,15 +445,22 @@ struct StageOf<TRAKHIP_F32, true, W, ROWS> {
 
 // ---- Rademacher projection -------------------------------------------------------------------
 
-// Workgroup id -> (column block, tile).  Workgroups are handed to the 8 XCDs round-robin
-// by linear id; this puts the column blocks of one feature tile on the same XCD, next to
-// each other in time, so the tile is fetched from HBM once and then served by that XCD's L2.
-__device__ __forceinline__ void map_workgroup(uint32_t linear, uint32_t col_blocks, uint32_t& cb,
-                                              uint32_t& tile) {
-    const uint32_t xcd = linear & 7u;
-    const uint32_t idx = linear >> 3;
-    cb = idx % col_blocks;
-    tile = (idx / col_blocks) * 8u + xcd;
+// Workgroup id -> (column block, run of chunks).  The units u = run * col_blocks + column block are
+// numbered so that the column blocks of one run are neighbours, and the 8 XCDs - which are handed
+// the workgroups round-robin by linear id - each take a contiguous eighth of them: the column
+// blocks of a run then sit on the same XCD at the same time (a run cut by the border between two
+// eighths sits on two), so a gradient chunk is fetched from HBM once and then served by that XCD's
+// L2.  The launch has 8 * ceil(units / 8) workgroups; false = padding, nothing to do.
+__device__ __forceinline__ bool map_workgroup(uint32_t linear, uint32_t col_blocks, uint32_t groups, uint32_t& cb,
+                                              uint32_t& group) {
+    const uint32_t xcd = linear & 7u, idx = linear >> 3;
+    const uint64_t units = (uint64_t)groups * col_blocks;
+    const uint32_t lo = (uint32_t)(xcd * units / 8u), hi = (uint32_t)((xcd + 1u) * units / 8u);
+    const uint32_t u = lo + idx;
+    if (u >= hi) return false;
+    group = u / col_blocks;
+    cb = u - group * col_blocks;
+    return true;
 }
 
 // The B operand of one MFMA is eight signs = one byte of a Philox block, looked up in LDS:
@@ -528,7 +535,7 @@ template <int IN, bool GATHER, int GPW, int RB>
 __global__ __launch_bounds__(512) void jl_project_kernel(
     const void* __restrict__ g_in, uint64_t ld, uint32_t rows, uint64_t P, uint32_t k,
     uint32_t seed, uint32_t tiles, uint64_t tile_size, uint32_t chunks_per_tile,
-    uint32_t chunks_per_group, float* __restrict__ partial) {
+    uint32_t chunks_per_group, uint32_t groups, float* __restrict__ partial) {
     constexpr int W = 8;
     typedef InTraits<IN> Tr;
     typedef typename StageOf<IN, GATHER, W, 32 * RB>::type Stage;
@@ -555,12 +562,12 @@ __global__ __launch_bounds__(512) void jl_project_kernel(
 
     const uint32_t col_blocks = k / kColsPerWG;
     uint32_t cb, group;
-    map_workgroup(blockIdx.x, col_blocks, cb, group);
+    if (!map_workgroup(blockIdx.x, col_blocks, groups, cb, group)) return;
     // this workgroup's share of the flattened (tile, chunk) sequence; the streams are counter
     // based, so a workgroup can start in the middle of a tile
     const uint64_t total_chunks = (uint64_t)tiles * chunks_per_tile;
     const uint64_t c_begin = (uint64_t)group * chunks_per_group;
-    if (c_begin >= total_chunks) return;  // padding of the group count to a multiple of 8
+    if (c_begin >= total_chunks) return;  // (the plan leaves no empty run)
     const uint64_t c_end = c_begin + chunks_per_group < total_chunks ? c_begin + chunks_per_group : total_chunks;
     const uint32_t t0 = (uint32_t)(c_begin / chunks_per_tile), s0 = (uint32_t)(c_begin % chunks_per_tile);
 
@@ -987,7 +994,7 @@ __device__ __forceinline__ uint32_t normal_pair(uint32_t w, const char* r_tab, c
 template <int IN, bool GATHER, int GPW, int RB>
 __global__ __launch_bounds__(512) void jl_project_normal_kernel(
     const void* __restrict__ g_in, uint64_t ld, uint32_t rows, uint64_t P, uint32_t k, uint32_t seed,
-    uint32_t tiles, uint64_t tile_size, uint32_t chunks_per_tile, uint32_t chunks_per_group,
+    uint32_t tiles, uint64_t tile_size, uint32_t chunks_per_tile, uint32_t chunks_per_group, uint32_t groups,
     float* __restrict__ partial) {
     constexpr int W = 8;
     typedef NormalTraits<IN> Tr;
@@ -1015,10 +1022,10 @@ __global__ __launch_bounds__(512) void jl_project_normal_kernel(
 
     const uint32_t col_blocks = k / kColsPerWG;
     uint32_t cb, group;
-    map_workgroup(blockIdx.x, col_blocks, cb, group);
+    if (!map_workgroup(blockIdx.x, col_blocks, groups, cb, group)) return;
     const uint64_t total_chunks = (uint64_t)tiles * chunks_per_tile;
     const uint64_t c_begin = (uint64_t)group * chunks_per_group;
-    if (c_begin >= total_chunks) return;  // padding of the group count to a multiple of 8
+    if (c_begin >= total_chunks) return;  // (the plan leaves no empty run)
     const uint64_t c_end = c_begin + chunks_per_group < total_chunks ? c_begin + chunks_per_group : total_chunks;
     const uint32_t t0 = (uint32_t)(c_begin / chunks_per_tile), s0 = (uint32_t)(c_begin % chunks_per_tile);
     const uint32_t t_last = (uint32_t)((c_end - 1) / chunks_per_tile);
@@ -1174,48 +1181,61 @@ __global__ __launch_bounds__(512) void jl_project_normal_kernel(
     }
 }
 
-// out[b, c] = scale * sum over tile groups, in group order.
+// out[b, c] = scale * sum over the runs (tile groups) of their partial sums, in a fixed order: eight
+// running sums over the runs g = u (mod 8), each in increasing g, combined as
+// ((s0 + s1) + (s2 + s3)) + ((s4 + s5) + (s6 + s7)) - the result depends on the shape only.
+// Eight neighbouring lanes share one output quad (four consecutive columns of a row), lane u holding
+// s_u: a launch has 8 * B * k / 4 threads (with one thread per quad the CPU-runnable configuration had
+// eight workgroups on 256 CUs and took 20 us for 8 MB).  kReduceThreads = 64: one wave per workgroup.
+constexpr int kReduceThreads = 64;
 template <int OUT_DTYPE>
-__global__ __launch_bounds__(256) void jl_reduce_kernel(const float* __restrict__ partial,
-                                                        uint32_t groups, uint64_t n4, uint32_t k4,
-                                                        float scale, void* __restrict__ out,
-                                                        uint64_t ld_out) {
-    const uint64_t i = (uint64_t)blockIdx.x * 256 + threadIdx.x;
+__global__ __launch_bounds__(kReduceThreads) void jl_reduce_kernel(const float* __restrict__ partial,
+                                                                   uint32_t groups, uint64_t n4, uint32_t k4,
+                                                                   float scale, void* __restrict__ out,
+                                                                   uint64_t ld_out) {
+    const uint64_t t = (uint64_t)blockIdx.x * kReduceThreads + threadIdx.x;
+    const uint64_t i = t >> 3;  // n4 is a multiple of 128 (k of 512): every wave is full
+    const uint32_t u = (uint32_t)t & 7u;
     if (i >= n4) return;
     const float4* p = reinterpret_cast<const float4*>(partial) + i;
-    // eight running sums over groups g = u (mod 8) keep eight loads in flight; they are combined
-    // in a fixed order, so the result depends only on the shape
-    float4 s[8];
-#pragma unroll
-    for (int u = 0; u < 8; ++u) s[u] = {0.f, 0.f, 0.f, 0.f};
-    uint32_t g = 0;
-    for (; g + 8 <= groups; g += 8) {
+    float4 s = {0.f, 0.f, 0.f, 0.f};
+    uint32_t g = u;
+    for (; g + 56 < groups; g += 64) {  // eight loads in flight
         float4 v[8];
 #pragma unroll
-        for (int u = 0; u < 8; ++u) v[u] = p[(uint64_t)(g + u) * n4];
+        for (int j = 0; j < 8; ++j) v[j] = p[(uint64_t)(g + 8 * j) * n4];
 #pragma unroll
-        for (int u = 0; u < 8; ++u) {
-            s[u].x += v[u].x;
-            s[u].y += v[u].y;
-            s[u].z += v[u].z;
-            s[u].w += v[u].w;
+        for (int j = 0; j < 8; ++j) {
+            s.x += v[j].x;
+            s.y += v[j].y;
+            s.z += v[j].z;
+            s.w += v[j].w;
         }
     }
+    {
+        float4 v[8];
 #pragma unroll
-    for (int u = 0; u < 7; ++u) {
-        if (g + u < groups) {
-            const float4 v = p[(uint64_t)(g + u) * n4];
-            s[u].x += v.x;
-            s[u].y += v.y;
-            s[u].z += v.z;
-            s[u].w += v.w;
+        for (int j = 0; j < 8; ++j) v[j] = (g + 8 * j < groups) ? p[(uint64_t)(g + 8 * j) * n4] : float4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            if (g + 8 * j < groups) {
+                s.x += v[j].x;
+                s.y += v[j].y;
+                s.z += v[j].z;
+                s.w += v[j].w;
+            }
         }
     }
-    float4 r;
-    r.x = ((s[0].x + s[1].x) + (s[2].x + s[3].x)) + ((s[4].x + s[5].x) + (s[6].x + s[7].x));
-    r.y = ((s[0].y + s[1].y) + (s[2].y + s[3].y)) + ((s[4].y + s[5].y) + (s[6].y + s[7].y));
-    r.z = ((s[0].z + s[1].z) + (s[2].z + s[3].z)) + ((s[4].z + s[5].z) + (s[6].z + s[7].z));
-    r.w = ((s[0].w + s[1].w) + (s[2].w + s[3].w)) + ((s[4].w + s[5].w) + (s[6].w + s[7].w));
+    // lane 0 of each eight ends up with the sum in the order stated above (own value first in every step)
+#pragma unroll
+    for (int d = 1; d < 8; d <<= 1) {
+        s.x += __shfl_xor(s.x, d, 64);
+        s.y += __shfl_xor(s.y, d, 64);
+        s.z += __shfl_xor(s.z, d, 64);
+        s.w += __shfl_xor(s.w, d, 64);
+    }
+    if (u != 0) return;
+    float4 r = s;
     r.x *= scale;
     r.y *= scale;
     r.z *= scale;
@@ -1241,11 +1261,33 @@ __global__ __launch_bounds__(256) void jl_materialize_kernel(uint32_t seed, uint
                                                : jl::entry_normal(seed, c, tile, o);
 }
 
+// Compute units of the current device, asked once per device.  256 (MI355X) where no device can be
+// asked, so that the workspace functions still answer in a process without a GPU.
+constexpr int kMaxDevices = 64;
+constexpr uint32_t kDefaultCus = 256;
+uint32_t device_cus() {
+    static std::atomic<uint32_t> cached[kMaxDevices];
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return kDefaultCus;
+    uint32_t n = cached[dev].load(std::memory_order_relaxed);
+    if (!n) {
+        int v = 0;
+        if (hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || v <= 0)
+            v = (int)kDefaultCus;
+        n = (uint32_t)v;
+        cached[dev].store(n, std::memory_order_relaxed);
+    }
+    return n;
+}
+
 // How a launch is cut into workgroups.  The (tile, chunk) pairs of all feature tiles form one
 // sequence of tiles * chunks_per_tile chunks; every workgroup takes chunks_per_group consecutive
 // ones (adding their products in its accumulators) for one block of 1024 columns (512 when the
-// projection dimension is an odd multiple of 512).  The split depends only on the shape, so results
-// are reproducible; it aims at one workgroup of 8 waves per CU.
+// projection dimension is an odd multiple of 512).  A workgroup of these kernels has a CU to itself
+// (8 waves, 99-133 KB of LDS), so the launch must not have more workgroups than the device has CUs:
+// the extra ones would start when the first ones end, and the launch would take two workgroup
+// lifetimes.  groups = floor(CUs / column blocks), at least 1.  The split depends on the shape and the
+// device's CU count only, so results are reproducible.
 struct Plan {
     jl::Tiling tl;
     uint32_t gpw, col_blocks, chunks_per_tile, chunks_per_group, groups;  // gpw: 32-column groups per wave
@@ -1258,8 +1300,7 @@ Plan make_plan(uint64_t P, uint32_t k, uint32_t num_feature_tiles) {
     p.col_blocks = k / (8 * p.gpw * 32);
     p.chunks_per_tile = (uint32_t)((p.tl.tile_size + kChunk - 1) / kChunk);
     const uint64_t total = (uint64_t)p.tl.tiles * p.chunks_per_tile;
-    const uint64_t target_wgs = 256;  // one workgroup of 8 waves per CU
-    uint64_t groups = (target_wgs + p.col_blocks - 1) / p.col_blocks;
+    uint64_t groups = device_cus() / p.col_blocks;
     if (groups > total) groups = total;
     if (groups < 1) groups = 1;
     p.chunks_per_group = (uint32_t)((total + groups - 1) / groups);
@@ -1267,11 +1308,13 @@ Plan make_plan(uint64_t P, uint32_t k, uint32_t num_feature_tiles) {
     return p;
 }
 
+// workgroups of a launch: the units rounded up to a multiple of 8 (see map_workgroup)
+uint64_t plan_workgroups(const Plan& pl) { return ((uint64_t)pl.groups * pl.col_blocks + 7u) / 8u * 8u; }
+
 template <int IN, bool GATHER, int GPW>
 hipError_t launch_rademacher(const void* in, uint64_t ld, uint32_t rows, uint64_t P, uint32_t k, uint32_t seed,
                              const Plan& pl, float* partial, hipStream_t s) {
-    const uint32_t groups8 = (pl.groups + 7u) / 8u * 8u;
-    const uint64_t wgs = (uint64_t)groups8 * pl.col_blocks;
+    const uint64_t wgs = plan_workgroups(pl);
     if (wgs > 0x7FFFFFFFull) return hipErrorInvalidValue;
     if (rows > 32) {
         // two 32-row blocks per pass (16-bit gradients only)
@@ -1279,11 +1322,11 @@ hipError_t launch_rademacher(const void* in, uint64_t ld, uint32_t rows, uint64_
             return hipErrorInvalidValue;
         } else {
             hipLaunchKernelGGL((jl_project_kernel<IN, GATHER, GPW, 2>), dim3((uint32_t)wgs), dim3(512), 0, s, in, ld, rows,
-                               P, k, seed, pl.tl.tiles, pl.tl.tile_size, pl.chunks_per_tile, pl.chunks_per_group, partial);
+                               P, k, seed, pl.tl.tiles, pl.tl.tile_size, pl.chunks_per_tile, pl.chunks_per_group, pl.groups, partial);
         }
     } else {
         hipLaunchKernelGGL((jl_project_kernel<IN, GATHER, GPW, 1>), dim3((uint32_t)wgs), dim3(512), 0, s, in, ld, rows, P,
-                           k, seed, pl.tl.tiles, pl.tl.tile_size, pl.chunks_per_tile, pl.chunks_per_group, partial);
+                           k, seed, pl.tl.tiles, pl.tl.tile_size, pl.chunks_per_tile, pl.chunks_per_group, pl.groups, partial);
     }
     return hipGetLastError();
 }
@@ -1291,8 +1334,7 @@ hipError_t launch_rademacher(const void* in, uint64_t ld, uint32_t rows, uint64_
 template <int IN, bool GATHER, int GPW>
 hipError_t launch_normal(const void* in, uint64_t ld, uint32_t rows, uint64_t P, uint32_t k, uint32_t seed,
                          const Plan& pl, float* partial, hipStream_t s) {
-    const uint32_t groups8 = (pl.groups + 7u) / 8u * 8u;
-    const uint64_t wgs = (uint64_t)groups8 * pl.col_blocks;
+    const uint64_t wgs = plan_workgroups(pl);
     if (wgs > 0x7FFFFFFFull) return hipErrorInvalidValue;
     if (rows > 32) {
         if constexpr (IN == TRAKHIP_F32) {
@@ -1300,12 +1342,12 @@ hipError_t launch_normal(const void* in, uint64_t ld, uint32_t rows, uint64_t P,
         } else {
             hipLaunchKernelGGL((jl_project_normal_kernel<IN, GATHER, GPW, 2>), dim3((uint32_t)wgs), dim3(512), 0, s, in,
                                ld, rows, P, k, seed, pl.tl.tiles, pl.tl.tile_size, pl.chunks_per_tile,
-                               pl.chunks_per_group, partial);
+                               pl.chunks_per_group, pl.groups, partial);
         }
     } else {
         hipLaunchKernelGGL((jl_project_normal_kernel<IN, GATHER, GPW, 1>), dim3((uint32_t)wgs), dim3(512), 0, s, in, ld,
                            rows, P, k, seed, pl.tl.tiles, pl.tl.tile_size, pl.chunks_per_tile, pl.chunks_per_group,
-                           partial);
+                           pl.groups, partial);
     }
     return hipGetLastError();
 }
@@ -1335,7 +1377,6 @@ LaunchFn pick(const Plan& pl, int dtype, int proj_type, bool gather) {
 // Scratch of trakhip_project_static (see project_static below): 36 MiB, enough for every shape with
 // proj_dim <= 65536.
 constexpr size_t kStaticScratchBytes = 36u << 20;
-constexpr int kMaxDevices = 64;
 static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
 static std::atomic<void*> static_scratch_ptr[kMaxDevices];
 
@@ -1421,7 +1462,7 @@ int project_reduce_store(const void* ws, uint64_t B, uint64_t P, uint32_t k, uin
     if (check_destination && !kernel_can_write(out)) return TRAKHIP_ERR_POINTER;
     const uint32_t groups = make_plan(P, k, num_feature_tiles).groups;
     const uint64_t n4 = B * k / 4;
-    const dim3 grid((uint32_t)((n4 + 255) / 256)), block(256);
+    const dim3 grid((uint32_t)((8 * n4 + kReduceThreads - 1) / kReduceThreads)), block(kReduceThreads);
     const float* part = static_cast<const float*>(ws);
     if (out_dtype == TRAKHIP_F32)
         hipLaunchKernelGGL(jl_reduce_kernel<TRAKHIP_F32>, grid, block, 0, s, part, groups, n4, k / 4, scale, out, ld_out);

@@ -5,35 +5,66 @@
 processes per kernel launch; here every variant walks the batch in passes of 64 rows (16-bit
 gradients) or 32 rows (fp32) and the suffix does not change the result.
 """
+import contextlib
 import ctypes
+from collections import OrderedDict
 
 import torch
 
 from . import _lib
 
 _DTYPES = {torch.float16: _lib.F16, torch.bfloat16: _lib.BF16, torch.float32: _lib.F32}
-_workspaces = {}      # (device, stream) -> scratch buffer
+_workspaces = OrderedDict()  # (device, stream) -> scratch buffer, least recently used first
+_WORKSPACE_CACHE = 8         # streams that keep a scratch buffer (tens of MiB each at proj_dim 4096)
 _segment_tables = {}  # (device, stream, rows) -> device table; the key holds every pointer, so a hit is exact
 _SEGMENT_TABLE_CACHE = 16
+_workspace_bytes = {}  # (B, P, N, tiles, device index) -> trakhip_project_workspace(...)
+_NO_CONTEXT = contextlib.nullcontext()
 
 
-def _workspace(device, nbytes):
+def _on(device):
+    """Context that makes `device` current; nothing to do (and nothing to pay) when it already is."""
+    index = device.index if device.index is not None else torch.cuda.current_device()
+    return _NO_CONTEXT if index == torch.cuda.current_device() else torch.cuda.device(device)
+
+
+def _workspace_size(lib, B, P, N, tiles, device):
+    key = (B, P, N, tiles, device.index)
+    n = _workspace_bytes.get(key)
+    if n is None:
+        if len(_workspace_bytes) > 256:
+            _workspace_bytes.clear()
+        n = _workspace_bytes[key] = lib.trakhip_project_workspace(B, P, N, tiles)
+    return n
+
+
+def _workspace(device, nbytes, stream=None):
     """One growing scratch buffer per device and stream (stands in for the per-call torch::zeros of
     fast_jl/fast_jl.cu:48-49): calls on different streams never share scratch, calls on one stream
-    are ordered by the stream."""
-    key = (device, torch.cuda.current_stream(device).cuda_stream)
+    are ordered by the stream.  The buffers of the `_WORKSPACE_CACHE` most recently used streams are
+    kept (a program that keeps making streams does not keep a buffer per stream handle ever seen);
+    `free_workspaces()` releases them all."""
+    if stream is None:
+        stream = torch.cuda.current_stream(device).cuda_stream
+    key = (device, stream)
     buf = _workspaces.get(key)
     if buf is None or buf.numel() < nbytes:
         buf = None
         _workspaces.pop(key, None)
+        while len(_workspaces) >= _WORKSPACE_CACHE:
+            _workspaces.popitem(last=False)
         buf = torch.empty(max(nbytes, 1), dtype=torch.uint8, device=device)
         _workspaces[key] = buf
+    else:
+        _workspaces.move_to_end(key)
     return buf
 
 
 def free_workspaces():
+    """Releases the cached scratch buffers, segment tables and size look-ups."""
     _workspaces.clear()
     _segment_tables.clear()
+    _workspace_bytes.clear()
 
 
 def _segment_table(device, rows):
@@ -74,11 +105,11 @@ def _project(input, N, seed, num_feature_tiles, proj_type, ld=None):
     lib = _lib.load()
     if N <= 0 or N % 512 != 0:
         _lib.check(_lib.ERR_PROJ_DIM)
-    with torch.cuda.device(input.device):
-        out = torch.empty((B, N), dtype=torch.float32, device=input.device)
-        nbytes = lib.trakhip_project_workspace(B, P, N, tiles)
-        ws = _workspace(input.device, nbytes)
-        stream = torch.cuda.current_stream(input.device).cuda_stream
+    device = input.device
+    with _on(device):
+        out = torch.empty((B, N), dtype=torch.float32, device=device)
+        stream = torch.cuda.current_stream(device).cuda_stream
+        ws = _workspace(device, _workspace_size(lib, B, P, N, tiles, device), stream)
         code = lib.trakhip_project(
             ctypes.c_void_p(input.data_ptr()),
             _DTYPES[input.dtype],
@@ -185,10 +216,9 @@ def project_into(source, N, seed, num_feature_tiles, proj_type, out, scale=1.0):
         P = first
     _check_destination(out, B, N, device)
     out_ld = out.stride(0) if B > 1 else N
-    with torch.cuda.device(device):
-        nbytes = lib.trakhip_project_workspace(B, P, N, tiles)
-        ws = _workspace(device, nbytes)
+    with _on(device):
         stream = torch.cuda.current_stream(device).cuda_stream
+        ws = _workspace(device, _workspace_size(lib, B, P, N, tiles, device), stream)
         step = int(lib.trakhip_project_rows_per_pass(_DTYPES[dtype], pt))
         for b0 in range(0, B, step):
             nb = min(step, B - b0)
@@ -221,7 +251,7 @@ def project_gather(tensors, N, seed, num_feature_tiles, proj_type, scale=1.0):
     if not gather_supported(tensors):
         raise RuntimeError("project_gather needs CUDA tensors of one supported dtype, device and batch size")
     t0 = tensors[0]
-    with torch.cuda.device(t0.device):
+    with _on(t0.device):
         out = torch.empty((t0.shape[0], int(N)), dtype=torch.float32, device=t0.device)
     return project_into(tensors, N, seed, num_feature_tiles, proj_type, out, scale)
 
