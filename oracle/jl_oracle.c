@@ -95,8 +95,8 @@ static uint32_t float_to_bits(float f) {
     return b;
 }
 
-/* Radius of a Box-Muller pair for the 15-bit index x: sqrt(-2 ln u) with u = (x + 1/2) / 2^15
- * = (2x + 1) / 2^16, evaluated in binary32 by a fixed sequence of IEEE operations. */
+/* Radius of a Box-Muller pair for the 14-bit index x: sqrt(-2 ln u) with u = (x + 1/2) / 2^14
+ * = (2x + 1) / 2^15, evaluated in binary32 by a fixed sequence of IEEE operations. */
 static float radius_from_index(uint32_t x) {
     uint32_t odd = 2u * x + 1u;
     float xf = (float)odd;
@@ -118,7 +118,7 @@ static float radius_from_index(uint32_t x) {
     float y = t * zp;
     y = fmaf(-0.5f, z, y);
     float ln_m = t + y;
-    float ln_u = fmaf((float)(expo - 16), 0.693147182f, ln_m);
+    float ln_u = fmaf((float)(expo - 15), 0.693147182f, ln_m);
     float s = -2.0f * ln_u;
     float guess = bits_to_float(0x5f3759dfu - (float_to_bits(s) >> 1));
     float half_s = 0.5f * s;
@@ -130,13 +130,16 @@ static float radius_from_index(uint32_t x) {
     return s * guess;
 }
 
-/* cos and sin of the angle (a + 1/2) * (pi/2) / 2^13 for the 13-bit index a.  Angles above pi/4
- * are evaluated at their mirror image pi/2 - angle (index 8191 - a) with cos and sin exchanged. */
+/* cos and sin of the angle (a + 1/2) * 2 pi / 2^14 for the 14-bit index a: a / 4096 is the quadrant,
+ * a % 4096 the angle (a % 4096 + 1/2) * (pi/2) / 2^12 inside it.  Inside a quadrant, angles above pi/4
+ * are evaluated at their mirror image pi/2 - angle (index 4095 - a % 4096) with cos and sin exchanged;
+ * the quadrant then turns the pair by k * pi/2: (c, s) -> (-s, c) per quarter turn. */
 static void cos_sin_from_index(uint32_t a, float* c, float* s) {
-    int upper = a > 4095u;
-    uint32_t idx = upper ? 8191u - a : a;
+    uint32_t turns = (a / 4096u) % 4u, in_q = a % 4096u;
+    int upper = in_q > 2047u;
+    uint32_t idx = upper ? 4095u - in_q : in_q;
     float steps = (float)idx + 0.5f;
-    float y = steps * 1.91747604e-4f; /* pi / 2^14 */
+    float y = steps * 3.83495208e-4f; /* pi / 2^13 */
     float y2 = y * y;
     float ps = fmaf(-1.9515295891e-4f, y2, 8.3321608736e-3f);
     ps = fmaf(ps, y2, -1.6666654611e-1f);
@@ -147,13 +150,14 @@ static void cos_sin_from_index(uint32_t a, float* c, float* s) {
     float pcy2 = pc * y2;
     float base = fmaf(-0.5f, y2, 1.0f);
     float cs = fmaf(pcy2, y2, base);
-    if (upper) {
-        *c = sn;
-        *s = cs;
-    } else {
-        *c = cs;
-        *s = sn;
+    float cq = upper ? sn : cs, sq = upper ? cs : sn;
+    for (uint32_t t = 0; t < turns; ++t) { /* a quarter turn */
+        float nc = -sq, ns = cq;
+        cq = nc;
+        sq = ns;
     }
+    *c = cq;
+    *s = sq;
 }
 
 /* IEEE binary32 -> binary16 bits, round to nearest even, finite inputs well inside range. */
@@ -200,41 +204,39 @@ static float half_bits_to_float(uint16_t h) {
 }
 
 /* The three factor tables as fp16 bit patterns (tests compare them with a float64 math library). */
-uint16_t jlo_radius_half(uint32_t x) { return half_bits_rne(radius_from_index(x & 0x7FFFu)); }
+uint16_t jlo_radius_half(uint32_t x) { return half_bits_rne(radius_from_index(x & 0x3FFFu)); }
 uint16_t jlo_cos_half(uint32_t a) {
     float c, s;
-    cos_sin_from_index(a & 0x1FFFu, &c, &s);
+    cos_sin_from_index(a & 0x3FFFu, &c, &s);
     return half_bits_rne(c);
 }
 uint16_t jlo_sin_half(uint32_t a) {
     float c, s;
-    cos_sin_from_index(a & 0x1FFFu, &c, &s);
+    cos_sin_from_index(a & 0x3FFFu, &c, &s);
     return half_bits_rne(s);
 }
 
-/* One normal entry from one random word: radius index = bits 16..30, angle index = bits 2..14;
- * the cosine entry takes its sign from bit 15, the sine entry from bit 31 (bit set: negative).
+/* One normal entry from one random word: radius index = bits 17..30, angle index = bits 2..15 (the
+ * cosine and sine tables carry their signs; bits 0, 1, 16 and 31 of the word are not used).
  * The two fp16 factors are multiplied exactly (22-bit product, exact in double) and rounded once. */
 float jlo_normal_from_word(uint32_t w, int sine) {
-    static uint16_t rtab[1 << 15], ctab[1 << 13], stab[1 << 13];
+    static uint16_t rtab[1 << 14], ctab[1 << 14], stab[1 << 14];
     static int ready = 0;
     if (!ready) {
-        for (uint32_t x = 0; x < (1u << 15); ++x) rtab[x] = jlo_radius_half(x);
-        for (uint32_t a = 0; a < (1u << 13); ++a) {
-            ctab[a] = jlo_cos_half(a);
-            stab[a] = jlo_sin_half(a);
+        for (uint32_t i = 0; i < (1u << 14); ++i) {
+            rtab[i] = jlo_radius_half(i);
+            ctab[i] = jlo_cos_half(i);
+            stab[i] = jlo_sin_half(i);
         }
         ready = 1;
     }
-    uint32_t x = (w >> 16) & 0x7FFFu;
-    uint32_t a = (w >> 2) & 0x1FFFu;
+    uint32_t x = (w >> 17) % 16384u;
+    uint32_t a = (w >> 2) % 16384u;
     double radius = (double)half_bits_to_float(rtab[x]);
     double trig = (double)half_bits_to_float(sine ? stab[a] : ctab[a]);
     double prod = radius * trig;
     float pf = (float)prod; /* exact: 22 significant bits, well inside the binary32 range */
-    float mag = half_bits_to_float(half_bits_rne(pf));
-    int negative = sine ? (int)(w >> 31) : (int)((w >> 15) & 1u);
-    return negative ? -mag : mag;
+    return half_bits_to_float(half_bits_rne(pf));
 }
 
 /* Value of S[f, c] (as float; always exactly an fp16 value). */

@@ -112,13 +112,13 @@ def _f32(x):
 
 
 def radius_f32(x):
-    """sqrt(-2 ln u), u = (x + 1/2) / 2^15, for 15-bit indices x: the specified binary32
+    """sqrt(-2 ln u), u = (x + 1/2) / 2^14, for 14-bit indices x: the specified binary32
     operation sequence (log by exponent/mantissa split and a degree-9 polynomial, square root by
     three Newton steps on the reciprocal root)."""
     x = np.asarray(x, dtype=np.uint32)
     one = np.float32(1.0)
     odd = (x << np.uint32(1)) | np.uint32(1)
-    xf = odd.astype(np.float32)  # exact, < 2^16
+    xf = odd.astype(np.float32)  # exact, < 2^15
     xb = xf.view(np.uint32)
     expo = (xb >> np.uint32(23)).astype(np.int32) - 127
     mant = ((xb & np.uint32(0x7FFFFF)) | np.uint32(0x3F800000)).view(np.float32)
@@ -144,7 +144,7 @@ def radius_f32(x):
     y = (t * (z * poly).astype(np.float32)).astype(np.float32)
     y = _fma32(np.float32(-0.5), z, y)
     ln_m = (t + y).astype(np.float32)
-    ln_u = _fma32((expo - 16).astype(np.float32), np.float32(0.693147182), ln_m)
+    ln_u = _fma32((expo - 15).astype(np.float32), np.float32(0.693147182), ln_m)
     s = (np.float32(-2.0) * ln_u).astype(np.float32)
     guess = (np.uint32(0x5F3759DF) - (s.view(np.uint32) >> np.uint32(1))).view(np.float32)
     half_s = (np.float32(0.5) * s).astype(np.float32)
@@ -156,13 +156,17 @@ def radius_f32(x):
 
 
 def cos_sin_f32(a):
-    """cos and sin of (a + 1/2) * (pi/2) / 2^13 for 13-bit indices a, as binary32: polynomials on
-    (0, pi/4); the upper half of the range is the mirror image (index 8191 - a, cos <-> sin)."""
+    """cos and sin of (a + 1/2) * 2 pi / 2^14 for 14-bit indices a, as binary32.  a // 4096 is the quadrant,
+    a % 4096 the angle (a % 4096 + 1/2) * (pi/2) / 2^12 inside it: polynomials on (0, pi/4), the upper half of
+    the quadrant as the mirror image (index 4095 - a % 4096, cos <-> sin), and the quadrant as an exact
+    rotation by a multiple of pi/2."""
     a = np.asarray(a, dtype=np.uint32)
     one = np.float32(1.0)
-    mirror = a >= np.uint32(4096)
-    am = np.where(mirror, np.uint32(8191) - a, a).astype(np.uint32)
-    yv = ((am.astype(np.float32) + np.float32(0.5)).astype(np.float32) * np.float32(1.91747604e-4)).astype(np.float32)
+    quadrant = (a >> np.uint32(12)) & np.uint32(3)
+    aq = a & np.uint32(4095)
+    mirror = aq >= np.uint32(2048)
+    am = np.where(mirror, np.uint32(4095) - aq, aq).astype(np.uint32)
+    yv = ((am.astype(np.float32) + np.float32(0.5)).astype(np.float32) * np.float32(3.83495208e-4)).astype(np.float32)
     y2 = (yv * yv).astype(np.float32)
     ps = _fma32(np.float32(-1.9515295891e-4), y2, np.float32(8.3321608736e-3))
     ps = _fma32(ps, y2, np.float32(-1.6666654611e-1))
@@ -170,7 +174,12 @@ def cos_sin_f32(a):
     pc = _fma32(np.float32(2.443315711809948e-5), y2, np.float32(-1.388731625493765e-3))
     pc = _fma32(pc, y2, np.float32(4.166664568298827e-2))
     cs = _fma32((pc * y2).astype(np.float32), y2, _fma32(np.float32(-0.5), y2, one))
-    return np.where(mirror, sn, cs).astype(np.float32), np.where(mirror, cs, sn).astype(np.float32)
+    c1 = np.where(mirror, sn, cs).astype(np.float32)
+    s1 = np.where(mirror, cs, sn).astype(np.float32)
+    # rotation by quadrant * pi/2: (c, s) -> (c, s), (-s, c), (-c, -s), (s, -c)
+    c = np.choose(quadrant, [c1, -s1, -c1, s1]).astype(np.float32)
+    sn_out = np.choose(quadrant, [s1, c1, -s1, -c1]).astype(np.float32)
+    return c, sn_out
 
 
 _TABLES = None
@@ -178,28 +187,26 @@ _TABLES = None
 
 def normal_tables():
     """(R, C, S): the fp16 factor tables of the normal entries (round to nearest even of the
-    binary32 sequences above), as float16 arrays of 2^15, 2^13 and 2^13 entries."""
+    binary32 sequences above), as float16 arrays of 2^14 entries each (C and S signed, around the circle)."""
     global _TABLES
     if _TABLES is None:
-        r = radius_f32(np.arange(1 << 15, dtype=np.uint32)).astype(np.float16)
-        c, s = cos_sin_f32(np.arange(1 << 13, dtype=np.uint32))
+        r = radius_f32(np.arange(1 << 14, dtype=np.uint32)).astype(np.float16)
+        c, s = cos_sin_f32(np.arange(1 << 14, dtype=np.uint32))
         _TABLES = (r, c.astype(np.float16), s.astype(np.float16))
     return _TABLES
 
 
 def normal_from_word(w, sine):
-    """fp16 normal entries (returned as float16) from random words w: radius index bits 16..30,
-    angle index bits 2..14; sign of the cosine entry bit 15, of the sine entry bit 31 (set ->
-    negative).  The product of the two fp16 factors is exact in float64 and rounded once."""
+    """fp16 normal entries (returned as float16) from random words w: radius index bits 17..30,
+    angle index bits 2..15 (the tables C and S are signed; bits 0, 1, 16, 31 are not used).  The
+    product of the two fp16 factors is exact in float64 and rounded once."""
     w = np.asarray(w, dtype=np.uint32)
     sine = np.asarray(sine, dtype=bool)
     R, C, S = normal_tables()
-    x = ((w >> np.uint32(16)) & np.uint32(0x7FFF)).astype(np.int64)
-    a = ((w >> np.uint32(2)) & np.uint32(0x1FFF)).astype(np.int64)
+    x = ((w >> np.uint32(17)) & np.uint32(0x3FFF)).astype(np.int64)
+    a = ((w >> np.uint32(2)) & np.uint32(0x3FFF)).astype(np.int64)
     trig = np.where(sine, S[a], C[a]).astype(np.float64)
-    mag = (R[x].astype(np.float64) * trig).astype(np.float16)  # numpy rounds float64 -> float16 once, to nearest even
-    neg = np.where(sine, w >> np.uint32(31), (w >> np.uint32(15)) & np.uint32(1)).astype(bool)
-    return np.where(neg, -mag, mag).astype(np.float16)
+    return (R[x].astype(np.float64) * trig).astype(np.float16)  # numpy rounds float64 -> float16 once, to nearest even
 
 
 def materialize(seed, num_feature_tiles, P, f0, nf, c0, nc, proj_type):

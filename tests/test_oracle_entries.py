@@ -106,59 +106,68 @@ def test_factor_tables_against_float64_math(c_oracle):
     # library can differ only where the exact value sits within the binary32 error (a few 2^-24)
     # of an fp16 rounding boundary: never by more than one fp16 step, and only rarely at all.
     R, C, S = npo.normal_tables()
-    assert R.dtype == np.float16 and R.shape == (1 << 15,) and C.shape == S.shape == (1 << 13,)
-    x = np.arange(1 << 15, dtype=np.float64)
-    want_r = np.sqrt(-2.0 * np.log((x + 0.5) / 2.0**15))
-    theta = (np.arange(1 << 13, dtype=np.float64) + 0.5) * (np.pi / 2) / 2.0**13
+    n = 1 << 14
+    assert R.dtype == np.float16 and R.shape == C.shape == S.shape == (n,)
+    x = np.arange(n, dtype=np.float64)
+    want_r = np.sqrt(-2.0 * np.log((x + 0.5) / n))
+    theta = (np.arange(n, dtype=np.float64) + 0.5) * (2 * np.pi) / n      # around the whole circle
     for got, want in ((R, want_r), (C, np.cos(theta)), (S, np.sin(theta))):
         got64 = got.astype(np.float64)
         exact = want.astype(np.float16).astype(np.float64)
         assert np.all(np.abs(got64 - want) <= 0.5 * _ulp16(want) * (1 + 2e-3))
         assert np.mean(got64 == exact) > 0.998
     # before the rounding the binary32 sequences are good to a few units in the last place
-    np.testing.assert_allclose(npo.radius_f32(np.arange(1 << 15)), want_r, rtol=4e-7)
-    c32, s32 = npo.cos_sin_f32(np.arange(1 << 13))
+    np.testing.assert_allclose(npo.radius_f32(np.arange(n)), want_r, rtol=4e-7)
+    c32, s32 = npo.cos_sin_f32(np.arange(n))
     np.testing.assert_allclose(c32, np.cos(theta), rtol=3e-7)
     np.testing.assert_allclose(s32, np.sin(theta), rtol=3e-7)
-    # extremes and symmetry: largest radius sqrt(2 * 16 ln 2), mirror image about pi/4
-    assert float(R[0]) == float(np.float16(np.sqrt(32 * np.log(2.0)))) and R[-1] > 0
+    # extremes and symmetry: largest radius sqrt(2 * 15 ln 2) = 4.56; inside the first quadrant the mirror
+    # image about pi/4; a quarter turn maps (c, s) to (-s, c); the signs of the four quadrants
+    assert float(R[0]) == float(np.float16(np.sqrt(30 * np.log(2.0)))) and R[-1] > 0
     assert np.all(np.diff(R.astype(np.float64)) <= 0)
-    assert np.array_equal(C, S[::-1])
+    q = n // 4
+    assert np.array_equal(C[:q], S[:q][::-1])
+    assert np.array_equal(C[q:], -S[:-q]) and np.array_equal(S[q:], C[:-q])
+    for k, (cs, ss) in enumerate(((1, 1), (-1, 1), (-1, -1), (1, -1))):
+        assert np.all(np.sign(C[k * q:(k + 1) * q]) == cs) and np.all(np.sign(S[k * q:(k + 1) * q]) == ss)
+    assert np.all(C != 0) and np.all(S != 0)
     # the C oracle holds the same tables
-    for i in list(range(0, 1 << 15, 509)) + [0, 1, (1 << 15) - 1]:
+    for i in list(range(0, n, 509)) + [0, 1, n - 1]:
         assert c_oracle.radius_half(i) == int(R[i].view(np.uint16))
-    for i in list(range(0, 1 << 13, 127)) + [0, 4095, 4096, 8191]:
+    for i in list(range(0, n, 127)) + [0, 2047, 2048, 4095, 4096, 8191, 8192, 12_287, 12_288, n - 1]:
         assert c_oracle.cos_half(i) == int(C[i].view(np.uint16))
         assert c_oracle.sin_half(i) == int(S[i].view(np.uint16))
 
 
 def test_normal_entry_is_box_muller_in_fp16(c_oracle):
-    # entry = +-fp16(R[x] * C[a] or S[a]); against Box-Muller in float64 with the same uniform
-    # u = (x + 1/2) / 2^15 and the same angle: each factor is off by at most 2^-11 of itself (half
+    # entry = fp16(R[x] * C[a] or S[a]); against Box-Muller in float64 with the same uniform
+    # u = (x + 1/2) / 2^14 and the same angle: each factor is off by at most 2^-11 of itself (half
     # an fp16 step), the rounding of the product adds half a step
     rng = np.random.default_rng(7)
     w = rng.integers(0, 2**32, size=20_000, dtype=np.uint64).astype(np.uint32)
-    w[:6] = [0, 0xFFFFFFFF, 0x7FFF0000, 0x00007FFC, 0x80008000, 0x7FFF7FFC]
-    x = ((w >> 16) & 0x7FFF).astype(np.float64)
-    a = ((w >> 2) & 0x1FFF).astype(np.float64)
-    r = np.sqrt(-2.0 * np.log((x + 0.5) / 2.0**15))
-    theta = (a + 0.5) * (np.pi / 2) / 2.0**13
+    w[:6] = [0, 0xFFFFFFFF, 0x7FFE0000, 0x0000FFFC, 0x80010003, 0x7FFEFFFC]
+    x = ((w >> 17) & 0x3FFF).astype(np.float64)
+    a = ((w >> 2) & 0x3FFF).astype(np.float64)
+    r = np.sqrt(-2.0 * np.log((x + 0.5) / 2.0**14))
+    theta = (a + 0.5) * (2 * np.pi) / 2.0**14
     R, C, S = npo.normal_tables()
-    for sine, trig, sign_bit, tab in ((False, np.cos(theta), 15, C), (True, np.sin(theta), 31, S)):
+    for sine, trig, tab in ((False, np.cos(theta), C), (True, np.sin(theta), S)):
         z = npo.normal_from_word(w, np.full(w.shape, sine))
         assert z.dtype == np.float16
-        sign = np.where((w >> sign_bit) & 1, -1.0, 1.0)
-        want = sign * r * trig
+        want = r * trig
         err = np.abs(z.astype(np.float64) - want)
         assert np.all(err <= (2.0**-10 * np.abs(want) + 0.5 * _ulp16(want)) * (1 + 1e-3))
         assert np.median(err / _ulp16(want)) < 0.5
+        # bits 0, 1, 16 and 31 of the word are not part of any field
+        assert np.array_equal(z, npo.normal_from_word(w ^ np.uint32(0x80010003), np.full(w.shape, sine)))
         # the definition itself, restated with exact rational arithmetic on a sample
         from fractions import Fraction
         for i in range(0, 20_000, 401):
             p = Fraction(float(R[int(x[i])])) * Fraction(float(tab[int(a[i])]))
             lo = np.float16(float(p))  # float(p) is exact (22 significant bits)
-            assert float(z[i]) == float(sign[i]) * float(lo)
+            assert float(z[i]) == float(lo)
             assert c_oracle.normal_from_word(int(w[i]), sine) == float(z[i])
+            assert c_oracle.normal_from_word(int(w[i]) ^ 0x80010003, sine) == float(z[i])
 
 
 def test_normal_block_uses_every_word_for_one_pair(c_oracle):
@@ -203,6 +212,6 @@ def test_normal_entries_are_fp16_standard_normals(c_oracle):
     # and their squares add up to the squared radius: chi-square with two degrees of freedom
     r2 = S[0::2].ravel() ** 2 + S[1::2].ravel() ** 2
     assert stats.kstest(r2[:50_000], "chi2", args=(2,)).pvalue > 1e-3
-    # tails: the radius grid ends at sqrt(32 ln 2) = 4.71
-    assert np.abs(S).max() <= 4.72 and np.abs(S).max() > 3.5
+    # tails: the radius grid ends at sqrt(30 ln 2) = 4.56
+    assert np.abs(S).max() <= 4.57 and np.abs(S).max() > 3.5
     assert abs(np.corrcoef(S[:, 0], S[:, 1])[0, 1]) < 5 / math.sqrt(S.shape[0])

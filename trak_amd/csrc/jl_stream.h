@@ -28,12 +28,15 @@
 //
 // Normal: feature offset o uses block n = o / 8; word (o % 8) / 2 of the block makes the
 //   Box-Muller pair of entries o % 8 = 2i (cosine) and 2i + 1 (sine):
-//       entry = +-fp16( R[x] * C[a] )   resp.   +-fp16( R[x] * S[a] )
-//   with a 15-bit radius index x, a 13-bit angle index a and two sign bits taken from the word,
-//       R[x] = fp16( sqrt(-2 ln((x + 1/2) / 2^15)) ),
-//       C[a], S[a] = fp16( cos, sin of (a + 1/2) * (pi/2) / 2^13 ),
-//   i.e. a uniform angle on a grid of 2^15 directions around the circle (quadrant by the two
-//   signs).  R, C and S are spelled out below in IEEE binary32 operations (add, mul, fma,
+//       entry = fp16( R[x] * C[a] )   resp.   fp16( R[x] * S[a] )
+//   with a 14-bit radius index x (bits 17..30 of the word) and a 14-bit angle index a (bits 2..15),
+//       R[x] = fp16( sqrt(-2 ln((x + 1/2) / 2^14)) ),
+//       C[a], S[a] = fp16( cos, sin of (a + 1/2) * 2 pi / 2^14 ),
+//   i.e. a uniform angle on a grid of 2^14 directions around the whole circle (C and S carry their
+//   signs) and a uniform u on a grid of 2^14 values.  The fields sit so that each table's byte address
+//   is one instruction: (w >> 16) & 0x7FFE for the 2-byte entries of R (a 16-bit sub-word select and a
+//   mask), w & 0xFFFC for the 4-byte pairs (C, S); with the quadrant in the table no sign is applied
+//   afterwards.  R, C and S are spelled out below in IEEE binary32 operations (add, mul, fma,
 //   int<->float conversions of exactly representable values) and rounded to fp16 (nearest even),
 //   so any IEEE machine reproduces them bit for bit; the product of the two fp16 factors is
 //   exact in binary32 and is rounded once.  The kernel keeps R and (C, S) as tables in LDS.
@@ -144,9 +147,11 @@ JL_HD float jl_add_(float a, float b) {
 #define JL_ADD(a, b) jl::jl_add_((a), (b))
 #endif
 
-// Radius table entry: r = sqrt(-2 ln u), u = (2x + 1) / 2^16 in (0, 1), for a 15-bit index x.
+constexpr uint32_t kRadiusBits = 14, kAngleBits = 14;  // 2^14 entries each: 32 KB of fp16 radii, 64 KB of fp16 pairs
+
+// Radius table entry: r = sqrt(-2 ln u), u = (2x + 1) / 2^15 in (0, 1), for a 14-bit index x.
 JL_HD float bm_radius(uint32_t x) {
-    const uint32_t odd = (x << 1) | 1u;  // < 2^16: exact as float
+    const uint32_t odd = (x << 1) | 1u;  // < 2^15: exact as float
     const uint32_t xb = f2u((float)odd);
     int e = (int)(xb >> 23) - 127;
     float m = u2f((xb & 0x007FFFFFu) | 0x3F800000u);  // [1, 2)
@@ -168,7 +173,7 @@ JL_HD float bm_radius(uint32_t x) {
     float y = JL_MUL(t, JL_MUL(z, p));
     y = JL_FMA(-0.5f, z, y);
     const float lnm = JL_ADD(t, y);
-    const float lnu = JL_FMA((float)(e - 16), 0.693147182f, lnm);
+    const float lnu = JL_FMA((float)(e - 15), 0.693147182f, lnm);
     const float s = JL_MUL(-2.0f, lnu);
     // sqrt(s) by three Newton steps on 1/sqrt(s) from an integer seed
     float g = u2f(0x5f3759dfu - (f2u(s) >> 1));
@@ -182,13 +187,15 @@ JL_HD float bm_radius(uint32_t x) {
     return JL_MUL(s, g);
 }
 
-// Angle table entry: cos and sin of theta = (a + 1/2) * (pi/2) / 2^13 in (0, pi/2) for a 13-bit
-// index a.  The upper half of the range is the mirror image of the lower one (cos <-> sin), so
-// the polynomials only see (0, pi/4).
+// Angle table entry: cos and sin of theta = (a + 1/2) * 2 pi / 2^14 for a 14-bit index a.  The two top
+// bits of a are the quadrant, the other twelve the angle (a' + 1/2) * (pi/2) / 2^12 in (0, pi/2) inside it;
+// the upper half of that range is the mirror image of the lower one (cos <-> sin), so the polynomials only
+// see (0, pi/4), and the quadrant turns the pair by a multiple of pi/2 (exact: swaps and sign changes).
 JL_HD void bm_cossin(uint32_t a, float* c_out, float* s_out) {
-    const bool mirror = a >= 4096u;
-    const uint32_t am = mirror ? 8191u - a : a;
-    const float yv = JL_MUL(JL_ADD((float)am, 0.5f), 1.91747604e-4f);  // pi / 2^14
+    const uint32_t quadrant = (a >> 12) & 3u, aq = a & 4095u;
+    const bool mirror = aq >= 2048u;
+    const uint32_t am = mirror ? 4095u - aq : aq;
+    const float yv = JL_MUL(JL_ADD((float)am, 0.5f), 3.83495208e-4f);  // pi / 2^13
     const float y2 = JL_MUL(yv, yv);
     float ps = JL_FMA(-1.9515295891e-4f, y2, 8.3321608736e-3f);
     ps = JL_FMA(ps, y2, -1.6666654611e-1f);
@@ -196,8 +203,9 @@ JL_HD void bm_cossin(uint32_t a, float* c_out, float* s_out) {
     float pc = JL_FMA(2.443315711809948e-5f, y2, -1.388731625493765e-3f);
     pc = JL_FMA(pc, y2, 4.166664568298827e-2f);
     const float cs = JL_FMA(JL_MUL(pc, y2), y2, JL_FMA(-0.5f, y2, 1.0f));
-    *c_out = mirror ? sn : cs;
-    *s_out = mirror ? cs : sn;
+    const float c1 = mirror ? sn : cs, s1 = mirror ? cs : sn;  // first quadrant
+    *c_out = quadrant == 0 ? c1 : quadrant == 1 ? -s1 : quadrant == 2 ? -c1 : s1;
+    *s_out = quadrant == 0 ? s1 : quadrant == 1 ? c1 : quadrant == 2 ? -s1 : -c1;
 }
 
 // binary32 -> binary16 bit pattern, round to nearest even (|v| < 65504 here, no NaN).  On the
@@ -258,10 +266,9 @@ JL_HD float entry_rademacher(uint32_t seed, uint32_t column, uint32_t tile, uint
 }
 
 // The fields of one random word: it makes one Box-Muller pair.
-//   bits 16..30  radius index x          bit 31  sign of the sine entry
-//   bits  2..14  angle index a           bit 15  sign of the cosine entry      (bits 0, 1 unused)
-JL_HD uint32_t normal_radius_index(uint32_t w) { return (w >> 16) & 0x7FFFu; }
-JL_HD uint32_t normal_angle_index(uint32_t w) { return (w >> 2) & 0x1FFFu; }
+//   bits 17..30  radius index x          bits 2..15  angle index a          (bits 0, 1, 16, 31 unused)
+JL_HD uint32_t normal_radius_index(uint32_t w) { return (w >> 17) & 0x3FFFu; }
+JL_HD uint32_t normal_angle_index(uint32_t w) { return (w >> 2) & 0x3FFFu; }
 
 // fp16 product of two fp16 values, round to nearest even (the product is exact in binary32).
 JL_HD uint16_t f16_mul_rne(uint16_t a, uint16_t b) {
@@ -281,8 +288,7 @@ JL_HD uint16_t entry_normal_f16bits(uint32_t seed, uint32_t column, uint32_t til
     float c, s;
     bm_cossin(normal_angle_index(w), &c, &s);
     const uint16_t t = f32_to_f16_rne((e & 1u) ? s : c);
-    const uint16_t sign = (uint16_t)(((e & 1u) ? (w >> 31) : (w >> 15)) << 15);
-    return (uint16_t)(f16_mul_rne(r, t) ^ sign);
+    return f16_mul_rne(r, t);
 }
 
 JL_HD float entry_normal(uint32_t seed, uint32_t column, uint32_t tile, uint32_t o) {

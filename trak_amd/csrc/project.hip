@@ -829,10 +829,11 @@ __global__ __launch_bounds__(512) void jl_project_kernel(
 // entry is used for 32 multiply-adds only, and making one costs about ten vector instructions
 // (Philox4x32-10: one block per eight entries) against 1.5 for a sign, so the kernel is bound by
 // the vector ALU, not by the matrix pipe.  What keeps the count that low:
-//   * one random word makes a whole Box-Muller pair: the radius R[x] and the pair (C[a], S[a])
-//     come out of two LDS tables (64 KB + 32 KB, filled at kernel start from the binary32
-//     sequences of jl_stream.h), one v_pk_mul_f16 multiplies and rounds both entries, one
-//     v_bitop3_b32 applies the two sign bits;
+//   * one random word makes a whole Box-Muller pair: the radius R[x] and the signed pair
+//     (C[a], S[a]) come out of two LDS tables (32 KB + 64 KB, filled at kernel start from the
+//     binary32 sequences of jl_stream.h), each addressed by ONE instruction (the fields of the
+//     word sit so that a masked 16-bit half of it is the byte offset), and one v_pk_mul_f16
+//     multiplies and rounds both entries: three vector instructions per pair;
 //   * the matrix entries are fp16 whatever the gradient type is, so the gradients are brought to
 //     fp16 once per chunk at staging time instead of splitting every entry into bf16 terms in the
 //     hot loop: bf16 and fp32 chunks are multiplied row by row by the power of two that puts the
@@ -844,8 +845,8 @@ __global__ __launch_bounds__(512) void jl_project_kernel(
 typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
 typedef unsigned short ushort2_t __attribute__((ext_vector_type(2)));
 
-constexpr int kRadiusEntries = 1 << 15;
-constexpr int kAngleEntries = 1 << 13;
+constexpr int kRadiusEntries = 1 << jl::kRadiusBits;
+constexpr int kAngleEntries = 1 << jl::kAngleBits;
 #ifndef JL_NORMAL_UNROLL
 #define JL_NORMAL_UNROLL 1
 #endif
@@ -902,14 +903,14 @@ __device__ __forceinline__ uint32_t pack_f16_rne(float a, float b) {
 }
 
 // bf16 chunk -> one scaled fp16 plane.  The 32 threads that share tid / 32 hold one row (N rows
-// per thread, 16 apart); sh_ref[] is the row's reference exponent so far; sh_delta / sh_use are the
-// per-row lists of this buffer (16 N entries each).
-template <int N>
+// per thread, 2 W apart for a workgroup of W waves); sh_ref[] is the row's reference exponent so far;
+// sh_delta / sh_use are the per-row lists of this buffer (2 W N entries each).
+template <int W, int N>
 __device__ __forceinline__ void store_scaled_bf16(const uint4 (&v)[N], uint16_t* lds, int* sh_delta, int* sh_use,
                                                   int tid, int (&sh_ref)[N]) {
 #pragma unroll
     for (int i = 0; i < N; ++i) {
-        const uint32_t row = (tid >> 5) + 16 * i, sg = tid & 31;
+        const uint32_t row = (tid >> 5) + 2 * W * i, sg = tid & 31;
         const uint32_t w[4] = {v[i].x, v[i].y, v[i].z, v[i].w};
         ushort2_t m = __builtin_bit_cast(ushort2_t, w[0] & 0x7F807F80u);
 #pragma unroll
@@ -934,13 +935,14 @@ __device__ __forceinline__ void store_scaled_bf16(const uint4 (&v)[N], uint16_t*
     }
 }
 
-// fp32 chunk -> two scaled fp16 planes.  The 64 threads of a wave hold one row (four rows per
-// thread, 8 apart).
-__device__ __forceinline__ void store_scaled_f32(const uint4 (&v)[4], uint16_t* lds, int* sh_delta, int* sh_use, int tid,
-                                                 int (&sh_ref)[4]) {
+// fp32 chunk -> two scaled fp16 planes.  The 64 threads of a wave hold one row (N = 32 / W rows per
+// thread, W apart).
+template <int W, int N>
+__device__ __forceinline__ void store_scaled_f32(const uint4 (&v)[N], uint16_t* lds, int* sh_delta, int* sh_use, int tid,
+                                                 int (&sh_ref)[N]) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const uint32_t row = (tid >> 6) + 8 * i, sg = tid & 63;
+    for (int i = 0; i < N; ++i) {
+        const uint32_t row = (tid >> 6) + W * i, sg = tid & 63;
         const uint32_t w[4] = {v[i].x, v[i].y, v[i].z, v[i].w};
         uint32_t e = 0;
 #pragma unroll
@@ -975,15 +977,16 @@ __device__ __forceinline__ void store_scaled_f32(const uint4 (&v)[4], uint16_t* 
 }
 
 // The Box-Muller pair of one random word as packed fp16 (cosine entry low, sine entry high):
-// fields of the word as in jl_stream.h (radius index bits 16..30, angle index bits 2..14, signs
-// bits 15 and 31).  r_tab holds fp16 R[x], cs_tab the packed fp16 pairs (C[a], S[a]).
+// fields of the word as in jl_stream.h (radius index bits 17..30, angle index bits 2..15).  r_tab
+// holds fp16 R[x], cs_tab the packed signed fp16 pairs (C[a], S[a]).  Each byte offset is one
+// instruction: the upper half of the word under the mask 0x7FFE (v_and_b32 with a 16-bit sub-word
+// select), the lower half under 0xFFFC.
 __device__ __forceinline__ uint32_t normal_pair(uint32_t w, const char* r_tab, const char* cs_tab) {
-    const _Float16 r = *reinterpret_cast<const _Float16*>(r_tab + ((w >> 15) & 0xFFFEu));
-    const uint32_t cs = *reinterpret_cast<const uint32_t*>(cs_tab + (w & 0x7FFCu));
+    const _Float16 r = *reinterpret_cast<const _Float16*>(r_tab + ((w >> 16) & 0x7FFEu));
+    const uint32_t cs = *reinterpret_cast<const uint32_t*>(cs_tab + (w & 0xFFFCu));
     const half2_t rr = {r, r};
     const half2_t z = rr * __builtin_bit_cast(half2_t, cs);  // v_pk_mul_f16: exact products, rounded once
-    // z ^ (w & 0x80008000): truth table of a ^ (b & c)
-    return __builtin_amdgcn_bitop3_b32(__builtin_bit_cast(uint32_t, z), w, 0x80008000u, 0x78);
+    return __builtin_bit_cast(uint32_t, z);
 }
 
 // GPW = 32-column groups per wave: 4 (workgroup = 1024 columns) or 2 (512 columns, for projection
@@ -991,12 +994,11 @@ __device__ __forceinline__ uint32_t normal_pair(uint32_t w, const char* r_tab, c
 // when the batch has more than 32 rows - every generated entry then feeds two MFMAs, which is worth
 // almost a factor of two to a kernel bound by the cost of making an entry (one LDS buffer then: two
 // do not fit next to the tables).  Always 8 waves; arguments as jl_project_kernel.
-template <int IN, bool GATHER, int GPW, int RB>
-__global__ __launch_bounds__(512) void jl_project_normal_kernel(
+template <int IN, bool GATHER, int GPW, int RB, int W>
+__global__ __launch_bounds__(64 * W) void jl_project_normal_kernel(
     const void* __restrict__ g_in, uint64_t ld, uint32_t rows, uint64_t P, uint32_t k, uint32_t seed,
     uint32_t tiles, uint64_t tile_size, uint32_t chunks_per_tile, uint32_t chunks_per_group, uint32_t groups,
     float* __restrict__ partial) {
-    constexpr int W = 8;
     typedef NormalTraits<IN> Tr;
     typedef typename StageOf<IN, GATHER, W, 32 * RB>::type Stage;
     typedef typename StageOf<IN, GATHER, W, 32 * RB>::elem Elem;
@@ -1010,12 +1012,14 @@ __global__ __launch_bounds__(512) void jl_project_normal_kernel(
     constexpr int kRows = 32 * RB;
 
     // One LDS block, tables first: a DS instruction adds a 16-bit immediate to the address register,
-    // so a table that starts below 64 KB is indexed without an extra addition per lookup.
+    // so a table that starts below 64 KB is indexed without an extra addition per lookup (the radii
+    // at 0, the pairs at 32 KB).
     constexpr int kCsBytes = kAngleEntries * 4, kRBytes = kRadiusEntries * 2;
+    static_assert(kRBytes < 65536, "the pair table must start below 64 KB");
     constexpr int kStageBytes = kBuffers * kBufElems * 2;
     __shared__ __attribute__((aligned(16))) char smem[kCsBytes + kRBytes + kStageBytes + kBuffers * 2 * kRows * 4];
-    uint32_t* cs_tab = reinterpret_cast<uint32_t*>(smem);
-    uint16_t* r_tab = reinterpret_cast<uint16_t*>(smem + kCsBytes);
+    uint16_t* r_tab = reinterpret_cast<uint16_t*>(smem);
+    uint32_t* cs_tab = reinterpret_cast<uint32_t*>(smem + kRBytes);
     uint16_t* lds = reinterpret_cast<uint16_t*>(smem + kCsBytes + kRBytes);
     // per buffer and row: change of the row's exponent against the previous chunk, and the exponent
     int (*sh_lds)[2][kRows] = reinterpret_cast<int (*)[2][kRows]>(smem + kCsBytes + kRBytes + kStageBytes);
@@ -1065,9 +1069,9 @@ __global__ __launch_bounds__(512) void jl_project_normal_kernel(
         if constexpr (IN == TRAKHIP_F16)
             st.store(lds + buf * kBufElems, tid);
         else if constexpr (IN == TRAKHIP_BF16)
-            store_scaled_bf16(st.v, lds + buf * kBufElems, sh_lds[buf][0], sh_lds[buf][1], tid, sh_ref);
+            store_scaled_bf16<W>(st.v, lds + buf * kBufElems, sh_lds[buf][0], sh_lds[buf][1], tid, sh_ref);
         else
-            store_scaled_f32(st.v, lds + buf * kBufElems, sh_lds[buf][0], sh_lds[buf][1], tid, sh_ref);
+            store_scaled_f32<W>(st.v, lds + buf * kBufElems, sh_lds[buf][0], sh_lds[buf][1], tid, sh_ref);
     };
     {
         const uint64_t lo = (uint64_t)t0 * tile_size;
@@ -1331,21 +1335,34 @@ hipError_t launch_rademacher(const void* in, uint64_t ld, uint32_t rows, uint64_
     return hipGetLastError();
 }
 
+#ifndef JL_NORMAL_WAVES
+#define JL_NORMAL_WAVES 16
+#endif
+#ifndef JL_NORMAL_WAVES_RB2
+#define JL_NORMAL_WAVES_RB2 16
+#endif
+// The normal kernel's workgroup: kNormalWaves waves that share the plan's column block, i.e.
+// 8 * GPW / kNormalWaves 32-column groups per wave (kNormalWaves2: the instance with two row blocks).
+constexpr int kNormalWaves = JL_NORMAL_WAVES, kNormalWaves2 = JL_NORMAL_WAVES_RB2;
+
 template <int IN, bool GATHER, int GPW>
 hipError_t launch_normal(const void* in, uint64_t ld, uint32_t rows, uint64_t P, uint32_t k, uint32_t seed,
                          const Plan& pl, float* partial, hipStream_t s) {
+    constexpr int W = kNormalWaves, G = 8 * GPW / W;  // same columns per workgroup as the plan's 8 waves x GPW
+    constexpr int W2 = kNormalWaves2, G2 = 8 * GPW / W2;
+    static_assert(G >= 1 && G * W == 8 * GPW && G2 >= 1 && G2 * W2 == 8 * GPW, "column groups per wave");
     const uint64_t wgs = plan_workgroups(pl);
     if (wgs > 0x7FFFFFFFull) return hipErrorInvalidValue;
     if (rows > 32) {
         if constexpr (IN == TRAKHIP_F32) {
             return hipErrorInvalidValue;
         } else {
-            hipLaunchKernelGGL((jl_project_normal_kernel<IN, GATHER, GPW, 2>), dim3((uint32_t)wgs), dim3(512), 0, s, in,
+            hipLaunchKernelGGL((jl_project_normal_kernel<IN, GATHER, G2, 2, W2>), dim3((uint32_t)wgs), dim3(64 * W2), 0, s, in,
                                ld, rows, P, k, seed, pl.tl.tiles, pl.tl.tile_size, pl.chunks_per_tile,
                                pl.chunks_per_group, pl.groups, partial);
         }
     } else {
-        hipLaunchKernelGGL((jl_project_normal_kernel<IN, GATHER, GPW, 1>), dim3((uint32_t)wgs), dim3(512), 0, s, in, ld,
+        hipLaunchKernelGGL((jl_project_normal_kernel<IN, GATHER, G, 1, W>), dim3((uint32_t)wgs), dim3(64 * W), 0, s, in, ld,
                            rows, P, k, seed, pl.tl.tiles, pl.tl.tile_size, pl.chunks_per_tile, pl.chunks_per_group,
                            pl.groups, partial);
     }
