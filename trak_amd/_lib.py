@@ -90,6 +90,10 @@ def load():
     lib.trakhip_spd_inverse_workspace.restype = sz
     lib.trakhip_spd_inverse.argtypes = [vp, u64, f32, vp, u64, u64, i32, vp, vp, vp, sz, vp]
     lib.trakhip_spd_inverse.restype = i32
+    lib.trakhip_general_inverse_workspace.argtypes = [u64]
+    lib.trakhip_general_inverse_workspace.restype = sz
+    lib.trakhip_general_inverse.argtypes = [vp, u64, f32, vp, u64, u64, i32, vp, vp, vp, sz, vp]
+    lib.trakhip_general_inverse.restype = i32
     _lib = lib
     return lib
 

@@ -175,4 +175,13 @@ int trakhip_spd_inverse(const float* A_dev, uint64_t lda, float lambda, float* i
                                 workspace_dev, workspace_bytes, static_cast<hipStream_t>(stream));
 }
 
+size_t trakhip_general_inverse_workspace(uint64_t n) { return trakhip::general_inverse_workspace_bytes(n); }
+
+int trakhip_general_inverse(const float* A_dev, uint64_t lda, float lambda, float* inv_dev, uint64_t ldi,
+                            uint64_t n, int normalize, float* mean_abs_dev, int32_t* status_dev,
+                            void* workspace_dev, size_t workspace_bytes, void* stream) {
+    return trakhip::general_inverse(A_dev, lda, lambda, inv_dev, ldi, n, normalize, mean_abs_dev, status_dev,
+                                    workspace_dev, workspace_bytes, static_cast<hipStream_t>(stream));
+}
+
 }  // extern "C"

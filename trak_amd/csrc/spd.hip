@@ -17,6 +17,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <type_traits>
+#include <utility>
 #include <vector>
 
 #include "short_k_tile.h"
@@ -534,6 +536,270 @@ int spd_inverse(const float* A, uint64_t lda, float lambda, float* inv, uint64_t
         if (hipGetLastError() != hipSuccess) return TRAKHIP_ERR_LAUNCH;
     }
     return TRAKHIP_OK;
+}
+
+}  // namespace trakhip
+
+namespace {
+
+// ---- inverse of a general matrix: Gauss-Jordan elimination with partial pivoting ---------------------------
+//
+// For the matrices the Cholesky route above refuses: a Gram matrix rounded to fp16, or one of deficient
+// rank with lambda = 0, is symmetric but need not be positive definite.  The reference inverts every
+// matrix with LU and partial pivoting (torch.linalg.inv, trak/score_computers.py:163); this is the same
+// pivoting on the device.  The augmented matrix [A + lambda I | I] (np x 2 np, np = n padded with an
+// identity block to a multiple of 128) is reduced to [I | A^-1], SP columns per step:
+//   1. gj_panel_kernel: ONE workgroup holds rows j.. of the SP panel columns in registers and eliminates
+//      them column by column with row pivoting (largest magnitude, lowest row on ties; rows are not
+//      moved, a row is marked once it has been a pivot).  It leaves the pivot rows' numbers, where the
+//      rows they displace go, and the factors L U of the SP x SP pivot block D;
+//   2. gj_rows_kernel: one thread per column of the rest of the matrix moves the rows into place and
+//      replaces the pivot rows by R = D^-1 * (pivot rows), solved with the two triangular factors (an
+//      explicit D^-1 would lose what the condition of D costs);
+//   3. every other row r gets  W[r, rest] -= W[r, panel] * R  (the fp32 MFMA product; the pivot rows'
+//      panel entries were set to zero, so they pass through unchanged).
+// The composition of the SP single-column eliminations of a step differs from the identity only in the
+// panel's columns, which is why steps 2 and 3 can apply it to all other columns at once.
+
+constexpr int kGjThreads = 1024;
+constexpr int kGjMaxSp = 16;
+
+struct GjStep {
+    int32_t piv[kGjMaxSp];   // the row that becomes row j + c
+    int32_t from[kGjMaxSp];  // rows of the pivot positions that were not chosen ...
+    int32_t to[kGjMaxSp];    // ... and the vacated positions they move to
+    int32_t moves;
+    int32_t pad[3];
+    float lu[kGjMaxSp * kGjMaxSp];  // the pivot block as packed factors: unit lower L below the diagonal, U on and above
+};
+
+__global__ __launch_bounds__(256) void gj_init_kernel(const float* __restrict__ A, uint64_t lda, float lambda,
+                                                      uint64_t n, uint64_t np, float* __restrict__ W,
+                                                      int32_t* __restrict__ status) {
+    const uint64_t idx = (uint64_t)blockIdx.x * 256 + threadIdx.x;
+    if (idx == 0 && status) *status = 0;
+    if (idx >= np * 2 * np) return;
+    const uint64_t i = idx / (2 * np), j = idx % (2 * np);
+    float v;
+    if (j >= np)
+        v = (j - np == i) ? 1.0f : 0.0f;
+    else if (i < n && j < n)
+        v = A[i * lda + j] + (i == j ? lambda : 0.0f);
+    else
+        v = (i == j) ? 1.0f : 0.0f;
+    W[idx] = v;
+}
+
+// larger magnitude wins; on equal magnitudes the lower row (what a sequential search finds first)
+__device__ __forceinline__ void gj_better(uint32_t& key, uint32_t& row, uint32_t okey, uint32_t orow) {
+    if (okey > key || (okey == key && orow < row)) {
+        key = okey;
+        row = orow;
+    }
+}
+
+template <class F, int... S>
+__device__ __forceinline__ void gj_for_each(F& f, std::integer_sequence<int, S...>) {
+    (f(std::integral_constant<int, S>{}), ...);
+}
+
+template <int SP, int RPT>
+__global__ __launch_bounds__(kGjThreads) void gj_panel_kernel(const float* __restrict__ W, uint64_t ld, uint32_t np,
+                                                              uint32_t j, GjStep* __restrict__ step,
+                                                              int32_t* __restrict__ status) {
+    __shared__ uint32_t cand_key[kGjThreads / 64], cand_row[kGjThreads / 64];
+    __shared__ float lu[SP][SP + 1];  // row c: the pivot row of column c as it was when chosen (packed L \ U)
+    __shared__ int32_t piv[SP];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    float a[RPT][SP];
+    uint32_t live = 0;  // bit i: row i of this thread exists and has not been a pivot
+#pragma unroll
+    for (int i = 0; i < RPT; ++i) {
+        const uint32_t r = j + (uint32_t)tid + (uint32_t)kGjThreads * i;
+        if (r < np) {
+            live |= 1u << i;
+            const float4* src = reinterpret_cast<const float4*>(W + (uint64_t)r * ld + j);
+#pragma unroll
+            for (int c4 = 0; c4 < SP / 4; ++c4) {
+                const float4 v = src[c4];
+                a[i][4 * c4] = v.x, a[i][4 * c4 + 1] = v.y, a[i][4 * c4 + 2] = v.z, a[i][4 * c4 + 3] = v.w;
+            }
+        } else {
+#pragma unroll
+            for (int c = 0; c < SP; ++c) a[i][c] = 0.0f;
+        }
+    }
+    // (the columns are written out through a compile-time sequence: `#pragma unroll` gives up on a body
+    // of this size, and the register array would be indexed at run time, i.e. live in scratch memory)
+    auto column = [&](auto c_const) __attribute__((always_inline)) {
+        constexpr int c = decltype(c_const)::value;
+        // the pivot of column c: largest |a| among the rows that have not been pivots
+        uint32_t key = 0, row = 0xFFFFFFFFu;
+#pragma unroll
+        for (int i = 0; i < RPT; ++i)
+            if (live & (1u << i))
+                gj_better(key, row, __float_as_uint(fabsf(a[i][c])), j + (uint32_t)tid + (uint32_t)kGjThreads * i);
+#pragma unroll
+        for (int d = 1; d < 64; d <<= 1)
+            gj_better(key, row, (uint32_t)__shfl_xor((int)key, d, 64), (uint32_t)__shfl_xor((int)row, d, 64));
+        if (lane == 0) cand_key[wave] = key, cand_row[wave] = row;
+        __syncthreads();
+        key = cand_key[0], row = cand_row[0];
+#pragma unroll
+        for (int w = 1; w < kGjThreads / 64; ++w) gj_better(key, row, cand_key[w], cand_row[w]);
+        // its owner publishes the row (multipliers of earlier columns in front, the eliminated row behind)
+#pragma unroll
+        for (int i = 0; i < RPT; ++i) {
+            if ((live & (1u << i)) && row == j + (uint32_t)tid + (uint32_t)kGjThreads * i) {
+                live &= ~(1u << i);
+#pragma unroll
+                for (int c2 = 0; c2 < SP; ++c2) lu[c][c2] = a[i][c2];
+                piv[c] = (int32_t)row;
+                if (a[i][c] == 0.0f && status) *status = (int32_t)(j + c + 1);  // exactly singular
+            }
+        }
+        __syncthreads();
+        const float pivot = lu[c][c];
+#pragma unroll
+        for (int i = 0; i < RPT; ++i) {
+            if (live & (1u << i)) {
+                const float l = a[i][c] / pivot;
+                a[i][c] = l;
+#pragma unroll
+                for (int c2 = c + 1; c2 < SP; ++c2) a[i][c2] = fmaf(-l, lu[c][c2], a[i][c2]);
+            }
+        }
+    };
+    gj_for_each(column, std::make_integer_sequence<int, SP>{});
+    // D = (rows piv[0..SP) of the panel as they were) = L U with the packed factors in lu
+    if (tid < SP) {
+#pragma unroll
+        for (int q = 0; q < SP; ++q) step->lu[tid * SP + q] = lu[tid][q];
+        step->piv[tid] = piv[tid];
+    }
+    if (tid == 0) {
+        // rows at the pivot positions j .. j+SP-1 that were not chosen go to the positions that the chosen
+        // rows from further down leave behind, both in ascending order
+        int32_t moves = 0, to_n = 0;
+        for (int q = 0; q < SP; ++q) {
+            const int32_t pos = (int32_t)j + q;
+            bool chosen = false;
+            for (int c = 0; c < SP; ++c) chosen |= piv[c] == pos;
+            if (!chosen) step->from[moves++] = pos;
+        }
+        // vacated positions below the pivot block, ascending (selection over at most SP values)
+        int32_t last = (int32_t)j + SP - 1;
+        for (int m = 0; m < moves; ++m) {
+            int32_t best = 0x7FFFFFFF;
+            for (int c = 0; c < SP; ++c)
+                if (piv[c] > last && piv[c] < best) best = piv[c];
+            step->to[to_n++] = best;
+            last = best;
+        }
+        step->moves = moves;
+    }
+}
+
+// One thread per column col of [j, 2 np): rows move into place, pivot rows become D^-1 * (pivot rows)
+// (zero in the panel's own columns, whose entries in the other rows are the multipliers of step 3).
+template <int SP>
+__global__ __launch_bounds__(256) void gj_rows_kernel(float* __restrict__ W, uint64_t ld, uint32_t np, uint32_t j,
+                                                      const GjStep* __restrict__ step) {
+    __shared__ GjStep st;
+    for (uint32_t i = threadIdx.x; i < sizeof(GjStep) / 4; i += 256)
+        reinterpret_cast<uint32_t*>(&st)[i] = reinterpret_cast<const uint32_t*>(step)[i];
+    __syncthreads();
+    const uint64_t col = (uint64_t)j + (uint64_t)blockIdx.x * 256 + threadIdx.x;
+    if (col >= 2ull * np) return;
+    float v[SP], d[SP];
+#pragma unroll
+    for (int c = 0; c < SP; ++c) v[c] = W[(uint64_t)st.piv[c] * ld + col];
+#pragma unroll
+    for (int m = 0; m < SP; ++m) d[m] = m < st.moves ? W[(uint64_t)st.from[m] * ld + col] : 0.0f;
+    const bool in_panel = col < (uint64_t)j + SP;
+    // R = U^-1 (L^-1 v): forward substitution with the unit lower factor, back substitution with the upper one
+#pragma unroll
+    for (int r = 1; r < SP; ++r)
+#pragma unroll
+        for (int q = 0; q < r; ++q) v[r] = fmaf(-st.lu[r * SP + q], v[q], v[r]);
+#pragma unroll
+    for (int r = SP - 1; r >= 0; --r) {
+#pragma unroll
+        for (int q = r + 1; q < SP; ++q) v[r] = fmaf(-st.lu[r * SP + q], v[q], v[r]);
+        v[r] = v[r] / st.lu[r * SP + r];
+    }
+#pragma unroll
+    for (int c = 0; c < SP; ++c) W[(uint64_t)(j + c) * ld + col] = in_panel ? 0.0f : v[c];
+#pragma unroll
+    for (int m = 0; m < SP; ++m)
+        if (m < st.moves) W[(uint64_t)st.to[m] * ld + col] = d[m];
+}
+
+__global__ __launch_bounds__(256) void gj_copy_out_kernel(const float* __restrict__ W, uint64_t ld, uint64_t np,
+                                                          uint64_t n, float* __restrict__ inv, uint64_t ldi) {
+    const uint64_t idx = (uint64_t)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= n * n) return;
+    const uint64_t i = idx / n, c = idx % n;
+    inv[i * ldi + c] = W[i * ld + np + c];
+}
+
+template <int SP, int RPT>
+int gj_run(float* W, uint32_t np, GjStep* steps, int32_t* status, hipStream_t s) {
+    const uint64_t ld = 2ull * np;
+    for (uint32_t j = 0; j < np; j += SP) {
+        GjStep* st = steps + (j / SP) % 2;  // two records in turn: the next panel never overwrites one still in use
+        hipLaunchKernelGGL((gj_panel_kernel<SP, RPT>), dim3(1), dim3(kGjThreads), 0, s, W, ld, np, j, st, status);
+        const uint32_t cols = 2 * np - j;
+        hipLaunchKernelGGL((gj_rows_kernel<SP>), dim3((cols + 255) / 256), dim3(256), 0, s, W, ld, np, j, st);
+        if (hipGetLastError() != hipSuccess) return TRAKHIP_ERR_LAUNCH;
+        const int e = trakhip::gemm_nn(W + j, ld, W + (uint64_t)j * ld + j + SP, ld, W + j + SP, ld, np,
+                                       2ull * np - j - SP, SP, -1.0f, 1.0f, s, 0);
+        if (e) return e;
+    }
+    return TRAKHIP_OK;
+}
+
+}  // namespace
+
+namespace trakhip {
+
+constexpr uint64_t kGeneralInverseMaxN = 12288;
+
+size_t general_inverse_workspace_bytes(uint64_t n) {
+    if (n == 0 || n > kGeneralInverseMaxN) return 0;
+    const uint64_t np = (n + NB - 1) / NB * NB;
+    return (size_t)(2 * np * np + kSumBlocks + 4) * sizeof(float) + 2 * sizeof(GjStep);
+}
+
+int general_inverse(const float* A, uint64_t lda, float lambda, float* inv, uint64_t ldi, uint64_t n, int normalize,
+                    float* mean_abs, int32_t* status, void* ws, size_t ws_bytes, hipStream_t s) {
+    if (n == 0) return TRAKHIP_OK;
+    if (!A || !inv || !ws) return TRAKHIP_ERR_NULL;
+    if (lda < n || ldi < n || n > kGeneralInverseMaxN) return TRAKHIP_ERR_SHAPE;
+    if (ws_bytes < general_inverse_workspace_bytes(n)) return TRAKHIP_ERR_WORKSPACE;
+    if (reinterpret_cast<uintptr_t>(ws) % 16) return TRAKHIP_ERR_ALIGN;
+    const uint64_t np = (n + NB - 1) / NB * NB;
+    float* W = static_cast<float*>(ws);
+    float* partial = W + 2 * np * np;
+    float* mean_dev = partial + kSumBlocks;
+    GjStep* steps = reinterpret_cast<GjStep*>(mean_dev + 4);
+    hipLaunchKernelGGL(gj_init_kernel, dim3((uint32_t)((2 * np * np + 255) / 256)), dim3(256), 0, s, A, lda, lambda, n,
+                       np, W, status);
+    if (hipGetLastError() != hipSuccess) return TRAKHIP_ERR_LAUNCH;
+    // the panel's rows live in the registers of one workgroup: 16 columns of up to 6144 rows, or 8 of up to 12288
+    const int e = np <= 6144 ? gj_run<16, 6>(W, (uint32_t)np, steps, status, s)
+                             : gj_run<8, 12>(W, (uint32_t)np, steps, status, s);
+    if (e) return e;
+    hipLaunchKernelGGL(gj_copy_out_kernel, dim3((uint32_t)((n * n + 255) / 256)), dim3(256), 0, s, W, 2 * np, np, n, inv,
+                       ldi);
+    if (normalize || mean_abs) {
+        hipLaunchKernelGGL(abs_sum_kernel, dim3(kSumBlocks), dim3(256), 0, s, inv, ldi, n, partial);
+        hipLaunchKernelGGL(mean_kernel, dim3(1), dim3(256), 0, s, partial, n, mean_dev, mean_abs);
+        if (normalize)
+            hipLaunchKernelGGL(scale_kernel, dim3((uint32_t)((n * n + 255) / 256)), dim3(256), 0, s, inv, ldi, n,
+                               mean_dev);
+    }
+    return hipGetLastError() == hipSuccess ? TRAKHIP_OK : TRAKHIP_ERR_LAUNCH;
 }
 
 }  // namespace trakhip

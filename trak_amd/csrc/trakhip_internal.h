@@ -78,5 +78,9 @@ int gemm_nt16(const void* A, uint64_t lda, const void* B, uint64_t ldb, int dtyp
 size_t spd_inverse_workspace_bytes(uint64_t n);
 int spd_inverse(const float* A, uint64_t lda, float lambda, float* inv, uint64_t ldi, uint64_t n,
                 int normalize, float* mean_abs, int32_t* status, void* ws, size_t ws_bytes, hipStream_t s);
+// the same for any nonsingular matrix (Gauss-Jordan elimination with partial pivoting)
+size_t general_inverse_workspace_bytes(uint64_t n);
+int general_inverse(const float* A, uint64_t lda, float lambda, float* inv, uint64_t ldi, uint64_t n,
+                    int normalize, float* mean_abs, int32_t* status, void* ws, size_t ws_bytes, hipStream_t s);
 
 }  // namespace trakhip

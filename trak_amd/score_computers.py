@@ -72,9 +72,11 @@ class BasicScoreComputer(AbstractScoreComputer):
       * `X^T X + lambda I` is inverted by a Cholesky factorization.  When that fails - the matrix is
         symmetric but not positive definite, which happens to a Gram matrix that was rounded to fp16
         (TRAKer's default) or has deficient rank (fewer training points than proj_dim with
-        lambda_reg = 0) - it falls back to LU through torch.linalg.inv on the device, the call the
-        reference itself makes (trak/score_computers.py:163), and logs a warning; only an exactly
-        singular matrix or a non-finite inverse raises torch.linalg.LinAlgError;
+        lambda_reg = 0) - the matrix is inverted by this library's elimination with partial pivoting
+        (`utils.general_inverse`: the pivoting of the LU behind the reference's torch.linalg.inv,
+        trak/score_computers.py:163; matrices up to 12288 x 12288) and a warning is logged; an exactly
+        singular matrix (a zero pivot) raises torch.linalg.LinAlgError as the reference's call does, an
+        inverse with huge or non-finite entries is handed on as it is;
       * sums are kept in fp32 and rounded to `dtype` once.  accumulate_in_dtype=True reproduces the
         reference's arithmetic instead: `X^T X` is the sum over blocks of CUDA_MAX_DIM_SIZE rows of
         block products each rounded to `dtype`, the running sum rounded to `dtype` after every

@@ -359,31 +359,24 @@ def gram_split(a, out=None, alpha=1.0, beta=0.0):
     return out
 
 
-def spd_inverse(a, lambda_reg=0.0, normalize=False, general_fallback=False):
-    """(a + lambda*I)^-1 for a symmetric positive definite fp32 matrix on the GPU; with
-    normalize=True the result is divided by mean(|inverse|) (trak/score_computers.py:160-166).
-    Returns (inverse, mean_abs tensor of 1 element).
-
-    A matrix that is not positive definite raises torch.linalg.LinAlgError, unless
-    general_fallback=True: then it is inverted by LU with torch.linalg.inv on the device - the very
-    call the reference makes at trak/score_computers.py:163 - which returns something for every
-    matrix that is not exactly singular (a Gram matrix rounded to fp16, or one of deficient rank,
-    is symmetric but need not be positive definite)."""
-    if a.dim() != 2 or a.shape[0] != a.shape[1]:
-        raise RuntimeError("spd_inverse needs a square matrix")
-    a = _as_f32_rows(a, "a")
-    if not a.is_cuda:
-        raise RuntimeError("spd_inverse needs a GPU tensor")
+def _inverse_call(a, lambda_reg, normalize, general):
+    """One call of trakhip_spd_inverse (Cholesky) or trakhip_general_inverse (pivoted Gauss-Jordan):
+    (inverse, mean_abs, status word)."""
     n = a.shape[0]
     lib = _lib.load()
+    size, run = ((lib.trakhip_general_inverse_workspace, lib.trakhip_general_inverse) if general
+                 else (lib.trakhip_spd_inverse_workspace, lib.trakhip_spd_inverse))
     with torch.cuda.device(a.device):
+        nbytes = size(n)
+        if general and nbytes == 0:
+            raise torch.linalg.LinAlgError(
+                f"the matrix is not positive definite and too large (n = {n}) for the general inverse of this library")
         inv = torch.empty((n, n), dtype=torch.float32, device=a.device)
         mean_abs = torch.zeros(1, dtype=torch.float32, device=a.device)
         status = torch.zeros(1, dtype=torch.int32, device=a.device)
-        nbytes = lib.trakhip_spd_inverse_workspace(n)
         ws = torch.empty(max(nbytes, 1), dtype=torch.uint8, device=a.device)
         stream = torch.cuda.current_stream(a.device).cuda_stream
-        code = lib.trakhip_spd_inverse(
+        code = run(
             ctypes.c_void_p(a.data_ptr()),
             _ld(a),
             float(lambda_reg),
@@ -399,21 +392,53 @@ def spd_inverse(a, lambda_reg=0.0, normalize=False, general_fallback=False):
         )
         _lib.check(code)
         bad = int(status.item())  # also orders the workspace's lifetime after the kernels
+    return inv, mean_abs, bad
+
+
+def general_inverse(a, lambda_reg=0.0, normalize=False):
+    """(a + lambda*I)^-1 for any nonsingular fp32 matrix on the GPU, by Gauss-Jordan elimination with
+    partial pivoting - the pivoting of the LU behind torch.linalg.inv, the reference's call
+    (trak/score_computers.py:163); with normalize=True divided by mean(|inverse|).  Returns (inverse,
+    mean_abs).  An exactly singular matrix (a zero pivot) raises torch.linalg.LinAlgError, as the
+    reference's call does; an inverse with huge or non-finite entries is returned as it is."""
+    if a.dim() != 2 or a.shape[0] != a.shape[1]:
+        raise RuntimeError("general_inverse needs a square matrix")
+    a = _as_f32_rows(a, "a")
+    if not a.is_cuda:
+        raise RuntimeError("general_inverse needs a GPU tensor")
+    inv, mean_abs, bad = _inverse_call(a, lambda_reg, normalize, general=True)
+    if bad != 0:
+        raise torch.linalg.LinAlgError(f"general_inverse: the matrix is singular (pivot {bad - 1} is zero)")
+    return inv, mean_abs
+
+
+def spd_inverse(a, lambda_reg=0.0, normalize=False, general_fallback=False):
+    """(a + lambda*I)^-1 for a symmetric positive definite fp32 matrix on the GPU; with
+    normalize=True the result is divided by mean(|inverse|) (trak/score_computers.py:160-166).
+    Returns (inverse, mean_abs tensor of 1 element).
+
+    A matrix that is not positive definite raises torch.linalg.LinAlgError, unless
+    general_fallback=True: then it is inverted by `general_inverse` (elimination with partial
+    pivoting on the device, the pivoting of the reference's torch.linalg.inv at
+    trak/score_computers.py:163), which returns something for every matrix that is not exactly
+    singular (a Gram matrix rounded to fp16, or one of deficient rank, is symmetric but need not
+    be positive definite)."""
+    if a.dim() != 2 or a.shape[0] != a.shape[1]:
+        raise RuntimeError("spd_inverse needs a square matrix")
+    a = _as_f32_rows(a, "a")
+    if not a.is_cuda:
+        raise RuntimeError("spd_inverse needs a GPU tensor")
+    inv, mean_abs, bad = _inverse_call(a, lambda_reg, normalize, general=False)
     if bad != 0:
         if not general_fallback:
             raise torch.linalg.LinAlgError(
                 f"spd_inverse: the matrix is not positive definite (pivot {bad - 1} is not positive)"
             )
         logging.getLogger("ScoreComputer").warning(
-            "X^T X + lambda I is not positive definite (pivot %d): inverting it by LU, as the reference does", bad - 1
+            "X^T X + lambda I is not positive definite (pivot %d): inverting it with partial pivoting, as the "
+            "reference's LU does", bad - 1
         )
-        reg = a + float(lambda_reg) * torch.eye(n, device=a.device, dtype=torch.float32)
-        inv = torch.linalg.inv(reg)  # raises LinAlgError for an exactly singular matrix, like the reference
-        if not bool(torch.isfinite(inv).all()):
-            raise torch.linalg.LinAlgError("spd_inverse: the inverse has non-finite entries")
-        mean_abs = inv.abs().mean().reshape(1)
-        if normalize:
-            inv = inv / mean_abs
+        return general_inverse(a, lambda_reg, normalize)
     return inv, mean_abs
 
 
