@@ -92,7 +92,7 @@ def test_workspace_size():
     assert lib.trakhip_project_workspace(16, 1_048_576, 512, 256) == 256 * 16 * 512 * 4  # one 512-column block
     assert lib.trakhip_project_workspace(0, 25, 1024, 256) == 0
     # column-block counts that do not divide 256: never more workgroups than CUs
-    for k, blocks in ((1536, 3), (3072, 3), (5120, 5), (15_360, 15), (40_960, 40)):
+    for k, blocks in ((1536, 2), (2560, 5), (3072, 3), (4608, 6), (5120, 5), (15_360, 15), (40_960, 40)):  # 768-, 512-, 1024-column blocks
         groups = 256 // blocks
         assert lib.trakhip_project_workspace(32, 11_689_512, k, 256) == groups * 32 * k * 4, k
     assert lib.trakhip_spd_inverse_workspace(4096) >= 3 * 4096 * 4096 * 4
@@ -129,6 +129,15 @@ def test_gemm_argument_validation_needs_no_device():
     assert lib.trakhip_gemm_tn(p, 2, p, 8, p, 8, 4, 4, 16, 1.0, 0.0, None) == -2          # lda < M
     assert lib.trakhip_spd_inverse(p, 2, 0.0, p, 4, 4, 0, None, None, p, 1 << 30, None) == -2
     assert lib.trakhip_spd_inverse(p, 4, 0.0, p, 4, 4, 0, None, None, p, 16, None) == -6
+    # the general (pivoted) inverse: same argument checks; an augmented matrix [A | I] as workspace; n <= 12288
+    assert lib.trakhip_general_inverse_workspace(4096) >= 2 * 4096 * 4096 * 4
+    assert lib.trakhip_general_inverse_workspace(100) >= 2 * 128 * 128 * 4
+    assert lib.trakhip_general_inverse_workspace(0) == 0 and lib.trakhip_general_inverse_workspace(12_289) == 0
+    assert lib.trakhip_general_inverse(p, 2, 0.0, p, 4, 4, 0, None, None, p, 1 << 30, None) == -2
+    assert lib.trakhip_general_inverse(p, 4, 0.0, p, 4, 4, 0, None, None, p, 16, None) == -6
+    assert lib.trakhip_general_inverse(None, 4, 0.0, p, 4, 4, 0, None, None, p, 1 << 30, None) == -5
+    assert lib.trakhip_general_inverse(p, 20_000, 0.0, p, 20_000, 20_000, 0, None, None, p, 1 << 40, None) == -2
+    assert lib.trakhip_general_inverse(p, 4, 0.0, p, 4, 0, 0, None, None, p, 0, None) == 0      # empty matrix
 
 
 def test_store_entry_points_validate_before_touching_the_device():

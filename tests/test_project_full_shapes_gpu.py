@@ -27,13 +27,13 @@ CHUNK = 256
 
 def launch_plan(P, k, tiles, cus):
     """The split of a launch as the library documents it: feature tiles of ceil(P / T) features walked in
-    chunks of 256, column blocks of 1024 columns (512 when k is an odd multiple of 512), and
+    chunks of 256, column blocks of 1024 columns (768 or 512 when k is an odd multiple of 512), and
     floor(CUs / column blocks) runs of consecutive chunks."""
     T = min(P, tiles)
     fts = (P - 1) // T + 1
     cpt = (fts + CHUNK - 1) // CHUNK
     total = T * cpt
-    col_blocks = k // 1024 if k % 1024 == 0 else k // 512
+    col_blocks = k // 1024 if k % 1024 == 0 else k // 768 if k % 768 == 0 else k // 512
     groups = max(1, min(total, cus // col_blocks))
     cpg = (total + groups - 1) // groups
     groups = (total + cpg - 1) // cpg
@@ -86,7 +86,9 @@ CASES = [
     ("resnet9", 32, 4_825_610, 2048, 0, torch.float16, R),
     ("resnet18_k3072", 32, 11_689_512, 3072, 7, torch.float16, R),     # runs that start inside a tile
     ("resnet18_k15360", 32, 11_689_512, 15_360, 7, torch.float16, R),  # 15 column blocks, 17 runs
-    ("resnet18_k1536", 32, 11_689_512, 1536, 7, torch.bfloat16, R),    # 512-column workgroups
+    ("resnet18_k1536", 32, 11_689_512, 1536, 7, torch.bfloat16, R),    # 768-column workgroups
+    ("resnet18_k2560", 32, 11_689_512, 2560, 7, torch.float16, R),     # 512-column workgroups
+    ("resnet18_k1536_normal_64rows", 64, 11_689_512, 1536, 7, torch.float16, G),
     ("bert_chunk_normal", 32, 27_370_560, 4096, 123, torch.bfloat16, G),
     ("bert_chunk_normal_64rows", 64, 27_370_560, 4096, 123, torch.bfloat16, G),
 ]

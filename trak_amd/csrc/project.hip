@@ -517,7 +517,8 @@ __device__ __forceinline__ void for_each_step(F& f, std::integer_sequence<int, S
 
 // GATHER: g_in is a device array of trakhip_segment and ld their number; otherwise g_in is the
 // dense [rows, P] matrix with row pitch ld.  GPW = 32-column groups per wave: 4 (workgroup = 1024
-// columns) or 2 (512 columns, for projection dimensions that are an odd multiple of 512).
+// columns), or for projection dimensions that are an odd multiple of 512: 3 (768 columns) when 768
+// divides the dimension, else 2 (512 columns).
 //
 // The main loop is written out step by step.  A chunk is 16 * GPW steps (q, j): one table lookup
 // and one MFMA (three for fp32 gradients) for column group j and features 8q..8q+7 of the lane's
@@ -1300,7 +1301,9 @@ struct Plan {
 Plan make_plan(uint64_t P, uint32_t k, uint32_t num_feature_tiles) {
     Plan p;
     p.tl = jl::make_tiling(P, num_feature_tiles);
-    p.gpw = (k % (8 * 4 * 32) == 0) ? 4 : 2;
+    // columns per workgroup: 1024 (four 32-column groups per wave) when that divides k, else 768 (three),
+    // else 512 (two); k is a multiple of 512
+    p.gpw = (k % (8 * 4 * 32) == 0) ? 4 : (k % (8 * 3 * 32) == 0) ? 3 : 2;
     p.col_blocks = k / (8 * p.gpw * 32);
     p.chunks_per_tile = (uint32_t)((p.tl.tile_size + kChunk - 1) / kChunk);
     const uint64_t total = (uint64_t)p.tl.tiles * p.chunks_per_tile;
@@ -1348,8 +1351,9 @@ constexpr int kNormalWaves = JL_NORMAL_WAVES, kNormalWaves2 = JL_NORMAL_WAVES_RB
 template <int IN, bool GATHER, int GPW>
 hipError_t launch_normal(const void* in, uint64_t ld, uint32_t rows, uint64_t P, uint32_t k, uint32_t seed,
                          const Plan& pl, float* partial, hipStream_t s) {
-    constexpr int W = kNormalWaves, G = 8 * GPW / W;  // same columns per workgroup as the plan's 8 waves x GPW
-    constexpr int W2 = kNormalWaves2, G2 = 8 * GPW / W2;
+    // same columns per workgroup as the plan's 8 waves x GPW groups; an odd GPW keeps 8 waves
+    constexpr int W = (8 * GPW) % kNormalWaves == 0 ? kNormalWaves : 8, G = 8 * GPW / W;
+    constexpr int W2 = (8 * GPW) % kNormalWaves2 == 0 ? kNormalWaves2 : 8, G2 = 8 * GPW / W2;
     static_assert(G >= 1 && G * W == 8 * GPW && G2 >= 1 && G2 * W2 == 8 * GPW, "column groups per wave");
     const uint64_t wgs = plan_workgroups(pl);
     if (wgs > 0x7FFFFFFFull) return hipErrorInvalidValue;
@@ -1386,7 +1390,9 @@ LaunchFn pick_w(int dtype, int proj_type, bool gather) {
 }
 
 LaunchFn pick(const Plan& pl, int dtype, int proj_type, bool gather) {
-    return pl.gpw == 4 ? pick_w<4>(dtype, proj_type, gather) : pick_w<2>(dtype, proj_type, gather);
+    return pl.gpw == 4   ? pick_w<4>(dtype, proj_type, gather)
+           : pl.gpw == 3 ? pick_w<3>(dtype, proj_type, gather)
+                         : pick_w<2>(dtype, proj_type, gather);
 }
 
 }  // namespace
