@@ -21,7 +21,7 @@ other_configs = whole calls (Python wrapper included) of the other benchmark con
             a gradient dict, and projection dimensions 3072 and 15 360.
 `--only NAME` runs one workload alone (for profiler runs): c1 | c2 | c3_b40 | c3_b48 | c3_b64 | c3_k1536 | c3_k3072 |
             c3_k15360 | c3_k40960 | c3_normal_b32 | c3_normal_b64 | c3_dict | c4 | c4_rademacher | vendor_gemm | scoring |
-            mfma_rate.
+            general_inverse | mfma_rate.
 """
 import argparse
 import ctypes
@@ -332,6 +332,32 @@ def bench_config(torch, dev, name, reps, warm_seconds=0.1, min_seconds=0.25):
     torch.cuda.synchronize()
     ms = a.elapsed_time(b) / reps
     return {"what": what, "ms": ms, "tflops": flop / ms / 1e9, "calls": reps}
+
+
+def bench_general_inverse(torch, dev, n=4096, reps=3):
+    """The inverse of a Gram matrix that is not positive definite (rounded to fp16) at proj_dim n: this library's
+    pivoted elimination against the Cholesky route on the same matrix plus a ridge, and torch.linalg.inv (the
+    reference's call, the vendor's LU) for comparison."""
+    from trak_amd.utils import general_inverse, spd_inverse
+
+    gen = torch.Generator(device=dev).manual_seed(5)
+    q, _ = torch.linalg.qr(torch.randn(n, n, generator=gen, device=dev, dtype=torch.float64))
+    spectrum = 1000.0 / torch.arange(1, n + 1, dtype=torch.float64, device=dev) ** 1.5
+    gram = ((q * spectrum) @ q.T).half().float()
+    del q
+
+    def timed(fn):
+        fn()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            fn()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) * 1e3 / reps
+
+    return {"n": n, "general_inverse_ms": timed(lambda: general_inverse(gram, normalize=True)),
+            "spd_inverse_with_ridge_ms": timed(lambda: spd_inverse(gram, lambda_reg=1.0, normalize=True)),
+            "torch_linalg_inv_ms": timed(lambda: torch.linalg.inv(gram))}
 
 
 MFMA_RATE_CASES = [
@@ -667,8 +693,11 @@ def main():
     ap.add_argument("--only", default=None, metavar="NAME",
                     help="run just one workload for --steps calls and print its timing (for profiler runs): "
                          "c1 | c2 | c3_b40 | c3_b48 | c3_b64 | c3_k1536 | c3_k3072 | c3_k15360 | c3_k40960 | c3_normal_b32 | "
-                         "c3_normal_b64 | c3_dict | c4 | c4_rademacher | scoring | mfma_rate | vendor_gemm "
+                         "c3_normal_b64 | c3_dict | c4 | c4_rademacher | scoring | general_inverse | mfma_rate | vendor_gemm "
                          "(torch.mm on the scoring operands, for comparison)")
+    ap.add_argument("--steady", action="store_true",
+                    help="with --only: at least 0.1 s of untimed calls first and at least 0.25 s timed (for timing without "
+                         "a profiler: an idle GPU's clocks take tens of milliseconds to come up)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run one 1 GiB device-to-device copy (reference point for rocprofv3 byte counters)")
     args = ap.parse_args()
@@ -694,10 +723,14 @@ def main():
             print(json.dumps({"only": "mfma_rate", **bench_mfma_rate(torch, dev)}))
         elif args.only == "vendor_gemm":
             print(json.dumps({"only": "vendor_gemm", **bench_vendor_gemm(torch, dev)}))
+        elif args.only == "general_inverse":
+            print(json.dumps({"only": "general_inverse", **bench_general_inverse(torch, dev)}))
         elif args.only == "scoring":
             print(json.dumps({"only": "scoring", **bench_scoring(torch, dev, reps=max(1, min(args.steps, 3)))}))
         else:
-            print(json.dumps({"only": args.only, **bench_config(torch, dev, args.only, args.steps)}))
+            # exactly --steps calls after one warm-up call (profiler runs); --steady: warmed up and timed by wall time
+            w, m = (0.1, 0.25) if args.steady else (0.0, 0.0)
+            print(json.dumps({"only": args.only, **bench_config(torch, dev, args.only, args.steps, w, m)}))
         return
     proj = bench_projection(torch, dev, args.steps, args.warmup, args.batches, args.sustain)
     torch.cuda.empty_cache()

@@ -613,6 +613,8 @@ __global__ __launch_bounds__(kGjThreads) void gj_panel_kernel(const float* __res
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     float a[RPT][SP];
     uint32_t live = 0;  // bit i: row i of this thread exists and has not been a pivot
+    // row slots of a thread that hold rows at all at this j (the panel shrinks as j grows)
+    const int slots = (int)((np - j + kGjThreads - 1) / kGjThreads);
 #pragma unroll
     for (int i = 0; i < RPT; ++i) {
         const uint32_t r = j + (uint32_t)tid + (uint32_t)kGjThreads * i;
@@ -637,7 +639,7 @@ __global__ __launch_bounds__(kGjThreads) void gj_panel_kernel(const float* __res
         uint32_t key = 0, row = 0xFFFFFFFFu;
 #pragma unroll
         for (int i = 0; i < RPT; ++i)
-            if (live & (1u << i))
+            if (i < slots && (live & (1u << i)))
                 gj_better(key, row, __float_as_uint(fabsf(a[i][c])), j + (uint32_t)tid + (uint32_t)kGjThreads * i);
 #pragma unroll
         for (int d = 1; d < 64; d <<= 1)
@@ -650,7 +652,7 @@ __global__ __launch_bounds__(kGjThreads) void gj_panel_kernel(const float* __res
         // its owner publishes the row (multipliers of earlier columns in front, the eliminated row behind)
 #pragma unroll
         for (int i = 0; i < RPT; ++i) {
-            if ((live & (1u << i)) && row == j + (uint32_t)tid + (uint32_t)kGjThreads * i) {
+            if (i < slots && (live & (1u << i)) && row == j + (uint32_t)tid + (uint32_t)kGjThreads * i) {
                 live &= ~(1u << i);
 #pragma unroll
                 for (int c2 = 0; c2 < SP; ++c2) lu[c][c2] = a[i][c2];
@@ -659,11 +661,12 @@ __global__ __launch_bounds__(kGjThreads) void gj_panel_kernel(const float* __res
             }
         }
         __syncthreads();
-        const float pivot = lu[c][c];
+        // multipliers by the reciprocal of the pivot, as LAPACK's unblocked LU scales a column
+        const float rpivot = 1.0f / lu[c][c];
 #pragma unroll
         for (int i = 0; i < RPT; ++i) {
-            if (live & (1u << i)) {
-                const float l = a[i][c] / pivot;
+            if (i < slots && (live & (1u << i))) {  // (i < slots: the same for the whole workgroup)
+                const float l = a[i][c] * rpivot;
                 a[i][c] = l;
 #pragma unroll
                 for (int c2 = c + 1; c2 < SP; ++c2) a[i][c2] = fmaf(-l, lu[c][c2], a[i][c2]);
