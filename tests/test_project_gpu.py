@@ -622,3 +622,23 @@ def test_many_rows_gather(gpu):
     grads = {i: torch.randn(100, n, generator=gen).half().to(gpu) for i, n in enumerate([300, 1, 4097, 15, 2000])}
     flat = vectorize(grads, device=gpu)
     assert torch.equal(fast_jl.project_gather(list(grads.values()), 512, 3, 256, "rademacher"), fn(R)(flat, 512, 3, 256))
+
+
+def test_workspace_cache_is_bounded_and_streams_do_not_share_scratch(gpu):
+    # one scratch buffer per (device, stream), at most eight of them kept; a projection on a side stream gives
+    # the bits of one on the default stream
+    g = (torch.randn(8, 3_000, generator=torch.Generator().manual_seed(4)) * 1e-2).half().to(gpu)
+    want = fn(R)(g, 512, 3, 256)
+    torch.cuda.synchronize()
+    fast_jl.free_workspaces()
+    streams = [torch.cuda.Stream(device=gpu) for _ in range(11)]
+    for s in streams:
+        with torch.cuda.stream(s):
+            got = fn(R)(g, 512, 3, 256)
+        s.synchronize()
+        assert torch.equal(got, want)
+    assert 1 <= len(fast_jl._workspaces) <= fast_jl._WORKSPACE_CACHE
+    kept = {key[1] for key in fast_jl._workspaces}
+    assert streams[-1].cuda_stream in kept and streams[0].cuda_stream not in kept   # least recently used went first
+    fast_jl.free_workspaces()
+    assert not fast_jl._workspaces and not fast_jl._segment_tables

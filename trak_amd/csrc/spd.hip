@@ -638,38 +638,51 @@ __global__ __launch_bounds__(kGjThreads) void gj_panel_kernel(const float* __res
         // the pivot of column c: largest |a| among the rows that have not been pivots
         uint32_t key = 0, row = 0xFFFFFFFFu;
 #pragma unroll
-        for (int i = 0; i < RPT; ++i)
-            if (i < slots && (live & (1u << i)))
-                gj_better(key, row, __float_as_uint(fabsf(a[i][c])), j + (uint32_t)tid + (uint32_t)kGjThreads * i);
+        for (int i = 0; i < RPT; ++i) {
+            if (i < slots) {  // the same for the whole workgroup: a scalar branch
+                if (live & (1u << i))
+                    gj_better(key, row, __float_as_uint(fabsf(a[i][c])), j + (uint32_t)tid + (uint32_t)kGjThreads * i);
+            }
+        }
 #pragma unroll
         for (int d = 1; d < 64; d <<= 1)
             gj_better(key, row, (uint32_t)__shfl_xor((int)key, d, 64), (uint32_t)__shfl_xor((int)row, d, 64));
         if (lane == 0) cand_key[wave] = key, cand_row[wave] = row;
         __syncthreads();
-        key = cand_key[0], row = cand_row[0];
+        // the sixteen waves' candidates, one per lane of every group of sixteen lanes, reduced inside the group
+        static_assert(kGjThreads / 64 == 16, "one candidate per lane of a group of sixteen");
+        key = cand_key[lane & 15], row = cand_row[lane & 15];
 #pragma unroll
-        for (int w = 1; w < kGjThreads / 64; ++w) gj_better(key, row, cand_key[w], cand_row[w]);
-        // its owner publishes the row (multipliers of earlier columns in front, the eliminated row behind)
+        for (int d = 1; d < 16; d <<= 1)
+            gj_better(key, row, (uint32_t)__shfl_xor((int)key, d, 64), (uint32_t)__shfl_xor((int)row, d, 64));
+        // its owner - one thread, known to all: row = j + thread + 1024 * slot - publishes the row (multipliers of
+        // earlier columns in front, the eliminated row behind)
+        const uint32_t rel = __builtin_amdgcn_readfirstlane(row) - j;
+        const int owner = (int)(rel % kGjThreads), owner_slot = (int)(rel / kGjThreads);
+        if (tid == owner) {
 #pragma unroll
-        for (int i = 0; i < RPT; ++i) {
-            if (i < slots && (live & (1u << i)) && row == j + (uint32_t)tid + (uint32_t)kGjThreads * i) {
-                live &= ~(1u << i);
+            for (int i = 0; i < RPT; ++i) {
+                if (i == owner_slot) {
+                    live &= ~(1u << i);
 #pragma unroll
-                for (int c2 = 0; c2 < SP; ++c2) lu[c][c2] = a[i][c2];
-                piv[c] = (int32_t)row;
-                if (a[i][c] == 0.0f && status) *status = (int32_t)(j + c + 1);  // exactly singular
+                    for (int c2 = 0; c2 < SP; ++c2) lu[c][c2] = a[i][c2];
+                    if (a[i][c] == 0.0f && status) *status = (int32_t)(j + c + 1);  // exactly singular
+                }
             }
+            piv[c] = (int32_t)(rel + j);
         }
         __syncthreads();
         // multipliers by the reciprocal of the pivot, as LAPACK's unblocked LU scales a column
         const float rpivot = 1.0f / lu[c][c];
 #pragma unroll
         for (int i = 0; i < RPT; ++i) {
-            if (i < slots && (live & (1u << i))) {  // (i < slots: the same for the whole workgroup)
-                const float l = a[i][c] * rpivot;
-                a[i][c] = l;
+            if (i < slots) {
+                if (live & (1u << i)) {
+                    const float l = a[i][c] * rpivot;
+                    a[i][c] = l;
 #pragma unroll
-                for (int c2 = c + 1; c2 < SP; ++c2) a[i][c2] = fmaf(-l, lu[c][c2], a[i][c2]);
+                    for (int c2 = c + 1; c2 < SP; ++c2) a[i][c2] = fmaf(-l, lu[c][c2], a[i][c2]);
+                }
             }
         }
     };
