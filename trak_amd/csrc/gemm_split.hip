@@ -315,7 +315,9 @@ __device__ __forceinline__ void store_c(const floatx16 (&acc)[2][JT], float* __r
                         else
                             o[c] = alpha * v[c] * rs;
                     }
-                    *reinterpret_cast<float4u*>(p + 32 * j) = o;
+                    // streaming store: C is written once and is far larger than L2, where the operand panels
+                    // that other workgroups are about to read should stay
+                    __builtin_nontemporal_store(o, reinterpret_cast<float4u*>(p + 32 * j));
                 }
             }
         }
