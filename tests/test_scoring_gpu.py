@@ -202,7 +202,9 @@ def test_gram_matrices_that_are_not_positive_definite(gpu):
     assert out.dtype == torch.float16 and torch.isfinite(out).all()
 
 
-@pytest.mark.parametrize("n", [1, 5, 16, 100, 128, 129, 300, 1000, 2048])
+# (up to 2944 every elimination step goes over the whole matrix; from 3072 on the steps run inside blocks of 64
+# columns; above 6144 the panels are 8 columns wide instead of 16)
+@pytest.mark.parametrize("n", [1, 5, 16, 100, 128, 129, 300, 1000, 2048, 3100, 6200])
 def test_general_inverse_against_float64(gpu, n):
     # nonsymmetric, indefinite, well conditioned: inverse to fp32 accuracy, A * inv = I
     from trak_amd.utils import general_inverse
@@ -213,7 +215,9 @@ def test_general_inverse_against_float64(gpu, n):
     a64 = a.double().numpy() + 0.25 * np.eye(n)
     want = np.linalg.inv(a64)
     got = inv.cpu().numpy().astype(np.float64)
-    assert np.abs(got - want).max() <= 2e-5 * np.abs(want).max() * max(1.0, np.linalg.cond(a64) / 10)
+    # (the condition number in the 2-norm, or for the large cases its cheaper bound through 1-norms)
+    cond = np.linalg.cond(a64) if n <= 2048 else np.linalg.norm(a64, 1) * np.linalg.norm(want, 1)
+    assert np.abs(got - want).max() <= 2e-5 * np.abs(want).max() * max(1.0, cond / 10)
     assert np.abs(a64 @ got - np.eye(n)).max() < 1e-4
     assert abs(mean_abs.item() - np.abs(got).mean()) <= 1e-5 * np.abs(got).mean()
     norm, _ = general_inverse(a.to(gpu), lambda_reg=0.25, normalize=True)
@@ -245,6 +249,36 @@ def test_general_inverse_needs_its_pivoting(gpu):
         general_inverse(c.to(gpu))
     with pytest.raises(torch.linalg.LinAlgError):
         torch.linalg.inv(c.to(gpu))
+
+
+def test_general_inverse_in_column_blocks_needs_its_pivoting(gpu):
+    # the same three situations at a size where the steps run inside blocks of 64 columns
+    from trak_amd.utils import general_inverse
+
+    n = 3300
+    perm = torch.randperm(n, generator=torch.Generator().manual_seed(3))
+    a = torch.zeros(n, n)
+    a[torch.arange(n), perm] = 1.0 + torch.arange(n, dtype=torch.float32) / 1024    # a scaled permutation matrix
+    inv, _ = general_inverse(a.to(gpu))
+    assert torch.equal(inv.cpu(), torch.linalg.inv(a.double()).float())              # exact: one entry per row
+    # pivots far below the block, rows displaced more than once within a block and from block to block
+    gen = torch.Generator().manual_seed(4)
+    b = torch.randn(n, n, generator=gen)
+    b[:700] *= 1e-3
+    got, _ = general_inverse(b.to(gpu))
+    # condition number about 1e7: measured against what LU with the same pivoting makes of it in fp32
+    ref = torch.linalg.inv(b.to(gpu)).double()
+    b64 = b.double().to(gpu)
+    want = torch.linalg.inv(b64)
+    eye = torch.eye(n, device=gpu, dtype=torch.float64)
+    err, ref_err = (float((m - want).abs().max() / want.abs().max()) for m in (got.double(), ref))
+    resid, ref_resid = (float((b64 @ m - eye).abs().max()) for m in (got.double(), ref))
+    assert err <= 4 * ref_err + 1e-5 and resid <= 2 * ref_resid + 1e-3, (err, ref_err, resid, ref_resid)
+    # a zero column in the last panel of a block
+    c = torch.randn(n, n, generator=gen)
+    c[:, 3135] = 0.0
+    with pytest.raises(torch.linalg.LinAlgError):
+        general_inverse(c.to(gpu))
 
 
 def test_general_inverse_of_an_indefinite_gram_matrix_at_proj_dim_4096(gpu):

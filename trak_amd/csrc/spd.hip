@@ -560,6 +560,16 @@ namespace {
 //      panel entries were set to zero, so they pass through unchanged).
 // The composition of the SP single-column eliminations of a step differs from the identity only in the
 // panel's columns, which is why steps 2 and 3 can apply it to all other columns at once.
+//
+// Steps 2 and 3 over the whole matrix for every SP columns would move 12 n^2 bytes per step.  So the
+// steps run inside blocks of kGjOb = 64 columns: within a block they touch the block's columns only,
+// and the rest of the matrix gets the block's 64 eliminations in one go.  For that the block's columns
+// are copied first (P0: their values when the block starts), a row map follows the row moves, and then,
+// with Pi = the block's 64 pivot rows in order and D = P0[Pi, :] (64 x 64),
+//     rows Pi      <-  R = D^-1 * (rows Pi of the rest)        (gj_block_rows_kernel; D = L U without
+//                                                               pivoting, the rows already are in pivot order)
+//     other rows r <-  row r - P0[r, :] * R                    (one product with 64 values of k)
+// which is what the four (or eight) steps would have done to the rest one after the other.
 
 constexpr int kGjThreads = 1024;
 constexpr int kGjMaxSp = 16;
@@ -718,15 +728,29 @@ __global__ __launch_bounds__(kGjThreads) void gj_panel_kernel(const float* __res
 
 // One thread per column col of [j, 2 np): rows move into place, pivot rows become D^-1 * (pivot rows)
 // (zero in the panel's own columns, whose entries in the other rows are the multipliers of step 3).
+// (columns [j, col_end) only; row_map[p] = the row, numbered as when the block of columns started, that
+// now sits at position p: the first thread takes it through the same moves)
 template <int SP>
-__global__ __launch_bounds__(256) void gj_rows_kernel(float* __restrict__ W, uint64_t ld, uint32_t np, uint32_t j,
-                                                      const GjStep* __restrict__ step) {
+__global__ __launch_bounds__(256) void gj_rows_kernel(float* __restrict__ W, uint64_t ld, uint32_t j, uint32_t col_end,
+                                                      const GjStep* __restrict__ step, int32_t* __restrict__ row_map) {
     __shared__ GjStep st;
     for (uint32_t i = threadIdx.x; i < sizeof(GjStep) / 4; i += 256)
         reinterpret_cast<uint32_t*>(&st)[i] = reinterpret_cast<const uint32_t*>(step)[i];
     __syncthreads();
+    if (row_map && blockIdx.x == 0 && threadIdx.x == 0) {
+        int32_t pv[SP], dv[SP];
+#pragma unroll
+        for (int c = 0; c < SP; ++c) pv[c] = row_map[st.piv[c]];
+#pragma unroll
+        for (int m = 0; m < SP; ++m) dv[m] = m < st.moves ? row_map[st.from[m]] : 0;
+#pragma unroll
+        for (int c = 0; c < SP; ++c) row_map[j + c] = pv[c];
+#pragma unroll
+        for (int m = 0; m < SP; ++m)
+            if (m < st.moves) row_map[st.to[m]] = dv[m];
+    }
     const uint64_t col = (uint64_t)j + (uint64_t)blockIdx.x * 256 + threadIdx.x;
-    if (col >= 2ull * np) return;
+    if (col >= col_end) return;
     float v[SP], d[SP];
 #pragma unroll
     for (int c = 0; c < SP; ++c) v[c] = W[(uint64_t)st.piv[c] * ld + col];
@@ -759,17 +783,214 @@ __global__ __launch_bounds__(256) void gj_copy_out_kernel(const float* __restric
     inv[i * ldi + c] = W[i * ld + np + c];
 }
 
+// ---- one block of kGjOb columns ----
+
+constexpr int kGjOb = 64;
+
+struct GjBlock {
+    int32_t moves;        // rows that leave the block's pivot positions for a position further down
+    int32_t pad[3];
+    int32_t to[kGjOb];    // where they go ...
+    int32_t from[kGjOb];  // ... and where they were when the block started
+    float lu[kGjOb * kGjOb];  // D = L U, packed: unit lower L below the diagonal, U on and above
+};
+
+// P0 = the block's columns as they are now; the row map starts as the identity
+__global__ __launch_bounds__(256) void gj_block_begin_kernel(const float* __restrict__ W, uint64_t ld, uint32_t np,
+                                                             uint32_t j0, float* __restrict__ P0,
+                                                             int32_t* __restrict__ row_map, GjBlock* __restrict__ blk) {
+    const uint64_t idx = (uint64_t)blockIdx.x * 256 + threadIdx.x;
+    if (idx == 0) blk->moves = 0;
+    if (idx >= (uint64_t)np * kGjOb) return;
+    const uint32_t r = (uint32_t)(idx / kGjOb), c = (uint32_t)(idx % kGjOb);
+    P0[idx] = W[(uint64_t)r * ld + j0 + c];
+    if (c == 0) row_map[r] = (int32_t)r;
+}
+
+// P1 = the multipliers of the block in the rows' final order: P1[p] = P0[row_map[p]], zero for the pivot
+// positions (they are replaced, not updated).  Rows below the block that changed place are listed in blk.
+__global__ __launch_bounds__(256) void gj_block_gather_kernel(const float* __restrict__ P0, float* __restrict__ P1,
+                                                              const int32_t* __restrict__ row_map, uint32_t np,
+                                                              uint32_t j0, GjBlock* __restrict__ blk) {
+    const uint64_t idx = (uint64_t)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= (uint64_t)np * kGjOb) return;
+    const uint32_t p = (uint32_t)(idx / kGjOb), c = (uint32_t)(idx % kGjOb);
+    const int32_t o = row_map[p];
+    const bool pivot_position = p >= j0 && p < j0 + kGjOb;
+    P1[idx] = pivot_position ? 0.0f : P0[(uint64_t)o * kGjOb + c];
+    if (c == 0 && !pivot_position && o != (int32_t)p) {
+        // at most kGjOb rows are displaced; their order in the list does not matter
+        const int32_t k = atomicAdd(&blk->moves, 1);
+        if (k < kGjOb) blk->to[k] = (int32_t)p, blk->from[k] = o;
+    }
+}
+
+// D = P0[the block's pivot rows, in order] = L U without pivoting.  One wave, lane r holds row r in
+// registers; the pivot row of a step reaches the other lanes through v_readlane (a scalar operand), so the
+// 63 steps need no barrier and no LDS.
+__global__ __launch_bounds__(64) void gj_block_lu_kernel(const float* __restrict__ P0,
+                                                         const int32_t* __restrict__ row_map, uint32_t j0,
+                                                         GjBlock* __restrict__ blk) {
+    static_assert(kGjOb == 64, "one row per lane");
+    const int lane = threadIdx.x;
+    const float4* src = reinterpret_cast<const float4*>(P0 + (uint64_t)row_map[j0 + lane] * kGjOb);
+    float d[kGjOb];
+#pragma unroll
+    for (int q4 = 0; q4 < kGjOb / 4; ++q4) {
+        const float4 t = src[q4];
+        d[4 * q4] = t.x, d[4 * q4 + 1] = t.y, d[4 * q4 + 2] = t.z, d[4 * q4 + 3] = t.w;
+    }
+    auto column = [&](auto k_const) __attribute__((always_inline)) {
+        constexpr int k = decltype(k_const)::value;
+        // multipliers by the reciprocal of the pivot, as in the panels
+        const float rpivot = 1.0f / __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, d[k]), k));
+        const bool below = lane > k;
+        const float l = below ? d[k] * rpivot : 0.0f;
+        if (below) d[k] = l;
+#pragma unroll
+        for (int q = k + 1; q < kGjOb; ++q) {
+            const float u = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, d[q]), k));
+            d[q] = fmaf(-l, u, d[q]);  // l = 0 in the rows above: unchanged
+        }
+    };
+    gj_for_each(column, std::make_integer_sequence<int, kGjOb - 1>{});
+    float4* dst = reinterpret_cast<float4*>(blk->lu + lane * kGjOb);
+#pragma unroll
+    for (int q4 = 0; q4 < kGjOb / 4; ++q4) dst[q4] = make_float4(d[4 * q4], d[4 * q4 + 1], d[4 * q4 + 2], d[4 * q4 + 3]);
+}
+
+// One thread per column of the rest (col >= j0 + kGjOb): the pivot rows, fetched from where they were when
+// the block started, become R = U^-1 L^-1 (pivot rows) at the block's positions; displaced rows move.
+// The column's 64 values live in LDS (one column of v per thread) and are worked on eight at a time in
+// registers; the factors are read with wave-uniform addresses.
+__global__ __launch_bounds__(256) void gj_block_rows_kernel(float* __restrict__ W, uint64_t ld, uint32_t np, uint32_t j0,
+                                                            const int32_t* __restrict__ row_map,
+                                                            const GjBlock* __restrict__ blk) {
+    constexpr int T = 8, NB8 = kGjOb / T;
+    __shared__ float v[kGjOb][256];
+    const float* __restrict__ lu = blk->lu;
+    const int tid = threadIdx.x;
+    const int moves = blk->moves < kGjOb ? blk->moves : kGjOb;
+    const uint64_t col = (uint64_t)j0 + kGjOb + (uint64_t)blockIdx.x * 256 + tid;
+    if (col >= 2ull * np) return;  // (no barrier below: a thread only reads the column of v that it wrote)
+    float d[kGjOb];
+#pragma unroll
+    for (int m = 0; m < kGjOb; ++m) d[m] = m < moves ? W[(uint64_t)blk->from[m] * ld + col] : 0.0f;
+#pragma unroll 8
+    for (int c = 0; c < kGjOb; ++c) v[c][tid] = W[(uint64_t)row_map[j0 + c] * ld + col];
+    // forward substitution with the unit lower factor, block row by block row
+    for (int rb = 0; rb < NB8; ++rb) {
+        float x[T];
+#pragma unroll
+        for (int i = 0; i < T; ++i) x[i] = v[rb * T + i][tid];
+        for (int cb = 0; cb < rb; ++cb) {
+            float y[T];
+#pragma unroll
+            for (int q = 0; q < T; ++q) y[q] = v[cb * T + q][tid];
+            const float* l = lu + (rb * T) * kGjOb + cb * T;
+#pragma unroll
+            for (int i = 0; i < T; ++i)
+#pragma unroll
+                for (int q = 0; q < T; ++q) x[i] = fmaf(-l[i * kGjOb + q], y[q], x[i]);
+        }
+        const float* l = lu + (rb * T) * kGjOb + rb * T;
+#pragma unroll
+        for (int i = 1; i < T; ++i)
+#pragma unroll
+            for (int q = 0; q < i; ++q) x[i] = fmaf(-l[i * kGjOb + q], x[q], x[i]);
+#pragma unroll
+        for (int i = 0; i < T; ++i) v[rb * T + i][tid] = x[i];
+    }
+    // back substitution with the upper factor
+    for (int rb = NB8 - 1; rb >= 0; --rb) {
+        float x[T];
+#pragma unroll
+        for (int i = 0; i < T; ++i) x[i] = v[rb * T + i][tid];
+        for (int cb = rb + 1; cb < NB8; ++cb) {
+            float y[T];
+#pragma unroll
+            for (int q = 0; q < T; ++q) y[q] = v[cb * T + q][tid];
+            const float* u = lu + (rb * T) * kGjOb + cb * T;
+#pragma unroll
+            for (int i = 0; i < T; ++i)
+#pragma unroll
+                for (int q = 0; q < T; ++q) x[i] = fmaf(-u[i * kGjOb + q], y[q], x[i]);
+        }
+        const float* u = lu + (rb * T) * kGjOb + rb * T;
+#pragma unroll
+        for (int i = T - 1; i >= 0; --i) {
+#pragma unroll
+            for (int q = i + 1; q < T; ++q) x[i] = fmaf(-u[i * kGjOb + q], x[q], x[i]);
+            x[i] = x[i] / u[i * kGjOb + i];
+        }
+#pragma unroll
+        for (int i = 0; i < T; ++i) v[rb * T + i][tid] = x[i];
+    }
+#pragma unroll 8
+    for (int c = 0; c < kGjOb; ++c) W[(uint64_t)(j0 + c) * ld + col] = v[c][tid];
+#pragma unroll
+    for (int m = 0; m < kGjOb; ++m)
+        if (m < moves) W[(uint64_t)blk->to[m] * ld + col] = d[m];
+}
+
+// Every step applied to the whole matrix at once: fewer launches per column, 12 n^2 bytes per step.  The
+// faster way for small matrices, where a step's launches cost more than its memory traffic.
 template <int SP, int RPT>
-int gj_run(float* W, uint32_t np, GjStep* steps, int32_t* status, hipStream_t s) {
+int gj_run_flat(float* W, uint32_t np, GjStep* steps, int32_t* status, hipStream_t s) {
     const uint64_t ld = 2ull * np;
     for (uint32_t j = 0; j < np; j += SP) {
         GjStep* st = steps + (j / SP) % 2;  // two records in turn: the next panel never overwrites one still in use
         hipLaunchKernelGGL((gj_panel_kernel<SP, RPT>), dim3(1), dim3(kGjThreads), 0, s, W, ld, np, j, st, status);
         const uint32_t cols = 2 * np - j;
-        hipLaunchKernelGGL((gj_rows_kernel<SP>), dim3((cols + 255) / 256), dim3(256), 0, s, W, ld, np, j, st);
+        hipLaunchKernelGGL((gj_rows_kernel<SP>), dim3((cols + 255) / 256), dim3(256), 0, s, W, ld, j, 2 * np, st,
+                           (int32_t*)nullptr);
         if (hipGetLastError() != hipSuccess) return TRAKHIP_ERR_LAUNCH;
         const int e = trakhip::gemm_nn(W + j, ld, W + (uint64_t)j * ld + j + SP, ld, W + j + SP, ld, np,
                                        2ull * np - j - SP, SP, -1.0f, 1.0f, s, 0);
+        if (e) return e;
+    }
+    return TRAKHIP_OK;
+}
+
+struct GjBuffers {
+    float* W;           // np x 2 np
+    float* P0;          // np x kGjOb
+    float* P1;          // np x kGjOb
+    int32_t* row_map;   // np
+    GjBlock* blk;
+    GjStep* steps;      // kGjOb / 8 records
+};
+
+template <int SP, int RPT>
+int gj_run(const GjBuffers& b, uint32_t np, int32_t* status, hipStream_t s) {
+    const uint64_t ld = 2ull * np;
+    float* W = b.W;
+    const uint32_t panel_blocks = (uint32_t)(((uint64_t)np * kGjOb + 255) / 256);
+    for (uint32_t j0 = 0; j0 < np; j0 += kGjOb) {
+        hipLaunchKernelGGL(gj_block_begin_kernel, dim3(panel_blocks), dim3(256), 0, s, W, ld, np, j0, b.P0, b.row_map,
+                           b.blk);
+        const uint32_t block_end = j0 + kGjOb;
+        for (uint32_t j = j0; j < block_end; j += SP) {
+            GjStep* st = b.steps + (j - j0) / SP;
+            hipLaunchKernelGGL((gj_panel_kernel<SP, RPT>), dim3(1), dim3(kGjThreads), 0, s, W, ld, np, j, st, status);
+            hipLaunchKernelGGL((gj_rows_kernel<SP>), dim3((block_end - j + 255) / 256), dim3(256), 0, s, W, ld, j,
+                               block_end, st, b.row_map);
+            if (hipGetLastError() != hipSuccess) return TRAKHIP_ERR_LAUNCH;
+            if (j + SP < block_end) {
+                const int e = trakhip::gemm_nn(W + j, ld, W + (uint64_t)j * ld + j + SP, ld, W + j + SP, ld, np,
+                                               block_end - j - SP, SP, -1.0f, 1.0f, s, 0);
+                if (e) return e;
+            }
+        }
+        hipLaunchKernelGGL(gj_block_gather_kernel, dim3(panel_blocks), dim3(256), 0, s, b.P0, b.P1, b.row_map, np, j0,
+                           b.blk);
+        hipLaunchKernelGGL(gj_block_lu_kernel, dim3(1), dim3(64), 0, s, b.P0, b.row_map, j0, b.blk);
+        const uint32_t rest = 2 * np - block_end;
+        hipLaunchKernelGGL(gj_block_rows_kernel, dim3((rest + 255) / 256), dim3(256), 0, s, W, ld, np, j0, b.row_map,
+                           b.blk);
+        if (hipGetLastError() != hipSuccess) return TRAKHIP_ERR_LAUNCH;
+        const int e = trakhip::gemm_nn(b.P1, kGjOb, W + (uint64_t)j0 * ld + block_end, ld, W + block_end, ld, np, rest,
+                                       kGjOb, -1.0f, 1.0f, s, 0);
         if (e) return e;
     }
     return TRAKHIP_OK;
@@ -784,7 +1005,8 @@ constexpr uint64_t kGeneralInverseMaxN = 12288;
 size_t general_inverse_workspace_bytes(uint64_t n) {
     if (n == 0 || n > kGeneralInverseMaxN) return 0;
     const uint64_t np = (n + NB - 1) / NB * NB;
-    return (size_t)(2 * np * np + kSumBlocks + 4) * sizeof(float) + 2 * sizeof(GjStep);
+    return (size_t)(2 * np * np + 2 * np * kGjOb + np + kSumBlocks + 4) * sizeof(float) + sizeof(GjBlock) +
+           (kGjOb / 8) * sizeof(GjStep);
 }
 
 int general_inverse(const float* A, uint64_t lda, float lambda, float* inv, uint64_t ldi, uint64_t n, int normalize,
@@ -796,15 +1018,24 @@ int general_inverse(const float* A, uint64_t lda, float lambda, float* inv, uint
     if (reinterpret_cast<uintptr_t>(ws) % 16) return TRAKHIP_ERR_ALIGN;
     const uint64_t np = (n + NB - 1) / NB * NB;
     float* W = static_cast<float*>(ws);
-    float* partial = W + 2 * np * np;
+    GjBuffers b;
+    b.W = W;
+    b.P0 = W + 2 * np * np;
+    b.P1 = b.P0 + np * kGjOb;
+    b.row_map = reinterpret_cast<int32_t*>(b.P1 + np * kGjOb);
+    float* partial = reinterpret_cast<float*>(b.row_map + np);
     float* mean_dev = partial + kSumBlocks;
-    GjStep* steps = reinterpret_cast<GjStep*>(mean_dev + 4);
+    b.blk = reinterpret_cast<GjBlock*>(mean_dev + 4);
+    b.steps = reinterpret_cast<GjStep*>(b.blk + 1);
     hipLaunchKernelGGL(gj_init_kernel, dim3((uint32_t)((2 * np * np + 255) / 256)), dim3(256), 0, s, A, lda, lambda, n,
                        np, W, status);
     if (hipGetLastError() != hipSuccess) return TRAKHIP_ERR_LAUNCH;
     // the panel's rows live in the registers of one workgroup: 16 columns of up to 6144 rows, or 8 of up to 12288
-    const int e = np <= 6144 ? gj_run<16, 6>(W, (uint32_t)np, steps, status, s)
-                             : gj_run<8, 12>(W, (uint32_t)np, steps, status, s);
+    // (measured: whole-matrix steps 1.8 / 3.5 / 7.9 / 16.2 ms at n = 512 / 1024 / 2048 / 3072, blocks of 64 columns
+    // 2.2 / 4.4 / 9.2 / 15.5 ms)
+    const int e = np < 3072      ? gj_run_flat<16, 6>(W, (uint32_t)np, b.steps, status, s)
+                  : np <= 6144   ? gj_run<16, 6>(b, (uint32_t)np, status, s)
+                                 : gj_run<8, 12>(b, (uint32_t)np, status, s);
     if (e) return e;
     hipLaunchKernelGGL(gj_copy_out_kernel, dim3((uint32_t)((n * n + 255) / 256)), dim3(256), 0, s, W, 2 * np, np, n, inv,
                        ldi);
