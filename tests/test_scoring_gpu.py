@@ -266,13 +266,13 @@ def test_general_inverse_in_column_blocks_needs_its_pivoting(gpu):
     b = torch.randn(n, n, generator=gen)
     b[:700] *= 1e-3
     got, _ = general_inverse(b.to(gpu))
-    # condition number about 1e7: measured against what LU with the same pivoting makes of it in fp32
-    ref = torch.linalg.inv(b.to(gpu)).double()
-    b64 = b.double().to(gpu)
-    want = torch.linalg.inv(b64)
-    eye = torch.eye(n, device=gpu, dtype=torch.float64)
-    err, ref_err = (float((m - want).abs().max() / want.abs().max()) for m in (got.double(), ref))
-    resid, ref_resid = (float((b64 @ m - eye).abs().max()) for m in (got.double(), ref))
+    # condition number about 1e7: measured against what LAPACK's LU with the same pivoting makes of it in fp32
+    b64 = b.double().numpy()
+    want = np.linalg.inv(b64)
+    ref = torch.linalg.inv(b).double().numpy()      # (on the CPU; numpy's inverse of an fp32 matrix computes in double)
+    g64 = got.cpu().numpy().astype(np.float64)
+    err, ref_err = (float(np.abs(m - want).max() / np.abs(want).max()) for m in (g64, ref))
+    resid, ref_resid = (float(np.abs(b64 @ m - np.eye(n)).max()) for m in (g64, ref))
     assert err <= 4 * ref_err + 1e-5 and resid <= 2 * ref_resid + 1e-3, (err, ref_err, resid, ref_resid)
     # a zero column in the last panel of a block
     c = torch.randn(n, n, generator=gen)
@@ -295,7 +295,7 @@ def test_general_inverse_of_an_indefinite_gram_matrix_at_proj_dim_4096(gpu):
     inv, mean_abs = general_inverse(gram, normalize=True)
     assert torch.isfinite(inv).all()
     resid = (gram.double() @ (inv.double() * mean_abs.double()) - torch.eye(k, device=gpu, dtype=torch.float64)).abs().max()
-    ref = torch.linalg.inv(gram)                    # LU with the same pivoting, for the size of the residual
+    ref = torch.linalg.inv(gram.cpu()).to(gpu)      # LAPACK's LU in fp32 on the CPU, same pivoting: the size of the residual
     ref_resid = (gram.double() @ ref.double() - torch.eye(k, device=gpu, dtype=torch.float64)).abs().max()
     assert float(resid) < max(1e-2, 20 * float(ref_resid)), (float(resid), float(ref_resid))
 
