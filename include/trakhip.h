@@ -268,8 +268,8 @@ int trakhip_spd_inverse(const float* A_dev, uint64_t lda, float lambda, float* i
                         uint64_t n, int normalize, float* mean_abs_dev, int32_t* status_dev,
                         void* workspace_dev, size_t workspace_bytes, void* stream);
 
-/* The same result for ANY nonsingular fp32 matrix A + lambda * I, by Gauss-Jordan elimination with partial
- * (row) pivoting on the device: the route for a matrix that trakhip_spd_inverse reports as not positive
+/* The same result for ANY nonsingular fp32 matrix A + lambda * I, by elimination with partial (row)
+ * pivoting on the device: the route for a matrix that trakhip_spd_inverse reports as not positive
  * definite (status != 0) - a Gram matrix rounded to fp16, or one of deficient rank with lambda = 0, is
  * symmetric but need not be positive definite, and the reference inverts every matrix with LU and partial
  * pivoting (torch.linalg.inv, trak/score_computers.py:163).  n <= 12288 (TRAKHIP_ERR_SHAPE beyond, and

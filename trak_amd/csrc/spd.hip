@@ -542,34 +542,36 @@ int spd_inverse(const float* A, uint64_t lda, float lambda, float* inv, uint64_t
 
 namespace {
 
-// ---- inverse of a general matrix: Gauss-Jordan elimination with partial pivoting ---------------------------
+// ---- inverse of a general matrix: elimination with partial pivoting -----------------------------------------
 //
 // For the matrices the Cholesky route above refuses: a Gram matrix rounded to fp16, or one of deficient
 // rank with lambda = 0, is symmetric but need not be positive definite.  The reference inverts every
 // matrix with LU and partial pivoting (torch.linalg.inv, trak/score_computers.py:163); this is the same
 // pivoting on the device.  The augmented matrix [A + lambda I | I] (np x 2 np, np = n padded with an
-// identity block to a multiple of 128) is reduced to [I | A^-1], SP columns per step:
-//   1. gj_panel_kernel: ONE workgroup holds rows j.. of the SP panel columns in registers and eliminates
-//      them column by column with row pivoting (largest magnitude, lowest row on ties; rows are not
-//      moved, a row is marked once it has been a pivot).  It leaves the pivot rows' numbers, where the
-//      rows they displace go, and the factors L U of the SP x SP pivot block D;
-//   2. gj_rows_kernel: one thread per column of the rest of the matrix moves the rows into place and
-//      replaces the pivot rows by R = D^-1 * (pivot rows), solved with the two triangular factors (an
-//      explicit D^-1 would lose what the condition of D costs);
-//   3. every other row r gets  W[r, rest] -= W[r, panel] * R  (the fp32 MFMA product; the pivot rows'
-//      panel entries were set to zero, so they pass through unchanged).
-// The composition of the SP single-column eliminations of a step differs from the identity only in the
-// panel's columns, which is why steps 2 and 3 can apply it to all other columns at once.
+// identity block to a multiple of 128) is reduced to [I | A^-1] block of columns by block of columns.
+// For a block J of OB columns starting at j0 (the rows above j0 are finished pivot rows of earlier blocks):
+//   1. the block's columns are factored as in a right-looking LU, SP columns at a time: gj_panel_kernel
+//      (ONE workgroup holds rows j.. of the SP panel columns in registers) eliminates them column by column
+//      with row pivoting (largest magnitude, lowest row on ties), leaves the multipliers (|l| <= 1) in the
+//      rows below, the pivot rows' numbers, where the rows they displace go, and the packed factors of the
+//      SP x SP pivot block; gj_rows_kernel moves the rows of the block's columns into place and turns the
+//      pivot rows right of the panel into L11^-1 * (pivot rows); a product with SP values of k updates the
+//      block's columns further right in the rows below.  Afterwards rows j0.. of J hold L \ U of the block.
+//   2. the rest of the matrix (all columns right of the block, the identity half included) gets the block's
+//      OB eliminations at once: gj_block_rows_kernel (one thread per column) applies the row moves, computes
+//      Y = L_J^-1 * (pivot rows) (kept aside) and R = U_J^-1 * Y, which replaces the pivot rows;
+//          rows below the block:  W[r, rest] -= L[r, J] * Y        (the LU update, multipliers at most 1)
+//          rows above the block:  W[r, rest] -= W[r, J] * R        (the Gauss-Jordan part: back substitution
+//                                                                   folded into the elimination)
+//      two products with OB values of k.  No permutation is left to undo at the end: the row moves act on
+//      whole rows of [A | I].
+// OB = 64 from np = 3072 on (four or eight panels per block: the products over the rest move 12 np^2 bytes per
+// block instead of per panel); below that OB = SP = 16 (fewer launches per column, which is what small
+// matrices pay for).
 //
-// Steps 2 and 3 over the whole matrix for every SP columns would move 12 n^2 bytes per step.  So the
-// steps run inside blocks of kGjOb = 64 columns: within a block they touch the block's columns only,
-// and the rest of the matrix gets the block's 64 eliminations in one go.  For that the block's columns
-// are copied first (P0: their values when the block starts), a row map follows the row moves, and then,
-// with Pi = the block's 64 pivot rows in order and D = P0[Pi, :] (64 x 64),
-//     rows Pi      <-  R = D^-1 * (rows Pi of the rest)        (gj_block_rows_kernel; D = L U without
-//                                                               pivoting, the rows already are in pivot order)
-//     other rows r <-  row r - P0[r, :] * R                    (one product with 64 values of k)
-// which is what the four (or eight) steps would have done to the rest one after the other.
+// (An earlier form updated every row with the panel's original entries times D^-1 * (pivot rows), D the pivot
+// block: one product for all rows, but rounding errors of the size of cond(D) instead of the multipliers'
+// |l| <= 1 - up to 30 times the error of LAPACK's LU on matrices of condition 1e5..1e7.)
 
 constexpr int kGjThreads = 1024;
 constexpr int kGjMaxSp = 16;
@@ -614,7 +616,7 @@ __device__ __forceinline__ void gj_for_each(F& f, std::integer_sequence<int, S..
 }
 
 template <int SP, int RPT>
-__global__ __launch_bounds__(kGjThreads) void gj_panel_kernel(const float* __restrict__ W, uint64_t ld, uint32_t np,
+__global__ __launch_bounds__(kGjThreads) void gj_panel_kernel(float* __restrict__ W, uint64_t ld, uint32_t np,
                                                               uint32_t j, GjStep* __restrict__ step,
                                                               int32_t* __restrict__ status) {
     __shared__ uint32_t cand_key[kGjThreads / 64], cand_row[kGjThreads / 64];
@@ -697,6 +699,17 @@ __global__ __launch_bounds__(kGjThreads) void gj_panel_kernel(const float* __res
         }
     };
     gj_for_each(column, std::make_integer_sequence<int, SP>{});
+    // the rows that were never pivots now hold their SP multipliers: back to the matrix, where the row moves and
+    // the update of the other columns find them
+#pragma unroll
+    for (int i = 0; i < RPT; ++i) {
+        if (i < slots && (live & (1u << i))) {
+            float4* dst = reinterpret_cast<float4*>(W + (uint64_t)(j + (uint32_t)tid + (uint32_t)kGjThreads * i) * ld + j);
+#pragma unroll
+            for (int c4 = 0; c4 < SP / 4; ++c4)
+                dst[c4] = make_float4(a[i][4 * c4], a[i][4 * c4 + 1], a[i][4 * c4 + 2], a[i][4 * c4 + 3]);
+        }
+    }
     // D = (rows piv[0..SP) of the panel as they were) = L U with the packed factors in lu
     if (tid < SP) {
 #pragma unroll
@@ -726,50 +739,49 @@ __global__ __launch_bounds__(kGjThreads) void gj_panel_kernel(const float* __res
     }
 }
 
-// One thread per column col of [j, 2 np): rows move into place, pivot rows become D^-1 * (pivot rows)
-// (zero in the panel's own columns, whose entries in the other rows are the multipliers of step 3).
-// (columns [j, col_end) only; row_map[p] = the row, numbered as when the block of columns started, that
-// now sits at position p: the first thread takes it through the same moves)
+// One thread per column of [col_begin, col_end): the rows move into place (pivot rows to j.., the rows they
+// displace to the vacated positions).  Left of the panel that is all (multipliers of earlier panels travel with
+// their rows); in the panel's columns the pivot rows become the packed factors; right of it they become
+// Y = L^-1 * (pivot rows).  With y_out (the one-panel blocks of small matrices, where "right of the panel" is the
+// whole rest) Y goes to y_out[c * ld + col] and the pivot rows become R = U^-1 * Y.
 template <int SP>
-__global__ __launch_bounds__(256) void gj_rows_kernel(float* __restrict__ W, uint64_t ld, uint32_t j, uint32_t col_end,
-                                                      const GjStep* __restrict__ step, int32_t* __restrict__ row_map) {
+__global__ __launch_bounds__(256) void gj_rows_kernel(float* __restrict__ W, uint64_t ld, uint32_t j, uint32_t col_begin,
+                                                      uint32_t col_end, const GjStep* __restrict__ step,
+                                                      float* __restrict__ y_out) {
     __shared__ GjStep st;
     for (uint32_t i = threadIdx.x; i < sizeof(GjStep) / 4; i += 256)
         reinterpret_cast<uint32_t*>(&st)[i] = reinterpret_cast<const uint32_t*>(step)[i];
     __syncthreads();
-    if (row_map && blockIdx.x == 0 && threadIdx.x == 0) {
-        int32_t pv[SP], dv[SP];
-#pragma unroll
-        for (int c = 0; c < SP; ++c) pv[c] = row_map[st.piv[c]];
-#pragma unroll
-        for (int m = 0; m < SP; ++m) dv[m] = m < st.moves ? row_map[st.from[m]] : 0;
-#pragma unroll
-        for (int c = 0; c < SP; ++c) row_map[j + c] = pv[c];
-#pragma unroll
-        for (int m = 0; m < SP; ++m)
-            if (m < st.moves) row_map[st.to[m]] = dv[m];
-    }
-    const uint64_t col = (uint64_t)j + (uint64_t)blockIdx.x * 256 + threadIdx.x;
+    const uint64_t col = (uint64_t)col_begin + (uint64_t)blockIdx.x * 256 + threadIdx.x;
     if (col >= col_end) return;
     float v[SP], d[SP];
 #pragma unroll
     for (int c = 0; c < SP; ++c) v[c] = W[(uint64_t)st.piv[c] * ld + col];
 #pragma unroll
     for (int m = 0; m < SP; ++m) d[m] = m < st.moves ? W[(uint64_t)st.from[m] * ld + col] : 0.0f;
-    const bool in_panel = col < (uint64_t)j + SP;
-    // R = U^-1 (L^-1 v): forward substitution with the unit lower factor, back substitution with the upper one
+    if (col >= j && col < (uint64_t)j + SP) {
 #pragma unroll
-    for (int r = 1; r < SP; ++r)
+        for (int c = 0; c < SP; ++c) v[c] = st.lu[c * SP + (int)(col - j)];
+    } else if (col >= (uint64_t)j + SP) {
+        // forward substitution with the unit lower factor
 #pragma unroll
-        for (int q = 0; q < r; ++q) v[r] = fmaf(-st.lu[r * SP + q], v[q], v[r]);
+        for (int r = 1; r < SP; ++r)
 #pragma unroll
-    for (int r = SP - 1; r >= 0; --r) {
+            for (int q = 0; q < r; ++q) v[r] = fmaf(-st.lu[r * SP + q], v[q], v[r]);
+        if (y_out) {
 #pragma unroll
-        for (int q = r + 1; q < SP; ++q) v[r] = fmaf(-st.lu[r * SP + q], v[q], v[r]);
-        v[r] = v[r] / st.lu[r * SP + r];
+            for (int c = 0; c < SP; ++c) y_out[(uint64_t)c * ld + col] = v[c];
+            // back substitution with the upper one
+#pragma unroll
+            for (int r = SP - 1; r >= 0; --r) {
+#pragma unroll
+                for (int q = r + 1; q < SP; ++q) v[r] = fmaf(-st.lu[r * SP + q], v[q], v[r]);
+                v[r] = v[r] / st.lu[r * SP + r];
+            }
+        }
     }
 #pragma unroll
-    for (int c = 0; c < SP; ++c) W[(uint64_t)(j + c) * ld + col] = in_panel ? 0.0f : v[c];
+    for (int c = 0; c < SP; ++c) W[(uint64_t)(j + c) * ld + col] = v[c];
 #pragma unroll
     for (int m = 0; m < SP; ++m)
         if (m < st.moves) W[(uint64_t)st.to[m] * ld + col] = d[m];
@@ -783,101 +795,36 @@ __global__ __launch_bounds__(256) void gj_copy_out_kernel(const float* __restric
     inv[i * ldi + c] = W[i * ld + np + c];
 }
 
-// ---- one block of kGjOb columns ----
+constexpr int kGjOb = 64;  // columns of a block of the large-matrix route
 
-constexpr int kGjOb = 64;
-
-struct GjBlock {
-    int32_t moves;        // rows that leave the block's pivot positions for a position further down
-    int32_t pad[3];
-    int32_t to[kGjOb];    // where they go ...
-    int32_t from[kGjOb];  // ... and where they were when the block started
-    float lu[kGjOb * kGjOb];  // D = L U, packed: unit lower L below the diagonal, U on and above
-};
-
-// P0 = the block's columns as they are now; the row map starts as the identity
-__global__ __launch_bounds__(256) void gj_block_begin_kernel(const float* __restrict__ W, uint64_t ld, uint32_t np,
-                                                             uint32_t j0, float* __restrict__ P0,
-                                                             int32_t* __restrict__ row_map, GjBlock* __restrict__ blk) {
-    const uint64_t idx = (uint64_t)blockIdx.x * 256 + threadIdx.x;
-    if (idx == 0) blk->moves = 0;
-    if (idx >= (uint64_t)np * kGjOb) return;
-    const uint32_t r = (uint32_t)(idx / kGjOb), c = (uint32_t)(idx % kGjOb);
-    P0[idx] = W[(uint64_t)r * ld + j0 + c];
-    if (c == 0) row_map[r] = (int32_t)r;
-}
-
-// P1 = the multipliers of the block in the rows' final order: P1[p] = P0[row_map[p]], zero for the pivot
-// positions (they are replaced, not updated).  Rows below the block that changed place are listed in blk.
-__global__ __launch_bounds__(256) void gj_block_gather_kernel(const float* __restrict__ P0, float* __restrict__ P1,
-                                                              const int32_t* __restrict__ row_map, uint32_t np,
-                                                              uint32_t j0, GjBlock* __restrict__ blk) {
-    const uint64_t idx = (uint64_t)blockIdx.x * 256 + threadIdx.x;
-    if (idx >= (uint64_t)np * kGjOb) return;
-    const uint32_t p = (uint32_t)(idx / kGjOb), c = (uint32_t)(idx % kGjOb);
-    const int32_t o = row_map[p];
-    const bool pivot_position = p >= j0 && p < j0 + kGjOb;
-    P1[idx] = pivot_position ? 0.0f : P0[(uint64_t)o * kGjOb + c];
-    if (c == 0 && !pivot_position && o != (int32_t)p) {
-        // at most kGjOb rows are displaced; their order in the list does not matter
-        const int32_t k = atomicAdd(&blk->moves, 1);
-        if (k < kGjOb) blk->to[k] = (int32_t)p, blk->from[k] = o;
-    }
-}
-
-// D = P0[the block's pivot rows, in order] = L U without pivoting.  One wave, lane r holds row r in
-// registers; the pivot row of a step reaches the other lanes through v_readlane (a scalar operand), so the
-// 63 steps need no barrier and no LDS.
-__global__ __launch_bounds__(64) void gj_block_lu_kernel(const float* __restrict__ P0,
-                                                         const int32_t* __restrict__ row_map, uint32_t j0,
-                                                         GjBlock* __restrict__ blk) {
-    static_assert(kGjOb == 64, "one row per lane");
-    const int lane = threadIdx.x;
-    const float4* src = reinterpret_cast<const float4*>(P0 + (uint64_t)row_map[j0 + lane] * kGjOb);
-    float d[kGjOb];
-#pragma unroll
-    for (int q4 = 0; q4 < kGjOb / 4; ++q4) {
-        const float4 t = src[q4];
-        d[4 * q4] = t.x, d[4 * q4 + 1] = t.y, d[4 * q4 + 2] = t.z, d[4 * q4 + 3] = t.w;
-    }
-    auto column = [&](auto k_const) __attribute__((always_inline)) {
-        constexpr int k = decltype(k_const)::value;
-        // multipliers by the reciprocal of the pivot, as in the panels
-        const float rpivot = 1.0f / __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, d[k]), k));
-        const bool below = lane > k;
-        const float l = below ? d[k] * rpivot : 0.0f;
-        if (below) d[k] = l;
-#pragma unroll
-        for (int q = k + 1; q < kGjOb; ++q) {
-            const float u = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, d[q]), k));
-            d[q] = fmaf(-l, u, d[q]);  // l = 0 in the rows above: unchanged
-        }
-    };
-    gj_for_each(column, std::make_integer_sequence<int, kGjOb - 1>{});
-    float4* dst = reinterpret_cast<float4*>(blk->lu + lane * kGjOb);
-#pragma unroll
-    for (int q4 = 0; q4 < kGjOb / 4; ++q4) dst[q4] = make_float4(d[4 * q4], d[4 * q4 + 1], d[4 * q4 + 2], d[4 * q4 + 3]);
-}
-
-// One thread per column of the rest (col >= j0 + kGjOb): the pivot rows, fetched from where they were when
-// the block started, become R = U^-1 L^-1 (pivot rows) at the block's positions; displaced rows move.
-// The column's 64 values live in LDS (one column of v per thread) and are worked on eight at a time in
-// registers; the factors are read with wave-uniform addresses.
+// One thread per column of the rest (col >= j0 + kGjOb).  The block's panels' row moves are applied one panel
+// after the other (the pivot rows collect in LDS, one column of v per thread); then, with the factors L \ U that
+// rows j0.. of the block's columns hold (F, read with wave-uniform addresses), Y = L^-1 v goes to
+// y_out[c * ld + col] and R = U^-1 Y to rows j0.. of the column.  The 64 values are worked on eight at a time.
+template <int SP>
 __global__ __launch_bounds__(256) void gj_block_rows_kernel(float* __restrict__ W, uint64_t ld, uint32_t np, uint32_t j0,
-                                                            const int32_t* __restrict__ row_map,
-                                                            const GjBlock* __restrict__ blk) {
-    constexpr int T = 8, NB8 = kGjOb / T;
+                                                            const float* __restrict__ F,
+                                                            const GjStep* __restrict__ steps, float* __restrict__ y_out) {
+    constexpr int T = 8, NB8 = kGjOb / T, PANELS = kGjOb / SP;
     __shared__ float v[kGjOb][256];
-    const float* __restrict__ lu = blk->lu;
     const int tid = threadIdx.x;
-    const int moves = blk->moves < kGjOb ? blk->moves : kGjOb;
     const uint64_t col = (uint64_t)j0 + kGjOb + (uint64_t)blockIdx.x * 256 + tid;
     if (col >= 2ull * np) return;  // (no barrier below: a thread only reads the column of v that it wrote)
-    float d[kGjOb];
+    for (int p = 0; p < PANELS; ++p) {
+        const GjStep* st = steps + p;
+        const int moves = st->moves;
+        float x[SP], d[SP];
 #pragma unroll
-    for (int m = 0; m < kGjOb; ++m) d[m] = m < moves ? W[(uint64_t)blk->from[m] * ld + col] : 0.0f;
-#pragma unroll 8
-    for (int c = 0; c < kGjOb; ++c) v[c][tid] = W[(uint64_t)row_map[j0 + c] * ld + col];
+        for (int c = 0; c < SP; ++c) x[c] = W[(uint64_t)st->piv[c] * ld + col];
+#pragma unroll
+        for (int m = 0; m < SP; ++m) d[m] = m < moves ? W[(uint64_t)st->from[m] * ld + col] : 0.0f;
+#pragma unroll
+        for (int c = 0; c < SP; ++c) v[p * SP + c][tid] = x[c];
+        // (a position j0 + p SP + c is never a source of a later panel: those take rows from further down)
+#pragma unroll
+        for (int m = 0; m < SP; ++m)
+            if (m < moves) W[(uint64_t)st->to[m] * ld + col] = d[m];
+    }
     // forward substitution with the unit lower factor, block row by block row
     for (int rb = 0; rb < NB8; ++rb) {
         float x[T];
@@ -887,19 +834,22 @@ __global__ __launch_bounds__(256) void gj_block_rows_kernel(float* __restrict__ 
             float y[T];
 #pragma unroll
             for (int q = 0; q < T; ++q) y[q] = v[cb * T + q][tid];
-            const float* l = lu + (rb * T) * kGjOb + cb * T;
+            const float* l = F + (uint64_t)(rb * T) * ld + cb * T;
 #pragma unroll
             for (int i = 0; i < T; ++i)
 #pragma unroll
-                for (int q = 0; q < T; ++q) x[i] = fmaf(-l[i * kGjOb + q], y[q], x[i]);
+                for (int q = 0; q < T; ++q) x[i] = fmaf(-l[(uint64_t)i * ld + q], y[q], x[i]);
         }
-        const float* l = lu + (rb * T) * kGjOb + rb * T;
+        const float* l = F + (uint64_t)(rb * T) * ld + rb * T;
 #pragma unroll
         for (int i = 1; i < T; ++i)
 #pragma unroll
-            for (int q = 0; q < i; ++q) x[i] = fmaf(-l[i * kGjOb + q], x[q], x[i]);
+            for (int q = 0; q < i; ++q) x[i] = fmaf(-l[(uint64_t)i * ld + q], x[q], x[i]);
 #pragma unroll
-        for (int i = 0; i < T; ++i) v[rb * T + i][tid] = x[i];
+        for (int i = 0; i < T; ++i) {
+            v[rb * T + i][tid] = x[i];
+            y_out[(uint64_t)(rb * T + i) * ld + col] = x[i];
+        }
     }
     // back substitution with the upper factor
     for (int rb = NB8 - 1; rb >= 0; --rb) {
@@ -910,87 +860,84 @@ __global__ __launch_bounds__(256) void gj_block_rows_kernel(float* __restrict__ 
             float y[T];
 #pragma unroll
             for (int q = 0; q < T; ++q) y[q] = v[cb * T + q][tid];
-            const float* u = lu + (rb * T) * kGjOb + cb * T;
+            const float* u = F + (uint64_t)(rb * T) * ld + cb * T;
 #pragma unroll
             for (int i = 0; i < T; ++i)
 #pragma unroll
-                for (int q = 0; q < T; ++q) x[i] = fmaf(-u[i * kGjOb + q], y[q], x[i]);
+                for (int q = 0; q < T; ++q) x[i] = fmaf(-u[(uint64_t)i * ld + q], y[q], x[i]);
         }
-        const float* u = lu + (rb * T) * kGjOb + rb * T;
+        const float* u = F + (uint64_t)(rb * T) * ld + rb * T;
 #pragma unroll
         for (int i = T - 1; i >= 0; --i) {
 #pragma unroll
-            for (int q = i + 1; q < T; ++q) x[i] = fmaf(-u[i * kGjOb + q], x[q], x[i]);
-            x[i] = x[i] / u[i * kGjOb + i];
+            for (int q = i + 1; q < T; ++q) x[i] = fmaf(-u[(uint64_t)i * ld + q], x[q], x[i]);
+            x[i] = x[i] / u[(uint64_t)i * ld + i];
         }
 #pragma unroll
-        for (int i = 0; i < T; ++i) v[rb * T + i][tid] = x[i];
+        for (int i = 0; i < T; ++i) {
+            v[rb * T + i][tid] = x[i];
+            W[(uint64_t)(j0 + rb * T + i) * ld + col] = x[i];
+        }
     }
-#pragma unroll 8
-    for (int c = 0; c < kGjOb; ++c) W[(uint64_t)(j0 + c) * ld + col] = v[c][tid];
-#pragma unroll
-    for (int m = 0; m < kGjOb; ++m)
-        if (m < moves) W[(uint64_t)blk->to[m] * ld + col] = d[m];
 }
 
-// Every step applied to the whole matrix at once: fewer launches per column, 12 n^2 bytes per step.  The
-// faster way for small matrices, where a step's launches cost more than its memory traffic.
+// the two products that carry a block's eliminations to the columns right of it (OB values of k):
+// rows above the block with their own entries of the block's columns times R (which now is rows j0.. of W),
+// rows below with their multipliers times Y
+int gj_update_rest(float* W, uint64_t ld, uint32_t np, uint32_t j0, uint32_t ob, const float* Y, hipStream_t s) {
+    const uint32_t end = j0 + ob;
+    const uint64_t rest = 2ull * np - end;
+    if (j0 > 0) {
+        const int e = trakhip::gemm_nn(W + j0, ld, W + (uint64_t)j0 * ld + end, ld, W + end, ld, j0, rest, ob, -1.0f, 1.0f,
+                                       s, 0);
+        if (e) return e;
+    }
+    if (end < np)
+        return trakhip::gemm_nn(W + (uint64_t)end * ld + j0, ld, Y + end, ld, W + (uint64_t)end * ld + end, ld, np - end,
+                                rest, ob, -1.0f, 1.0f, s, 0);
+    return TRAKHIP_OK;
+}
+
+// blocks of one panel: the whole rest of the matrix after every SP columns
 template <int SP, int RPT>
-int gj_run_flat(float* W, uint32_t np, GjStep* steps, int32_t* status, hipStream_t s) {
+int gj_run_flat(float* W, float* Y, uint32_t np, GjStep* steps, int32_t* status, hipStream_t s) {
     const uint64_t ld = 2ull * np;
     for (uint32_t j = 0; j < np; j += SP) {
         GjStep* st = steps + (j / SP) % 2;  // two records in turn: the next panel never overwrites one still in use
         hipLaunchKernelGGL((gj_panel_kernel<SP, RPT>), dim3(1), dim3(kGjThreads), 0, s, W, ld, np, j, st, status);
         const uint32_t cols = 2 * np - j;
-        hipLaunchKernelGGL((gj_rows_kernel<SP>), dim3((cols + 255) / 256), dim3(256), 0, s, W, ld, j, 2 * np, st,
-                           (int32_t*)nullptr);
+        hipLaunchKernelGGL((gj_rows_kernel<SP>), dim3((cols + 255) / 256), dim3(256), 0, s, W, ld, j, j, 2 * np, st, Y);
         if (hipGetLastError() != hipSuccess) return TRAKHIP_ERR_LAUNCH;
-        const int e = trakhip::gemm_nn(W + j, ld, W + (uint64_t)j * ld + j + SP, ld, W + j + SP, ld, np,
-                                       2ull * np - j - SP, SP, -1.0f, 1.0f, s, 0);
+        const int e = gj_update_rest(W, ld, np, j, SP, Y, s);
         if (e) return e;
     }
     return TRAKHIP_OK;
 }
 
-struct GjBuffers {
-    float* W;           // np x 2 np
-    float* P0;          // np x kGjOb
-    float* P1;          // np x kGjOb
-    int32_t* row_map;   // np
-    GjBlock* blk;
-    GjStep* steps;      // kGjOb / 8 records
-};
-
+// blocks of kGjOb columns, kGjOb / SP panels each
 template <int SP, int RPT>
-int gj_run(const GjBuffers& b, uint32_t np, int32_t* status, hipStream_t s) {
+int gj_run(float* W, float* Y, uint32_t np, GjStep* steps, int32_t* status, hipStream_t s) {
     const uint64_t ld = 2ull * np;
-    float* W = b.W;
-    const uint32_t panel_blocks = (uint32_t)(((uint64_t)np * kGjOb + 255) / 256);
     for (uint32_t j0 = 0; j0 < np; j0 += kGjOb) {
-        hipLaunchKernelGGL(gj_block_begin_kernel, dim3(panel_blocks), dim3(256), 0, s, W, ld, np, j0, b.P0, b.row_map,
-                           b.blk);
-        const uint32_t block_end = j0 + kGjOb;
-        for (uint32_t j = j0; j < block_end; j += SP) {
-            GjStep* st = b.steps + (j - j0) / SP;
+        const uint32_t end = j0 + kGjOb;
+        for (uint32_t j = j0; j < end; j += SP) {
+            GjStep* st = steps + (j - j0) / SP;
             hipLaunchKernelGGL((gj_panel_kernel<SP, RPT>), dim3(1), dim3(kGjThreads), 0, s, W, ld, np, j, st, status);
-            hipLaunchKernelGGL((gj_rows_kernel<SP>), dim3((block_end - j + 255) / 256), dim3(256), 0, s, W, ld, j,
-                               block_end, st, b.row_map);
+            hipLaunchKernelGGL((gj_rows_kernel<SP>), dim3(1), dim3(256), 0, s, W, ld, j, j0, end, st, (float*)nullptr);
             if (hipGetLastError() != hipSuccess) return TRAKHIP_ERR_LAUNCH;
-            if (j + SP < block_end) {
-                const int e = trakhip::gemm_nn(W + j, ld, W + (uint64_t)j * ld + j + SP, ld, W + j + SP, ld, np,
-                                               block_end - j - SP, SP, -1.0f, 1.0f, s, 0);
+            if (j + SP < end && j + SP < np) {
+                // the block's columns right of the panel, rows below it
+                const int e = trakhip::gemm_nn(W + (uint64_t)(j + SP) * ld + j, ld, W + (uint64_t)j * ld + j + SP, ld,
+                                               W + (uint64_t)(j + SP) * ld + j + SP, ld, np - j - SP, end - j - SP, SP,
+                                               -1.0f, 1.0f, s, 0);
                 if (e) return e;
             }
         }
-        hipLaunchKernelGGL(gj_block_gather_kernel, dim3(panel_blocks), dim3(256), 0, s, b.P0, b.P1, b.row_map, np, j0,
-                           b.blk);
-        hipLaunchKernelGGL(gj_block_lu_kernel, dim3(1), dim3(64), 0, s, b.P0, b.row_map, j0, b.blk);
-        const uint32_t rest = 2 * np - block_end;
-        hipLaunchKernelGGL(gj_block_rows_kernel, dim3((rest + 255) / 256), dim3(256), 0, s, W, ld, np, j0, b.row_map,
-                           b.blk);
+        const uint32_t rest = 2 * np - end;
+        hipLaunchKernelGGL((gj_block_rows_kernel<SP>), dim3((rest + 255) / 256), dim3(256), 0, s, W, ld, np, j0,
+                           W + (uint64_t)j0 * ld + j0, steps, Y);
         if (hipGetLastError() != hipSuccess) return TRAKHIP_ERR_LAUNCH;
-        const int e = trakhip::gemm_nn(b.P1, kGjOb, W + (uint64_t)j0 * ld + block_end, ld, W + block_end, ld, np, rest,
-                                       kGjOb, -1.0f, 1.0f, s, 0);
+        const int e = gj_update_rest(W, ld, np, j0, kGjOb, Y, s);
         if (e) return e;
     }
     return TRAKHIP_OK;
@@ -1005,8 +952,7 @@ constexpr uint64_t kGeneralInverseMaxN = 12288;
 size_t general_inverse_workspace_bytes(uint64_t n) {
     if (n == 0 || n > kGeneralInverseMaxN) return 0;
     const uint64_t np = (n + NB - 1) / NB * NB;
-    return (size_t)(2 * np * np + 2 * np * kGjOb + np + kSumBlocks + 4) * sizeof(float) + sizeof(GjBlock) +
-           (kGjOb / 8) * sizeof(GjStep);
+    return (size_t)(2 * np * np + 2 * np * kGjOb + kSumBlocks + 4) * sizeof(float) + (kGjOb / 8) * sizeof(GjStep);
 }
 
 int general_inverse(const float* A, uint64_t lda, float lambda, float* inv, uint64_t ldi, uint64_t n, int normalize,
@@ -1018,24 +964,18 @@ int general_inverse(const float* A, uint64_t lda, float lambda, float* inv, uint
     if (reinterpret_cast<uintptr_t>(ws) % 16) return TRAKHIP_ERR_ALIGN;
     const uint64_t np = (n + NB - 1) / NB * NB;
     float* W = static_cast<float*>(ws);
-    GjBuffers b;
-    b.W = W;
-    b.P0 = W + 2 * np * np;
-    b.P1 = b.P0 + np * kGjOb;
-    b.row_map = reinterpret_cast<int32_t*>(b.P1 + np * kGjOb);
-    float* partial = reinterpret_cast<float*>(b.row_map + np);
+    float* Y = W + 2 * np * np;  // kGjOb x 2 np: L^-1 * (pivot rows) of the block at work
+    float* partial = Y + 2 * np * kGjOb;
     float* mean_dev = partial + kSumBlocks;
-    b.blk = reinterpret_cast<GjBlock*>(mean_dev + 4);
-    b.steps = reinterpret_cast<GjStep*>(b.blk + 1);
+    GjStep* steps = reinterpret_cast<GjStep*>(mean_dev + 4);
     hipLaunchKernelGGL(gj_init_kernel, dim3((uint32_t)((2 * np * np + 255) / 256)), dim3(256), 0, s, A, lda, lambda, n,
                        np, W, status);
     if (hipGetLastError() != hipSuccess) return TRAKHIP_ERR_LAUNCH;
     // the panel's rows live in the registers of one workgroup: 16 columns of up to 6144 rows, or 8 of up to 12288
-    // (measured: whole-matrix steps 1.8 / 3.5 / 7.9 / 16.2 ms at n = 512 / 1024 / 2048 / 3072, blocks of 64 columns
-    // 2.2 / 4.4 / 9.2 / 15.5 ms)
-    const int e = np < 3072      ? gj_run_flat<16, 6>(W, (uint32_t)np, b.steps, status, s)
-                  : np <= 6144   ? gj_run<16, 6>(b, (uint32_t)np, status, s)
-                                 : gj_run<8, 12>(b, (uint32_t)np, status, s);
+    // the panel's rows live in the registers of one workgroup: 16 columns of up to 6144 rows, or 8 of up to 12288
+    const int e = np < 3072      ? gj_run_flat<16, 6>(W, Y, (uint32_t)np, steps, status, s)
+                  : np <= 6144   ? gj_run<16, 6>(W, Y, (uint32_t)np, steps, status, s)
+                                 : gj_run<8, 12>(W, Y, (uint32_t)np, steps, status, s);
     if (e) return e;
     hipLaunchKernelGGL(gj_copy_out_kernel, dim3((uint32_t)((n * n + 255) / 256)), dim3(256), 0, s, W, 2 * np, np, n, inv,
                        ldi);

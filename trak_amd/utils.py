@@ -360,7 +360,7 @@ def gram_split(a, out=None, alpha=1.0, beta=0.0):
 
 
 def _inverse_call(a, lambda_reg, normalize, general):
-    """One call of trakhip_spd_inverse (Cholesky) or trakhip_general_inverse (pivoted Gauss-Jordan):
+    """One call of trakhip_spd_inverse (Cholesky) or trakhip_general_inverse (pivoted elimination):
     (inverse, mean_abs, status word)."""
     n = a.shape[0]
     lib = _lib.load()
@@ -396,7 +396,7 @@ def _inverse_call(a, lambda_reg, normalize, general):
 
 
 def general_inverse(a, lambda_reg=0.0, normalize=False):
-    """(a + lambda*I)^-1 for any nonsingular fp32 matrix on the GPU, by Gauss-Jordan elimination with
+    """(a + lambda*I)^-1 for any nonsingular fp32 matrix on the GPU, by elimination with
     partial pivoting - the pivoting of the LU behind torch.linalg.inv, the reference's call
     (trak/score_computers.py:163); with normalize=True divided by mean(|inverse|).  Returns (inverse,
     mean_abs).  An exactly singular matrix (a zero pivot) raises torch.linalg.LinAlgError, as the
