@@ -224,7 +224,9 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_nn_batched_kernel(const floa
                                                                       uint64_t N, uint64_t K, float alpha, float beta,
                                                                       uint32_t tiles_n, trakhip::GemmBatch batch) {
     const uint32_t y = blockIdx.y;
-    gemm_tile<false, true, true, 2>(A + batch.a[y], lda, B + batch.b[y], ldb, C + batch.c[y], ldc, M, N, K, alpha,
+    const uint64_t my = batch.m[y] ? batch.m[y] : M;
+    if ((uint64_t)(blockIdx.x / tiles_n) * BM >= my) return;  // (the whole workgroup: the grid is sized for the call's M)
+    gemm_tile<false, true, true, 2>(A + batch.a[y], lda, B + batch.b[y], ldb, C + batch.c[y], ldc, my, N, K, alpha,
                                     beta, nullptr, tiles_n, 0u, blockIdx.x);
 }
 
@@ -339,8 +341,10 @@ int gemm_nn_batched(const float* A, uint64_t lda, const float* B, uint64_t ldb, 
     // the batched kernel uses 16-byte loads: every operand start and pitch must allow them
     if ((reinterpret_cast<uintptr_t>(A) % 16) || (reinterpret_cast<uintptr_t>(B) % 16) || (lda % 4) || (ldb % 4))
         return TRAKHIP_ERR_ALIGN;
-    for (uint32_t y = 0; y < batch.count; ++y)
+    for (uint32_t y = 0; y < batch.count; ++y) {
         if ((batch.a[y] % 4) || (batch.b[y] % 4)) return TRAKHIP_ERR_ALIGN;
+        if (batch.m[y] > M) return TRAKHIP_ERR_SHAPE;
+    }
     const uint64_t tm = (M + BM - 1) / BM, tn = (N + 127) / 128;
     if (tm * tn > 0x7FFFFFFFull) return TRAKHIP_ERR_SHAPE;
     hipLaunchKernelGGL(gemm_nn_batched_kernel, dim3((uint32_t)(tm * tn), batch.count), dim3(kThreads), 0, s, A, lda, B,

@@ -887,6 +887,17 @@ __global__ __launch_bounds__(256) void gj_block_rows_kernel(float* __restrict__ 
 int gj_update_rest(float* W, uint64_t ld, uint32_t np, uint32_t j0, uint32_t ob, const float* Y, hipStream_t s) {
     const uint32_t end = j0 + ob;
     const uint64_t rest = 2ull * np - end;
+    if (ob < kGjOb && j0 > 0 && end < np) {
+        // one-panel blocks (small matrices): both products in one launch, a launch being what they cost.
+        // Y lies behind W in the same workspace, so one base pointer serves both B operands.
+        trakhip::GemmBatch two;
+        two.count = 2;
+        two.a[0] = j0, two.b[0] = (uint64_t)j0 * ld + end, two.c[0] = end, two.m[0] = j0;
+        two.a[1] = (uint64_t)end * ld + j0, two.b[1] = (uint64_t)(Y - W) + end, two.c[1] = (uint64_t)end * ld + end;
+        two.m[1] = np - end;
+        const uint64_t m = j0 > np - end ? j0 : np - end;
+        return trakhip::gemm_nn_batched(W, ld, W, ld, W, ld, m, rest, ob, -1.0f, 1.0f, two, s);
+    }
     if (j0 > 0) {
         const int e = trakhip::gemm_nn(W + j0, ld, W + (uint64_t)j0 * ld + end, ld, W + end, ld, j0, rest, ob, -1.0f, 1.0f,
                                        s, 0);

@@ -44,6 +44,7 @@ constexpr uint32_t kGemmBatchMax = 32;
 struct GemmBatch {
     uint32_t count;
     uint64_t a[kGemmBatchMax], b[kGemmBatchMax], c[kGemmBatchMax];
+    uint64_t m[kGemmBatchMax] = {};  // rows of product y when not zero (at most the call's M); zero: the call's M
 };
 int gemm_nn_batched(const float* A, uint64_t lda, const float* B, uint64_t ldb, float* C, uint64_t ldc, uint64_t M,
                     uint64_t N, uint64_t K, float alpha, float beta, const GemmBatch& batch, hipStream_t s);
