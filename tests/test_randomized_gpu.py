@@ -3,7 +3,8 @@
 Projection: random (rows, features, proj_dim, feature tiles, element type, matrix type, dense matrix or list of
 tensors) through the C ABI against the CPU oracle's float64 contraction on a window of columns, the list
 form against the dense form bit for bit.  GEMMs: random (M, N, K, alpha, beta, element type, kernel family)
-against float64.  The fixed-shape tests cover the cases somebody thought of; these cover combinations nobody
+against float64.  The inverse of matrices that are not positive definite: random sizes and structures against
+the float64 inverse, with a bound that follows the condition number.  The fixed-shape tests cover the cases somebody thought of; these cover combinations nobody
 listed.
 """
 import math
@@ -16,7 +17,8 @@ import torch
 
 from oracle import jl_oracle as npo
 from trak_amd import fast_jl
-from trak_amd.utils import gemm_nt, gemm_nt16, gemm_nt_split, gemm_tn, gram_split, split2_rows, split_rows
+from trak_amd.utils import (gemm_nt, gemm_nt16, gemm_nt_split, gemm_tn, general_inverse, gram_split, split2_rows,
+                            split_rows)
 
 pytestmark = pytest.mark.gpu
 
@@ -125,3 +127,36 @@ def test_random_gram_shapes_against_float64(gpu):
             want = (src.T @ src).numpy()
             assert torch.equal(got, got.T), (kind, N, K)
             assert _rel(got.cpu().numpy(), want) < 2.0 ** -19 + _tol(K), (kind, N, K)
+
+
+def test_random_matrices_through_the_general_inverse(gpu):
+    # sizes on both sides of the routes' limits are covered by fixed tests; here the structure varies: what the
+    # pivoting meets (rows of very different size, near-permutations, low rank + noise, symmetric indefinite)
+    rng = random.Random(4711)
+    gen = torch.Generator(device="cpu").manual_seed(4712)
+    for it in range(14):
+        n = rng.choice([3, 17, 64, 129, 200, 333, 512, 777, 1000, 1290])
+        kind = rng.choice(["normal", "graded_rows", "near_permutation", "low_rank_noise", "symmetric_indefinite"])
+        if kind == "normal":
+            a = torch.randn(n, n, generator=gen)
+        elif kind == "graded_rows":
+            a = torch.randn(n, n, generator=gen) * 10 ** (-3 * torch.rand(n, 1, generator=gen))
+        elif kind == "near_permutation":
+            a = 1e-3 * torch.randn(n, n, generator=gen)
+            a[torch.arange(n), torch.randperm(n, generator=gen)] += 1 + torch.rand(n, generator=gen)
+        elif kind == "low_rank_noise":
+            u = torch.randn(n, max(1, n // 20), generator=gen)
+            a = u @ u.T / u.shape[1] + 1e-2 * torch.randn(n, n, generator=gen)
+        else:
+            x = torch.randn(n, n, generator=gen) / math.sqrt(n)
+            a = (x + x.T) / 2 + torch.diag(torch.where(torch.rand(n, generator=gen) < 0.5, -1.0, 1.0))
+        lam = rng.choice([0.0, 1e-3])
+        case = (it, n, kind, lam)
+        got, mean_abs = general_inverse(a.to(gpu), lambda_reg=lam)
+        a64 = a.double().numpy() + lam * np.eye(n)
+        want = np.linalg.inv(a64)
+        cond = np.linalg.norm(a64, 1) * np.linalg.norm(want, 1)
+        err = np.abs(got.cpu().numpy() - want).max() / np.abs(want).max()
+        # LU with partial pivoting in fp32 measures 0.02 .. 0.05 of cond * 2^-24 on such matrices
+        assert err <= 0.5 * cond * 2.0 ** -24 + 1e-6, (case, err, cond)
+        assert abs(mean_abs.item() - np.abs(want).mean()) <= (0.5 * cond * 2.0 ** -24 + 1e-5) * np.abs(want).max(), case
