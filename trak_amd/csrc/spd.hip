@@ -569,9 +569,9 @@ namespace {
 // block instead of per panel); below that OB = SP = 16 (fewer launches per column, which is what small
 // matrices pay for).
 //
-// (An earlier form updated every row with the panel's original entries times D^-1 * (pivot rows), D the pivot
-// block: one product for all rows, but rounding errors of the size of cond(D) instead of the multipliers'
-// |l| <= 1 - up to 30 times the error of LAPACK's LU on matrices of condition 1e5..1e7.)
+// (Updating the rows below with the panel's original entries times D^-1 * (pivot rows), D the pivot block, would
+// be one product for all rows; it is not done because its rounding errors grow with the condition of D, where
+// the multipliers are at most 1.)
 
 constexpr int kGjThreads = 1024;
 constexpr int kGjMaxSp = 16;
